@@ -1,0 +1,55 @@
+/* AMD-specific additions to the mops C ABI. None of these exist in
+ * lab-cosmo/mops; callers that only use the reference's 61 symbols never
+ * need them.
+ *
+ * Stream and synchronisation. The reference's device entry points launch on
+ * the null stream and block until the device is idle
+ * (e.g. mops/src/opsa/opsa.cu:85-87). That stays the default here. A caller
+ * that manages its own HIP streams (PyTorch does) can instead name the
+ * stream to launch on and turn the blocking wait off; both settings are per
+ * calling thread.
+ */
+#ifndef MOPS_AMD_H
+#define MOPS_AMD_H
+
+#include <stdint.h>
+
+#include "mops/exports.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Launch all following mops_cuda_* calls of this thread on `hip_stream`
+ * (a hipStream_t; NULL selects the null stream). Returns 0. */
+MOPS_EXPORT int mops_amd_set_stream(void* hip_stream);
+
+/* The stream set by mops_amd_set_stream on this thread (NULL by default). */
+MOPS_EXPORT void* mops_amd_get_stream(void);
+
+/* synchronous != 0 (default): every mops_cuda_* call waits for its kernels
+ * before returning, as the reference does. synchronous == 0: calls return
+ * once the work is enqueued; the caller orders later work on the same stream
+ * or synchronises itself. Returns the previous setting. */
+MOPS_EXPORT int mops_amd_set_synchronous(int synchronous);
+
+/* Segment boundaries of a sorted index vector, on the device.
+ *
+ * `sorted_indices` holds n_input non-decreasing int32 values (device
+ * memory). `first_occurrences` receives 2*n_output int32 values (device
+ * memory): [v] is the position of the first element equal to v and
+ * [n_output + v] one past the last; both are -1 for a value that does not
+ * occur. Integer work, bit-exact. Replaces the reference's internal
+ * calculate_first_occurences_cuda (mops/src/internal/cuda_first_occurences.cu:82-117),
+ * which is what its scatter kernels use to find the rows of each output
+ * segment; exposed here so the result can be checked on its own.
+ * Returns 0 / 1 / 2 like every other entry point. */
+MOPS_EXPORT int mops_amd_first_occurrences(
+    const int32_t* sorted_indices, int64_t n_input, int64_t n_output, int32_t* first_occurrences
+);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif

@@ -1,0 +1,47 @@
+/* C ABI of outer_product_scatter_add_with_weights (OPSAW).
+ *
+ *   O[indices_output[e], :, :] += A[e, :, None] * B[e, None, :] * W[indices_W[e], None, :]
+ *
+ * Tensors (row-major, caller-owned, outputs are fully overwritten):
+ *   output [n_nodes, size_A, size_B]
+ *   A [n_edges, size_A]
+ *   B [n_edges, size_B]
+ *   W [n_nodes, size_B]
+ *   indices_W, indices_output int32 [n_edges]
+ *
+ * This header declares twelve functions, replacing mops/include/mops/opsaw.h:12-175
+ * of lab-cosmo/mops one for one:
+ *
+ *   mops_outer_product_scatter_add_with_weights[_vjp[_vjp]]_{f32,f64}        host memory
+ *   mops_cuda_outer_product_scatter_add_with_weights[_vjp[_vjp]]_{f32,f64}   device memory
+ *
+ * The "cuda" in the device entry points is the reference's spelling and is
+ * kept so that existing callers (which build the symbol name as
+ * "mops_" + "cuda_" + op + "_" + dtype, python/mops/src/mops/dispatch_operation.py:24-28)
+ * resolve without change; behind it is the HIP implementation for gfx950.
+ *
+ * Return value: 0 on success, 1 when a C++ exception was caught (text via
+ * mops_get_last_error_message()), 2 for an unknown error. A gradient whose
+ * `data` is NULL is skipped. The argument orders live in
+ * mops/detail/signatures.h.
+ */
+#ifndef MOPS_OPSAW_H
+#define MOPS_OPSAW_H
+
+#include "mops/exports.h"
+#include "mops/tensor.h"
+#include "mops/detail/signatures.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+MOPS_C_DECLARE_ALL(outer_product_scatter_add_with_weights, MOPS_OPSAW_PARAMS)
+MOPS_C_DECLARE_ALL(outer_product_scatter_add_with_weights_vjp, MOPS_OPSAW_VJP_PARAMS)
+MOPS_C_DECLARE_ALL(outer_product_scatter_add_with_weights_vjp_vjp, MOPS_OPSAW_VJP_VJP_PARAMS)
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif

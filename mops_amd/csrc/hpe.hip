@@ -1,0 +1,354 @@
+// Homogeneous polynomial evaluation (HPE), forward and vector-Jacobian
+// product, for gfx950.
+//
+//   O[i] = sum_j C[j] * prod_k A[i, P[j, k]]
+//   grad_A[i, P[j, f]] += C[j] * grad_O[i] * prod_{k != f} A[i, P[j, k]]
+//
+// Semantics restated from mops/src/hpe/cpu.tpp:13-272 of lab-cosmo/mops:
+// each monomial's product starts from C[j] and multiplies the factors left
+// to right; a polynomial of order 0 gives O[i] = sum_j C[j]; the vjp is a
+// no-op when grad_A is not requested. (The CPU reference stops at order 10;
+// there is no such limit here.)
+//
+// Work split: a workgroup takes `R` consecutive batch rows (R a power of two,
+// 1..64) and G = blockDim / R monomial groups; thread (r, g) evaluates the
+// monomials j = g, g + G, ... for row r. The rows' A values sit in LDS as
+// [feature][row]. Small batches get R = 1 (the whole workgroup shares one row
+// and spreads over the monomials), large batches R = 64 (one row per lane,
+// the table read once per wavefront), so that there are always enough
+// workgroups to fill the device.
+//
+// The partial sums of the G groups are combined in group order, so results
+// are reproducible from run to run. The reference's CUDA vjp accumulates
+// with shared-memory float atomics (mops/src/hpe/hpe.cu:288) and is not.
+#include <algorithm>
+
+#include "mops/hpe.hpp"
+
+#include "checks.hpp"
+#include "device_common.hpp"
+#include "index_validation.hpp"
+#include "runtime.hpp"
+
+namespace mops::amd {
+namespace {
+
+constexpr size_t LDS_BUDGET = 60 * 1024;
+
+// ---------------------------------------------------------------------------
+// forward. LDS: a[nA][R] partial[G][R]
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void forward_kernel(
+    T* __restrict__ output,
+    const T* __restrict__ A,
+    const T* __restrict__ C,
+    const int32_t* __restrict__ P,
+    int32_t n_rows,
+    int32_t nA,
+    int32_t n_monomials,
+    int32_t order,
+    int32_t R
+) {
+    extern __shared__ __align__(16) unsigned char lds_bytes[];
+    T* a_stage = reinterpret_cast<T*>(lds_bytes);
+    T* partial = a_stage + static_cast<size_t>(nA) * R;
+
+    const int tid = threadIdx.x;
+    const int G = blockDim.x / R;
+    const int r = tid % R;
+    const int g = tid / R;
+    const int32_t row0 = blockIdx.x * R;
+    const int32_t rows = min(R, n_rows - row0);
+
+    const T* a_src = A + static_cast<size_t>(row0) * nA;
+    for (int32_t i = tid; i < rows * nA; i += blockDim.x) {
+        int32_t row = i / nA;
+        a_stage[(i - row * nA) * R + row] = a_src[i];
+    }
+    __syncthreads();
+
+    T sum = T(0);
+    if (r < rows) {
+        for (int32_t j = g; j < n_monomials; j += G) {
+            const int32_t* factors = P + static_cast<size_t>(j) * order;
+            T product = C[j];
+            for (int32_t k = 0; k < order; k++) {
+                int32_t feature = factors[k];
+                product *= in_bounds(feature, nA) ? a_stage[feature * R + r] : T(0);
+            }
+            sum += product;
+        }
+    }
+    partial[g * R + r] = sum;
+    __syncthreads();
+    if (g == 0 && r < rows) {
+        T total = T(0);
+        for (int group = 0; group < G; group++) {
+            total += partial[group * R + r];
+        }
+        output[row0 + r] = total;
+    }
+}
+
+// ---------------------------------------------------------------------------
+// vjp. One wavefront per workgroup. LDS: a[nA][R] accumulator[G][nA][R]
+// Thread (r, g) adds its monomials' terms into its private accumulator row
+// set; afterwards the G copies are added in group order.
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(WAVE) void vjp_kernel(
+    T* __restrict__ grad_A,
+    const T* __restrict__ grad_output,
+    const T* __restrict__ A,
+    const T* __restrict__ C,
+    const int32_t* __restrict__ P,
+    int32_t n_rows,
+    int32_t nA,
+    int32_t n_monomials,
+    int32_t order,
+    int32_t R
+) {
+    extern __shared__ __align__(16) unsigned char lds_bytes[];
+    T* a_stage = reinterpret_cast<T*>(lds_bytes);
+    T* accumulator = a_stage + static_cast<size_t>(nA) * R;
+
+    const int tid = threadIdx.x;
+    const int G = WAVE / R;
+    const int r = tid % R;
+    const int g = tid / R;
+    const int32_t row0 = blockIdx.x * R;
+    const int32_t rows = min(R, n_rows - row0);
+
+    const T* a_src = A + static_cast<size_t>(row0) * nA;
+    for (int32_t i = tid; i < rows * nA; i += WAVE) {
+        int32_t row = i / nA;
+        a_stage[(i - row * nA) * R + row] = a_src[i];
+    }
+    for (int32_t i = tid; i < G * nA * R; i += WAVE) {
+        accumulator[i] = T(0);
+    }
+    __syncthreads();
+
+    if (r < rows) {
+        T* mine = accumulator + static_cast<size_t>(g) * nA * R + r;
+        const T upstream = grad_output[row0 + r];
+        for (int32_t j = g; j < n_monomials; j += G) {
+            const int32_t* factors = P + static_cast<size_t>(j) * order;
+            const T base = C[j] * upstream;
+            for (int32_t f = 0; f < order; f++) {
+                int32_t target = factors[f];
+                if (!in_bounds(target, nA)) {
+                    continue;
+                }
+                T term = base;
+                for (int32_t k = 0; k < order; k++) {
+                    if (k == f) {
+                        continue;
+                    }
+                    int32_t feature = factors[k];
+                    term *= in_bounds(feature, nA) ? a_stage[feature * R + r] : T(0);
+                }
+                mine[target * R] += term;
+            }
+        }
+    }
+    __syncthreads();
+
+    T* dst = grad_A + static_cast<size_t>(row0) * nA;
+    for (int32_t i = tid; i < rows * nA; i += WAVE) {
+        int32_t row = i / nA;
+        int32_t feature = i - row * nA;
+        T total = T(0);
+        for (int group = 0; group < G; group++) {
+            total += accumulator[(static_cast<size_t>(group) * nA + feature) * R + row];
+        }
+        dst[i] = total;
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Fallbacks for feature counts whose tiles do not fit in LDS: one thread per
+// batch row, everything in global memory.
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void forward_global_kernel(
+    T* __restrict__ output,
+    const T* __restrict__ A,
+    const T* __restrict__ C,
+    const int32_t* __restrict__ P,
+    int32_t n_rows,
+    int32_t nA,
+    int32_t n_monomials,
+    int32_t order
+) {
+    const int32_t row = blockIdx.x * blockDim.x + threadIdx.x;
+    if (row >= n_rows) {
+        return;
+    }
+    const T* a_row = A + static_cast<size_t>(row) * nA;
+    T sum = T(0);
+    for (int32_t j = 0; j < n_monomials; j++) {
+        const int32_t* factors = P + static_cast<size_t>(j) * order;
+        T product = C[j];
+        for (int32_t k = 0; k < order; k++) {
+            int32_t feature = factors[k];
+            product *= in_bounds(feature, nA) ? a_row[feature] : T(0);
+        }
+        sum += product;
+    }
+    output[row] = sum;
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void vjp_global_kernel(
+    T* grad_A,
+    const T* __restrict__ grad_output,
+    const T* __restrict__ A,
+    const T* __restrict__ C,
+    const int32_t* __restrict__ P,
+    int32_t n_rows,
+    int32_t nA,
+    int32_t n_monomials,
+    int32_t order
+) {
+    const int32_t row = blockIdx.x * blockDim.x + threadIdx.x;
+    if (row >= n_rows) {
+        return;
+    }
+    const T* a_row = A + static_cast<size_t>(row) * nA;
+    T* g_row = grad_A + static_cast<size_t>(row) * nA;
+    for (int32_t feature = 0; feature < nA; feature++) {
+        g_row[feature] = T(0);
+    }
+    const T upstream = grad_output[row];
+    for (int32_t j = 0; j < n_monomials; j++) {
+        const int32_t* factors = P + static_cast<size_t>(j) * order;
+        const T base = C[j] * upstream;
+        for (int32_t f = 0; f < order; f++) {
+            int32_t target = factors[f];
+            if (!in_bounds(target, nA)) {
+                continue;
+            }
+            T term = base;
+            for (int32_t k = 0; k < order; k++) {
+                if (k == f) {
+                    continue;
+                }
+                int32_t feature = factors[k];
+                term *= in_bounds(feature, nA) ? a_row[feature] : T(0);
+            }
+            g_row[target] += term;
+        }
+    }
+}
+
+// Rows per workgroup: as many as possible (fewer table reads per row) while
+// the launch still has about a thousand workgroups and the tiles fit in LDS.
+// Returns 0 when even R = 1 does not fit.
+int pick_rows(size_t n_rows, size_t bytes_per_row) {
+    int R = 64;
+    while (R > 1 && (n_rows / R < 1024 || bytes_per_row * R > LDS_BUDGET)) {
+        R >>= 1;
+    }
+    return bytes_per_row * R > LDS_BUDGET ? 0 : R;
+}
+
+} // namespace
+} // namespace mops::amd
+
+namespace mops::cuda {
+
+template <typename scalar_t>
+void homogeneous_polynomial_evaluation(MOPS_HPE_PARAMS(MOPS_CXX_FIRST, MOPS_CXX_NEXT)) {
+    using namespace mops::amd;
+    const char* operation = "cuda_homogeneous_polynomial_evaluation";
+    checks::Validator validator(operation);
+    checks::hpe(validator, output, A, C, indices_A);
+    validate_gather_index(indices_A, A.shape[1], "indices_A", operation);
+
+    const int32_t n_rows = narrow_i32(A.shape[0], "A.shape[0]");
+    const int32_t nA = narrow_i32(A.shape[1], "A.shape[1]");
+    const int32_t n_monomials = narrow_i32(indices_A.shape[0], "indices_A.shape[0]");
+    const int32_t order = narrow_i32(indices_A.shape[1], "indices_A.shape[1]");
+    if (n_rows == 0) {
+        return;
+    }
+    hipStream_t stream = current_stream();
+    constexpr int THREADS = 256;
+    // per row: its A values plus one partial sum per group (G <= THREADS)
+    int R = pick_rows(n_rows, (static_cast<size_t>(nA) + THREADS) * sizeof(scalar_t));
+    if (R > 0) {
+        size_t lds = (static_cast<size_t>(nA) * R + THREADS) * sizeof(scalar_t);
+        unsigned blocks = static_cast<unsigned>(ceil_div(static_cast<size_t>(n_rows), R));
+        forward_kernel<scalar_t><<<blocks, THREADS, lds, stream>>>(
+            output.data, A.data, C.data, indices_A.data, n_rows, nA, n_monomials, order, R
+        );
+    } else {
+        unsigned blocks = static_cast<unsigned>(ceil_div(static_cast<size_t>(n_rows), THREADS));
+        forward_global_kernel<scalar_t><<<blocks, THREADS, 0, stream>>>(
+            output.data, A.data, C.data, indices_A.data, n_rows, nA, n_monomials, order
+        );
+    }
+    finish_call(operation);
+}
+
+template <typename scalar_t>
+void homogeneous_polynomial_evaluation_vjp(MOPS_HPE_VJP_PARAMS(MOPS_CXX_FIRST, MOPS_CXX_NEXT)) {
+    using namespace mops::amd;
+    const char* operation = "cuda_homogeneous_polynomial_evaluation_vjp";
+    checks::Validator validator(operation);
+    checks::hpe_vjp(validator, grad_A, grad_output, A, C, indices_A);
+    if (grad_A.data == nullptr) {
+        return;
+    }
+    validate_gather_index(indices_A, A.shape[1], "indices_A", operation);
+
+    const int32_t n_rows = narrow_i32(A.shape[0], "A.shape[0]");
+    const int32_t nA = narrow_i32(A.shape[1], "A.shape[1]");
+    const int32_t n_monomials = narrow_i32(indices_A.shape[0], "indices_A.shape[0]");
+    const int32_t order = narrow_i32(indices_A.shape[1], "indices_A.shape[1]");
+    if (n_rows == 0 || nA == 0) {
+        return;
+    }
+    hipStream_t stream = current_stream();
+    // LDS holds R rows of A and WAVE private accumulator rows, whatever R is
+    const size_t accumulator_bytes = static_cast<size_t>(nA) * WAVE * sizeof(scalar_t);
+    int R = 0;
+    if (accumulator_bytes < LDS_BUDGET) {
+        R = 64;
+        while (R > 1 && (static_cast<size_t>(n_rows) / R < 1024 ||
+                         accumulator_bytes + static_cast<size_t>(nA) * R * sizeof(scalar_t) > LDS_BUDGET)) {
+            R >>= 1;
+        }
+        if (accumulator_bytes + static_cast<size_t>(nA) * R * sizeof(scalar_t) > LDS_BUDGET) {
+            R = 0;
+        }
+    }
+    if (R > 0) {
+        size_t lds = accumulator_bytes + static_cast<size_t>(nA) * R * sizeof(scalar_t);
+        unsigned blocks = static_cast<unsigned>(ceil_div(static_cast<size_t>(n_rows), R));
+        vjp_kernel<scalar_t><<<blocks, WAVE, lds, stream>>>(
+            grad_A.data, grad_output.data, A.data, C.data, indices_A.data, n_rows, nA, n_monomials,
+            order, R
+        );
+    } else {
+        unsigned blocks = static_cast<unsigned>(ceil_div(static_cast<size_t>(n_rows), 256));
+        vjp_global_kernel<scalar_t><<<blocks, 256, 0, stream>>>(
+            grad_A.data, grad_output.data, A.data, C.data, indices_A.data, n_rows, nA, n_monomials, order
+        );
+    }
+    finish_call(operation);
+}
+
+template <typename scalar_t>
+void homogeneous_polynomial_evaluation_vjp_vjp(MOPS_HPE_VJP_VJP_PARAMS(MOPS_CXX_FIRST, MOPS_CXX_NEXT)) {
+    // same state as the reference's device path (mops/src/hpe/hpe.cu:402-413)
+    throw std::runtime_error("Not implemented");
+}
+
+MOPS_CXX_INSTANTIATE(homogeneous_polynomial_evaluation, MOPS_HPE_PARAMS)
+MOPS_CXX_INSTANTIATE(homogeneous_polynomial_evaluation_vjp, MOPS_HPE_VJP_PARAMS)
+MOPS_CXX_INSTANTIATE(homogeneous_polynomial_evaluation_vjp_vjp, MOPS_HPE_VJP_VJP_PARAMS)
+
+} // namespace mops::cuda

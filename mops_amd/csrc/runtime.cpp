@@ -1,0 +1,113 @@
+#include "runtime.hpp"
+
+#include <cstdlib>
+#include <limits>
+
+namespace mops::amd {
+
+void check_hip(hipError_t status, const char* what) {
+    if (status != hipSuccess) {
+        throw std::runtime_error(
+            std::string("HIP error in ") + what + ": " + hipGetErrorString(status)
+        );
+    }
+}
+
+namespace {
+
+struct ThreadState {
+    hipStream_t stream = nullptr;
+    bool synchronous = true;
+
+    // scratch cache
+    void* block = nullptr;
+    size_t capacity = 0;
+    int device = -1;
+    hipStream_t block_stream = nullptr;
+    hipEvent_t block_event = nullptr;
+};
+
+ThreadState& state() {
+    // Deliberately never destroyed: at thread or process exit the HIP runtime
+    // may already be gone, and freeing device memory then would fault.
+    static thread_local ThreadState* instance = new ThreadState();
+    return *instance;
+}
+
+} // namespace
+
+hipStream_t current_stream() { return state().stream; }
+
+void set_current_stream(hipStream_t stream) { state().stream = stream; }
+
+bool synchronous() { return state().synchronous; }
+
+bool set_synchronous(bool value) {
+    bool previous = state().synchronous;
+    state().synchronous = value;
+    return previous;
+}
+
+void finish_call(const char* operation) {
+    check_hip(hipGetLastError(), operation);
+    auto& st = state();
+    if (st.block != nullptr && st.block_event != nullptr) {
+        // mark the point after which the scratch block is free again
+        check_hip(hipEventRecord(st.block_event, st.stream), operation);
+        st.block_stream = st.stream;
+    }
+    if (st.synchronous) {
+        check_hip(hipStreamSynchronize(st.stream), operation);
+    }
+}
+
+void* scratch(size_t bytes) {
+    auto& st = state();
+    int device = 0;
+    MOPS_HIP_CHECK(hipGetDevice(&device));
+
+    if (st.block != nullptr && (device != st.device || bytes > st.capacity)) {
+        // hipFree waits for the device, so nothing can still be using the block
+        int restore = device;
+        MOPS_HIP_CHECK(hipSetDevice(st.device));
+        MOPS_HIP_CHECK(hipFree(st.block));
+        MOPS_HIP_CHECK(hipEventDestroy(st.block_event));
+        MOPS_HIP_CHECK(hipSetDevice(restore));
+        st.block = nullptr;
+        st.block_event = nullptr;
+        st.capacity = 0;
+    }
+
+    if (st.block == nullptr) {
+        size_t capacity = bytes + bytes / 2;
+        if (capacity < (size_t(1) << 20)) {
+            capacity = size_t(1) << 20;
+        }
+        MOPS_HIP_CHECK(hipMalloc(&st.block, capacity));
+        MOPS_HIP_CHECK(hipEventCreateWithFlags(&st.block_event, hipEventDisableTiming));
+        st.capacity = capacity;
+        st.device = device;
+        st.block_stream = st.stream;
+    } else if (st.block_stream != st.stream) {
+        // the previous user ran on another stream: order this one behind it
+        MOPS_HIP_CHECK(hipStreamWaitEvent(st.stream, st.block_event, 0));
+    }
+    return st.block;
+}
+
+int32_t narrow_i32(size_t value, const char* what) {
+    if (value > static_cast<size_t>(std::numeric_limits<int32_t>::max())) {
+        throw std::runtime_error(
+            std::string(what) + " = " + std::to_string(value) +
+            " does not fit the 32-bit indexing of the device kernels"
+        );
+    }
+    return static_cast<int32_t>(value);
+}
+
+bool validate_device_indices() {
+    const char* value = std::getenv("MOPS_AMD_CHECK_INDICES");
+    return value != nullptr && value[0] != '\0' && value[0] != '0';
+}
+
+} // namespace mops::amd

@@ -1,0 +1,60 @@
+// Host-side plumbing shared by every device operation: HIP error handling,
+// the per-thread stream / synchronisation settings, launch helpers and the
+// scratch-memory cache.
+#ifndef MOPS_AMD_RUNTIME_HPP
+#define MOPS_AMD_RUNTIME_HPP
+
+#include <cstddef>
+#include <cstdint>
+#include <stdexcept>
+#include <string>
+
+#include <hip/hip_runtime.h>
+
+namespace mops::amd {
+
+/// Throw std::runtime_error naming `what` when `status` is not hipSuccess.
+/// (The reference prints and calls exit() on a device error,
+/// mops/src/internal/cuda_utils.cuh:11-24; throwing lets the C ABI report
+/// status 1 instead of killing the caller's process.)
+void check_hip(hipError_t status, const char* what);
+
+#define MOPS_HIP_CHECK(expression) ::mops::amd::check_hip((expression), #expression)
+
+/// Stream that device work of the calling thread is enqueued on.
+hipStream_t current_stream();
+void set_current_stream(hipStream_t stream);
+
+/// Whether device entry points wait for their kernels before returning.
+bool synchronous();
+bool set_synchronous(bool value);
+
+/// Check the launch that was just issued, then wait for the stream if the
+/// calling thread is in synchronous mode. Called once at the end of every
+/// device entry point.
+void finish_call(const char* operation);
+
+/// Scratch device memory of at least `bytes` bytes, 256-byte aligned, valid
+/// until the next call of this function on the same thread. The block is
+/// cached per thread and grows on demand; work enqueued on a different
+/// stream than the previous user is ordered behind it by a stream wait.
+void* scratch(size_t bytes);
+
+/// ceil(a / b) for positive b.
+inline size_t ceil_div(size_t a, size_t b) { return (a + b - 1) / b; }
+
+/// Round `bytes` up to a multiple of 256 so that consecutive carve-outs of
+/// one scratch block keep every sub-buffer aligned for 128-bit accesses.
+inline size_t align256(size_t bytes) { return (bytes + 255) & ~static_cast<size_t>(255); }
+
+/// Convert a size to the 32-bit signed range the kernels index with.
+int32_t narrow_i32(size_t value, const char* what);
+
+/// True when the environment asks for index validation on the device path
+/// (MOPS_AMD_CHECK_INDICES=1): index tensors are then copied to the host and
+/// checked for range (and the scatter index for sortedness) on every call.
+bool validate_device_indices();
+
+} // namespace mops::amd
+
+#endif

@@ -1,0 +1,201 @@
+"""Parity of the HIP kernels with the CPU oracle, through the device C ABI.
+
+Bar (from the north star): max|x - ref| / max|ref| <= 1e-12 in float64 and
+<= 1e-5 in float32, for outputs and every gradient. Small seeded cases cover
+the shapes and edge cases of the reference's own tests (empty segments,
+ragged sizes, every subset of requested gradients, unsorted SAP output
+index); the BASELINE configurations are checked at full size against the
+oracle and through size-independent properties (linearity, adjoint identity,
+run-to-run bit reproducibility).
+"""
+import itertools
+
+import numpy as np
+import pytest
+
+from tests import support
+from tests.support import OPS, assert_close, cpu_forward, cpu_vjp, hip_forward, hip_vjp, to_device
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [np.float32, np.float64]
+
+# name -> builder(seed, dtype); shapes chosen to hit partial tiles, sizes
+# that are not multiples of the wavefront, and segments of very unequal length
+CASES = {
+    "hpe": {
+        "tiny": lambda s, d: support.hpe_case(s, d, I=5, nA=3, J=7, K=2),
+        "ragged": lambda s, d: support.hpe_case(s, d, I=203, nA=17, J=301, K=3),
+        "order0": lambda s, d: support.hpe_case(s, d, I=70, nA=4, J=33, K=0),
+        "order1": lambda s, d: support.hpe_case(s, d, I=70, nA=4, J=33, K=1),
+        "order6": lambda s, d: support.hpe_case(s, d, I=130, nA=9, J=90, K=6),
+        "many_rows": lambda s, d: support.hpe_case(s, d, I=70000, nA=12, J=40, K=3),
+        "wide": lambda s, d: support.hpe_case(s, d, I=64, nA=2000, J=500, K=4),
+    },
+    "sap": {
+        "tiny": lambda s, d: support.sap_case(s, d, I=3, nA=2, nB=2, K=5, nO=3),
+        "ragged": lambda s, d: support.sap_case(s, d, I=333, nA=13, nB=7, K=211, nO=20),
+        "unsorted": lambda s, d: support.sap_case(s, d, I=130, nA=6, nB=9, K=150, nO=11, sort_output=False),
+        "wide": lambda s, d: support.sap_case(s, d, I=100, nA=70, nB=50, K=400, nO=300),
+        "one_product": lambda s, d: support.sap_case(s, d, I=65, nA=3, nB=3, K=1, nO=4),
+    },
+    "opsa": {
+        "tiny": lambda s, d: support.opsa_case(s, d, J=6, K=2, L=3, n_out=4, allow_empty=True),
+        "ragged": lambda s, d: support.opsa_case(s, d, J=1000, K=13, L=20, n_out=37, allow_empty=True),
+        "long_segments": lambda s, d: support.opsa_case(s, d, J=3000, K=5, L=7, n_out=6),
+        "wide": lambda s, d: support.opsa_case(s, d, J=400, K=40, L=33, n_out=21, allow_empty=True),
+        "mostly_empty": lambda s, d: support.opsa_case(s, d, J=20, K=4, L=4, n_out=300, allow_empty=True),
+    },
+    "opsaw": {
+        "tiny": lambda s, d: support.opsaw_case(s, d, E=6, K=2, L=3, n_nodes=4, allow_empty=True),
+        "ragged": lambda s, d: support.opsaw_case(s, d, E=1000, K=13, L=32, n_nodes=37, allow_empty=True),
+        "long_segments": lambda s, d: support.opsaw_case(s, d, E=3000, K=5, L=7, n_nodes=6),
+        "hub_sender": lambda s, d: _hub(support.opsaw_case(s, d, E=2600, K=3, L=5, n_nodes=9), "indices_W"),
+        "mostly_empty": lambda s, d: support.opsaw_case(s, d, E=20, K=4, L=4, n_nodes=300, allow_empty=True),
+    },
+    "sasaw": {
+        "tiny": lambda s, d: support.sasaw_case(s, d, E=6, nA=2, L=3, n_nodes=4, n2=2, n3=2, N=5, allow_empty=True),
+        "ragged": lambda s, d: support.sasaw_case(s, d, E=700, nA=9, L=32, n_nodes=29, n2=9, n3=9, N=250, allow_empty=True),
+        "rectangular": lambda s, d: support.sasaw_case(s, d, E=300, nA=7, L=10, n_nodes=13, n2=5, n3=15, N=90, allow_empty=True),
+        "hub_sender": lambda s, d: _hub(
+            support.sasaw_case(s, d, E=2300, nA=3, L=4, n_nodes=7, n2=2, n3=3, N=10), "indices_W_1"
+        ),
+        "mostly_empty": lambda s, d: support.sasaw_case(s, d, E=15, nA=3, L=5, n_nodes=200, n2=3, n3=2, N=7, allow_empty=True),
+    },
+}  # fmt: skip
+
+
+def _hub(case, key):
+    """Most edges name the same sender: one gather list longer than the LDS sort buffer."""
+    case[key][: len(case[key]) * 3 // 4] = 2
+    return case
+
+
+ALL = [(op, name) for op, cases in CASES.items() for name in cases]
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=["f32", "f64"])
+@pytest.mark.parametrize("op,name", ALL)
+def test_forward(oracle, device, op, name, dtype):
+    case = CASES[op][name](101, dtype)
+    expected = cpu_forward(oracle, op, case)
+    actual = hip_forward(op, to_device(case, device)).cpu().numpy()
+    assert_close(actual, expected, dtype, f"{op}/{name}")
+    # also against the dense float64 formulation, which shares nothing with the oracle
+    assert_close(actual, OPS[op].dense(case), dtype, f"{op}/{name} dense", factor=2.0)
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=["f32", "f64"])
+@pytest.mark.parametrize("op,name", ALL)
+def test_vjp(oracle, device, op, name, dtype):
+    case = CASES[op][name](202, dtype)
+    expected = cpu_vjp(oracle, op, case)
+    actual = hip_vjp(op, to_device(case, device))
+    for key in OPS[op].differentiable:
+        assert_close(actual[key].cpu().numpy(), expected[key], dtype, f"{op}/{name} grad_{key}")
+
+
+@pytest.mark.parametrize("op", list(OPS))
+def test_vjp_subsets_of_gradients(oracle, device, op):
+    """Every subset of requested gradients gives the same values as all of them."""
+    case = CASES[op]["ragged"](303, np.float64)
+    on_device = to_device(case, device)
+    full = hip_vjp(op, on_device)
+    names = OPS[op].differentiable
+    for r in range(len(names)):
+        for wanted in itertools.combinations(names, r):
+            partial = hip_vjp(op, on_device, wanted=list(wanted))
+            for key in names:
+                if key in wanted:
+                    assert np.array_equal(partial[key].cpu().numpy(), full[key].cpu().numpy()), (op, wanted, key)
+                else:
+                    assert partial[key] is None
+
+
+@pytest.mark.parametrize("op", ["opsa", "opsaw", "sasaw"])
+def test_rows_without_edges_are_exactly_zero(device, op):
+    case = CASES[op]["ragged"](404, np.float32)
+    key = "indices_output_1" if op == "sasaw" else "indices_output"
+    index = case[key]
+    index[index == 1] = 2
+    case[key] = np.sort(index)
+    out = hip_forward(op, to_device(case, device)).cpu().numpy()
+    assert np.all(out[1] == 0.0)
+    assert not np.any(np.isnan(out))
+
+
+def test_no_edges_at_all(device):
+    """Zero input rows: outputs are all zero, gradients are empty."""
+    for op in ("opsa", "opsaw", "sasaw"):
+        case = CASES[op]["tiny"](1, np.float64)
+        for key in ("A", "B"):
+            case[key] = case[key][:0]
+        for key in ("indices_output", "indices_W", "indices_output_1", "indices_W_1"):
+            if key in case:
+                case[key] = case[key][:0]
+        out = hip_forward(op, to_device(case, device)).cpu().numpy()
+        assert out.size > 0 and np.all(out == 0.0)
+        grads = hip_vjp(op, to_device(case, device))
+        assert grads["A"].numel() == 0 and grads["B"].numel() == 0
+        if "W" in grads:
+            assert np.all(grads["W"].cpu().numpy() == 0.0)
+
+
+@pytest.mark.parametrize("op", list(OPS))
+def test_bit_reproducible(device, op):
+    """No atomics on floating-point data: two runs give identical bits."""
+    case = to_device(CASES[op]["ragged"](505, np.float32), device)
+    first = hip_forward(op, case).cpu().numpy()
+    second = hip_forward(op, case).cpu().numpy()
+    assert np.array_equal(first, second)
+    g1 = hip_vjp(op, case)
+    g2 = hip_vjp(op, case)
+    for key in OPS[op].differentiable:
+        assert np.array_equal(g1[key].cpu().numpy(), g2[key].cpu().numpy()), (op, key)
+
+
+# ---- BASELINE configurations at full size ---------------------------------
+BASELINE = [
+    ("hpe", 0, np.float64, lambda d: support.hpe_case(0, d)),
+    ("sap", 1, np.float32, lambda d: support.sap_case(1, d)),
+    ("sap", 1, np.float64, lambda d: support.sap_case(1, d)),
+    ("opsa", 2, np.float32, lambda d: support.opsa_case(2, d)),
+    ("opsa", 2, np.float64, lambda d: support.opsa_case(2, d)),
+    ("opsaw", 3, np.float32, lambda d: support.opsaw_case(3, d)),
+    ("sasaw", 4, np.float32, lambda d: support.sasaw_case(4, d)),
+    ("sasaw", 4, np.float64, lambda d: support.sasaw_case(4, d)),
+]
+
+
+@pytest.mark.parametrize(
+    "op,config,dtype,build", BASELINE, ids=[f"c{c}-{o}-{np.dtype(t).name}" for o, c, t, _ in BASELINE]
+)
+def test_baseline_configuration(oracle, device, op, config, dtype, build):
+    case = build(dtype)
+    on_device = to_device(case, device)
+    out = hip_forward(op, on_device).cpu().numpy()
+    assert_close(out, cpu_forward(oracle, op, case), dtype, f"c{config} {op} forward")
+    expected = cpu_vjp(oracle, op, case)
+    grads = hip_vjp(op, on_device)
+    for key in OPS[op].differentiable:
+        assert_close(grads[key].cpu().numpy(), expected[key], dtype, f"c{config} {op} grad_{key}")
+
+    # size-independent properties, float64 accumulation on the host
+    rng = np.random.default_rng(99)
+    g = case["grad_output"].astype(np.float64)
+    if op != "hpe":
+        # adjoint identity: <vjp_x(g), dx> == <g, f(x := dx)> (multilinear operations)
+        for key in OPS[op].differentiable:
+            dx = rng.normal(size=case[key].shape).astype(dtype)
+            swapped = dict(on_device)
+            swapped[key] = to_device({"x": dx}, device)["x"]
+            right = np.sum(g * hip_forward(op, swapped).cpu().numpy())
+            product = grads[key].cpu().numpy().astype(np.float64) * dx
+            left = np.sum(product)
+            assert abs(left - right) <= support.TOLERANCE[np.dtype(dtype)] * 100 * np.sum(np.abs(product)), (op, key)
+    else:
+        # homogeneity: scaling A by t scales O by t^order
+        scaled = dict(on_device)
+        scaled["A"] = on_device["A"] * 2.0
+        order = case["indices_A"].shape[1]
+        assert_close(hip_forward(op, scaled).cpu().numpy(), out * 2.0**order, dtype, "hpe homogeneity")
