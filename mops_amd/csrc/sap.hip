@@ -401,7 +401,11 @@ void sparse_accumulation_of_products_vjp(MOPS_SAP_VJP_PARAMS(MOPS_CXX_FIRST, MOP
     const size_t shared_elements = (static_cast<size_t>(nO) + nA + nB) * ROW_STRIDE;
     const size_t per_wave =
         ((want_A ? static_cast<size_t>(nA) : 0) + (want_B ? static_cast<size_t>(nB) : 0)) * ROWS;
-    int waves = pick_waves<scalar_t>(n_blocks, shared_elements, std::max<size_t>(per_wave, 1));
+    // how the table is split over waves fixes the order of the additions: size
+    // the split as if both gradients were requested, so that a gradient has
+    // the same bits whether or not the other one is computed alongside
+    const size_t per_wave_both = (static_cast<size_t>(nA) + nB) * ROWS;
+    int waves = pick_waves<scalar_t>(n_blocks, shared_elements, std::max<size_t>(per_wave_both, 1));
     // the grid depends on the batch size only, whichever gradients are
     // requested (the reference sizes it from grad_A and launches nothing when
     // only grad_B is wanted, mops/src/sap/sap.cu:300)
