@@ -24,7 +24,6 @@ struct ThreadState {
     size_t capacity = 0;
     int device = -1;
     hipStream_t block_stream = nullptr;
-    hipEvent_t block_event = nullptr;
 };
 
 ThreadState& state() {
@@ -51,11 +50,6 @@ bool set_synchronous(bool value) {
 void finish_call(const char* operation) {
     check_hip(hipGetLastError(), operation);
     auto& st = state();
-    if (st.block != nullptr && st.block_event != nullptr) {
-        // mark the point after which the scratch block is free again
-        check_hip(hipEventRecord(st.block_event, st.stream), operation);
-        st.block_stream = st.stream;
-    }
     if (st.synchronous) {
         check_hip(hipStreamSynchronize(st.stream), operation);
     }
@@ -71,10 +65,8 @@ void* scratch(size_t bytes) {
         int restore = device;
         MOPS_HIP_CHECK(hipSetDevice(st.device));
         MOPS_HIP_CHECK(hipFree(st.block));
-        MOPS_HIP_CHECK(hipEventDestroy(st.block_event));
         MOPS_HIP_CHECK(hipSetDevice(restore));
         st.block = nullptr;
-        st.block_event = nullptr;
         st.capacity = 0;
     }
 
@@ -84,13 +76,28 @@ void* scratch(size_t bytes) {
             capacity = size_t(1) << 20;
         }
         MOPS_HIP_CHECK(hipMalloc(&st.block, capacity));
-        MOPS_HIP_CHECK(hipEventCreateWithFlags(&st.block_event, hipEventDisableTiming));
         st.capacity = capacity;
         st.device = device;
         st.block_stream = st.stream;
     } else if (st.block_stream != st.stream) {
-        // the previous user ran on another stream: order this one behind it
-        MOPS_HIP_CHECK(hipStreamWaitEvent(st.stream, st.block_event, 0));
+        // The previous user of the block ran on another stream: let it finish
+        // before this stream overwrites the block. Streams that are being
+        // captured into a graph cannot be waited for (and their work does not
+        // run now anyway); ordering graph replays is the caller's business.
+        hipStreamCaptureStatus previous = hipStreamCaptureStatusNone;
+        hipStreamCaptureStatus next = hipStreamCaptureStatusNone;
+        // the previous stream may have been destroyed by its owner meanwhile:
+        // then there is nothing left to wait for
+        bool previous_alive = hipStreamIsCapturing(st.block_stream, &previous) == hipSuccess;
+        if (!previous_alive) {
+            (void)hipGetLastError();
+        }
+        MOPS_HIP_CHECK(hipStreamIsCapturing(st.stream, &next));
+        if (previous_alive && previous == hipStreamCaptureStatusNone &&
+            next == hipStreamCaptureStatusNone) {
+            MOPS_HIP_CHECK(hipStreamSynchronize(st.block_stream));
+        }
+        st.block_stream = st.stream;
     }
     return st.block;
 }

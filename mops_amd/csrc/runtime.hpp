@@ -36,8 +36,10 @@ void finish_call(const char* operation);
 
 /// Scratch device memory of at least `bytes` bytes, 256-byte aligned, valid
 /// until the next call of this function on the same thread. The block is
-/// cached per thread and grows on demand; work enqueued on a different
-/// stream than the previous user is ordered behind it by a stream wait.
+/// cached per thread and grows on demand (growing frees the old block, which
+/// waits for the device); when the calling thread switches to another stream
+/// the previous stream is drained first, so two streams never share the
+/// block at the same time.
 void* scratch(size_t bytes);
 
 /// ceil(a / b) for positive b.
