@@ -24,6 +24,17 @@ __host__ __device__ __forceinline__ int round_up_wave(int n) {
     return (n + WAVE - 1) / WAVE * WAVE;
 }
 
+/// `pointer[index]` when `ok`, else 0, WITHOUT a branch: the load is always
+/// issued (from element 0 when not ok, which must exist) and the value is
+/// selected afterwards. A conditional load would be compiled to a branch
+/// that waits for its own load, which serialises a batch of loads that are
+/// meant to be in flight together.
+template <typename T>
+__device__ __forceinline__ T load_or_zero(const T* __restrict__ pointer, size_t index, bool ok) {
+    const T value = pointer[ok ? index : 0];
+    return ok ? value : T(0);
+}
+
 } // namespace mops::amd
 
 #endif

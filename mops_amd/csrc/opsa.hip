@@ -4,21 +4,32 @@
 //   OPSA   O[P[j], k, l]  += A[j, k] * B[j, l]
 //   OPSAW  O[PO[e], k, l] += A[e, k] * B[e, l] * W[PW[e], l]
 //
-// The scatter index is sorted, so the edges of one output row are one
-// contiguous segment [first, last) given by first_occurrences. Each output
-// row is owned by one workgroup that reduces its segment in registers and
-// writes the row once: no atomics, a fixed summation order (ascending edge
-// number, the order of the reference's CPU loops), and rows without edges
-// are written as exact zeros.
-//
 // Reference semantics restated here: mops/src/opsa/cpu.tpp:9-112 and
 // mops/src/opsaw/cpu.tpp:9-131 of lab-cosmo/mops (formulas, optional
-// gradients, zero rows); the reference's CUDA OPSA kernels
-// (mops/src/opsa/opsa.cu:14-284) use the same one-block-per-row split but
-// read A and B from global memory once per output element; OPSAW has no
-// reference device code at all (mops/src/opsaw/opsaw.cu:1).
+// gradients, rows without edges are zero). The reference's CUDA OPSA kernels
+// (mops/src/opsa/opsa.cu:14-284) run first_occurrences as a separate launch
+// and then one block per output row that reads A and B from global memory
+// once per output element; OPSAW has no reference device code at all
+// (mops/src/opsaw/opsaw.cu:1).
+//
+// Here the scatter index is sorted, so the edges of one output row are one
+// contiguous segment, and per segment the operation is a small dense
+// contraction over the edges:
+//
+//   forward   O[i]      = A_seg^T  (K x n) * B_seg (n x L)        (B_seg scaled by W rows for OPSAW)
+//   vjp       grad_B_seg = A_seg   (n x K) * G[i]  (K x L)
+//             grad_A_seg = B_seg   (n x L) * G[i]^T (L x K)
+//
+// Each segment is owned by one wavefront (segment_walk.hpp: found from the
+// index itself inside the same kernel, no boundary table, no second launch),
+// which runs the contraction on the matrix cores with 16x16x4 MFMA tiles in
+// the element type of the data (mfma.hpp) and writes its rows once. Operands
+// are loaded from global memory directly in the register layout the
+// instruction wants: for A_seg^T that is 4 consecutive rows of A per load,
+// i.e. one contiguous stretch of memory. No LDS, no atomics; the summation
+// order is fixed (ascending edge number in steps of four), so results are
+// bit-reproducible.
 #include <algorithm>
-#include <vector>
 
 #include "mops/opsa.hpp"
 #include "mops/opsaw.hpp"
@@ -27,114 +38,277 @@
 #include "device_common.hpp"
 #include "first_occurrences.hpp"
 #include "index_validation.hpp"
+#include "mfma.hpp"
 #include "runtime.hpp"
+#include "segment_walk.hpp"
 #include "sender_buckets.hpp"
 
 namespace mops::amd {
 namespace {
 
-// LDS the staging buffers of one workgroup may use. Well below the 160 KB of
-// a gfx950 CU so that several workgroups stay resident per CU.
-constexpr size_t STAGING_BYTES = 32 * 1024;
-constexpr int MAX_THREADS = 1024;
+constexpr int CHUNK = 32;            // index positions per wavefront
+constexpr int WAVES_PER_BLOCK = 4;   // independent wavefronts share a workgroup
+constexpr int BLOCK = WAVES_PER_BLOCK * WAVE;
 
 // ---------------------------------------------------------------------------
-// forward
-//
-// grid: one workgroup per output row; thread t owns output element
-// (k, l) = (t / L, t % L) (and t + blockDim, ... when K*L > blockDim).
-// The segment is streamed through LDS in chunks of `chunk` edges with
-// coalesced loads of the contiguous rows A[first..], B[first..]; for OPSAW the
-// weight row W[PW[e]] is folded into the staged copy of B, so the inner loop
-// is the same two LDS reads and one FMA per edge for both operations.
+// forward, one segment: O_row[K, L] = sum_e A[e, :]^T (B[e, :] (* W[PW[e], :]))
+// NT = number of 16-column tiles of L accumulated at once.
+// MFMA roles: D rows = k, D columns = l, reduction = edges (4 per instruction)
 // ---------------------------------------------------------------------------
-template <typename T, bool WEIGHTED>
-__global__ __launch_bounds__(MAX_THREADS) void forward_kernel(
+template <typename T, int NT, bool WEIGHTED>
+__device__ __forceinline__ void forward_segment(
+    T* __restrict__ out_row,
+    const T* __restrict__ A,
+    const T* __restrict__ B,
+    const T* __restrict__ W,
+    const int32_t* __restrict__ indices_W,
+    int32_t n_weights,
+    int32_t first,
+    int32_t last,
+    int32_t K,
+    int32_t L
+) {
+    using M = Mfma<T>;
+    constexpr int UNROLL = 8; // 32 edges in flight per iteration
+    const int lane = threadIdx.x & (WAVE - 1);
+    const int sub = lane & 15;
+    const int quarter = lane >> 4;
+
+    for (int32_t k0 = 0; k0 < K; k0 += 16) {
+        const int32_t k = k0 + sub;
+        const bool k_ok = k < K;
+        for (int32_t l0 = 0; l0 < L; l0 += 16 * NT) {
+            typename M::Acc acc[NT];
+#pragma unroll
+            for (int t = 0; t < NT; t++) {
+                acc[t] = M::zero();
+            }
+            for (int32_t e0 = first; e0 < last; e0 += 4 * UNROLL) {
+                T a[UNROLL];
+                T b[UNROLL][NT];
+#pragma unroll
+                for (int u = 0; u < UNROLL; u++) {
+                    const int32_t e = e0 + 4 * u + quarter;
+                    const bool e_ok = e < last;
+                    a[u] = load_or_zero(A, static_cast<size_t>(e) * K + k, e_ok && k_ok);
+                    int32_t w_row = -1;
+                    if (WEIGHTED) {
+                        const int32_t loaded = indices_W[e_ok ? e : first];
+                        w_row = e_ok ? loaded : -1;
+                    }
+#pragma unroll
+                    for (int t = 0; t < NT; t++) {
+                        const int32_t col = l0 + 16 * t + sub;
+                        T value = load_or_zero(B, static_cast<size_t>(e) * L + col, e_ok && col < L);
+                        if (WEIGHTED) {
+                            value *= load_or_zero(
+                                W,
+                                static_cast<size_t>(w_row) * L + col,
+                                in_bounds(w_row, n_weights) && col < L
+                            );
+                        }
+                        b[u][t] = value;
+                    }
+                }
+                // keep every load above ahead of the first matrix instruction:
+                // the loads of all 32 edges are meant to be in flight together
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int u = 0; u < UNROLL; u++) {
+#pragma unroll
+                    for (int t = 0; t < NT; t++) {
+                        acc[t] = M::mma(a[u], b[u][t], acc[t]);
+                    }
+                }
+            }
+#pragma unroll
+            for (int t = 0; t < NT; t++) {
+                const int32_t col = l0 + 16 * t + sub;
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    const int32_t row_k = k0 + M::row(lane, r);
+                    if (row_k < K && col < L) {
+                        out_row[static_cast<size_t>(row_k) * L + col] = acc[t][r];
+                    }
+                }
+            }
+        }
+    }
+}
+
+template <typename T, int NT, bool WEIGHTED>
+__global__ __launch_bounds__(BLOCK) void forward_kernel(
     T* __restrict__ output,
     const T* __restrict__ A,
     const T* __restrict__ B,
     const T* __restrict__ W,
     const int32_t* __restrict__ indices_W,
-    const int32_t* __restrict__ segments,
+    const int32_t* __restrict__ indices_output,
+    int32_t n_edges,
     int32_t n_output,
-    int32_t n_weights,
     int32_t K,
-    int32_t L,
-    int32_t chunk
+    int32_t L
 ) {
-    extern __shared__ __align__(16) unsigned char lds_bytes[];
-    T* a_stage = reinterpret_cast<T*>(lds_bytes);
-    T* b_stage = a_stage + static_cast<size_t>(chunk) * K;
-
-    const int32_t row = blockIdx.x;
-    const int tid = threadIdx.x;
-    const int nthreads = blockDim.x;
-    const int32_t first = segments[row];
-    const int32_t last = segments[n_output + row];
-    const int32_t KL = K * L;
-    T* out_row = output + static_cast<size_t>(row) * KL;
-
-    for (int32_t tile = 0; tile < KL; tile += nthreads) {
-        const int32_t element = tile + tid;
-        const bool active = element < KL;
-        const int32_t k = active ? element / L : 0;
-        const int32_t l = active ? element - k * L : 0;
-        T sum = 0;
-
-        for (int32_t c0 = first; c0 < last; c0 += chunk) {
-            const int32_t n = min(chunk, last - c0);
-            __syncthreads();
-            const T* a_src = A + static_cast<size_t>(c0) * K;
-            for (int32_t i = tid; i < n * K; i += nthreads) {
-                a_stage[i] = a_src[i];
-            }
-            const T* b_src = B + static_cast<size_t>(c0) * L;
-            for (int32_t i = tid; i < n * L; i += nthreads) {
-                T value = b_src[i];
-                if (WEIGHTED) {
-                    int32_t e = i / L;
-                    int32_t col = i - e * L;
-                    int32_t w_row = indices_W[c0 + e];
-                    value = in_bounds(w_row, n_weights)
-                                ? value * W[static_cast<size_t>(w_row) * L + col]
-                                : T(0);
-                }
-                b_stage[i] = value;
-            }
-            __syncthreads();
-            if (active) {
-                const T* a_ptr = a_stage + k;
-                const T* b_ptr = b_stage + l;
-                for (int32_t e = 0; e < n; e++) {
-                    sum += a_ptr[e * K] * b_ptr[e * L];
-                }
+    const int32_t wave_index =
+        __builtin_amdgcn_readfirstlane(blockIdx.x * WAVES_PER_BLOCK + (threadIdx.x >> 6));
+    const int lane = threadIdx.x & (WAVE - 1);
+    const size_t row_elements = static_cast<size_t>(K) * L;
+    walk_owned_segments<CHUNK>(
+        indices_output,
+        n_edges,
+        n_output,
+        wave_index,
+        [&](int32_t row, int32_t first, int32_t last) {
+            forward_segment<T, NT, WEIGHTED>(
+                output + row * row_elements, A, B, W, indices_W, n_output, first, last, K, L
+            );
+        },
+        [&](int32_t begin, int32_t end) {
+            T* base = output + begin * row_elements;
+            const size_t count = (end - begin) * row_elements;
+            for (size_t i = lane; i < count; i += WAVE) {
+                base[i] = T(0);
             }
         }
-        if (active) {
-            out_row[element] = sum;
-        }
+    );
+}
+
+// every element of `data` := 0 (used when there is no edge at all)
+template <typename T>
+__global__ __launch_bounds__(256) void zero_kernel(T* __restrict__ data, size_t count) {
+    for (size_t i = blockIdx.x * static_cast<size_t>(256) + threadIdx.x; i < count;
+         i += static_cast<size_t>(gridDim.x) * 256) {
+        data[i] = T(0);
     }
 }
 
 // ---------------------------------------------------------------------------
-// vjp with respect to A and B (and, for OPSAW, the per-edge term of grad_W)
+// vjp. One wavefront per workgroup; per segment, in stages of up to 32 edges:
 //
-// grid: one workgroup per output row. The row's grad_output tile [K, L] is
-// staged once in LDS (row stride padded to an odd length so that walking a
-// column is conflict-free) and reused by every edge of the segment:
+//   S      = A_stage (n x K) * G (K x L)      -> grad_B = S (* W rows), edge_W = S * B
+//   grad_A = BW_stage (n x L) * G^T (L x K)   with BW = B (* W rows)
 //
-//   S[e, l]      = sum_k G[k, l] * A[e, k]
-//   grad_A[e, k] = sum_l G[k, l] * B[e, l] (* W[PW[e], l])
-//   grad_B[e, l] = S[e, l]                 (* W[PW[e], l])
-//   edge_W[e, l] = S[e, l] * B[e, l]        -> summed per sender afterwards
-//
-// Results are written with consecutive threads on consecutive addresses
-// (the edges of a segment are contiguous rows of grad_A / grad_B).
-// STAGE_G = false is the fallback for tiles too large for LDS: G is then read
-// from global memory.
+// MFMA roles: D rows = edges (16 per tile), D columns = l (or k), reduction =
+// k (or l). G (the segment's grad_output row) and the stage's rows of A, B
+// (and the gathered W rows) are first copied to LDS with row-contiguous loads
+// that are all in flight together, then fed to the matrix cores from LDS.
+// LDS rows have an odd stride so that the column walks of the operand reads
+// (stride = one row) spread over the banks. `shift_K` / `shift_L` are
+// log2 of the row widths rounded up to a power of two: a wavefront copies
+// 64 >> shift rows per load instruction, lane = (row, column) without any
+// integer division.
 // ---------------------------------------------------------------------------
-template <typename T, bool WEIGHTED, bool STAGE_G>
-__global__ __launch_bounds__(MAX_THREADS) void vjp_kernel(
+constexpr int STAGE_EDGES = 32;
+
+// A batch of up to U row-passes held in registers between the global loads
+// and the LDS stores, so that the loads of several batches (G, A and B) are
+// all issued before the first one is waited for.
+template <typename T, int U> struct RowBatch {
+    T value[U];
+    int32_t lds_offset[U]; // -1: nothing to store
+
+    /// Issue the loads of passes [pass0, pass0 + U) of a [n_rows, width] block.
+    __device__ __forceinline__ void load(
+        const T* __restrict__ source,
+        int32_t stage_stride,
+        int32_t n_rows,
+        int32_t width,
+        int32_t shift,
+        int32_t pass0
+    ) {
+        const int lane = threadIdx.x & (WAVE - 1);
+        const int32_t column = lane & ((1 << shift) - 1);
+        const int32_t row_in_pass = lane >> shift;
+        const int32_t rows_per_pass = WAVE >> shift;
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const int32_t row = (pass0 + u) * rows_per_pass + row_in_pass;
+            const bool ok = row < n_rows && column < width;
+            value[u] = load_or_zero(source, static_cast<size_t>(row) * width + column, ok);
+            lds_offset[u] = ok ? row * stage_stride + column : -1;
+        }
+    }
+
+    __device__ __forceinline__ void store(T* __restrict__ stage) const {
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            if (lds_offset[u] >= 0) {
+                stage[lds_offset[u]] = value[u];
+            }
+        }
+    }
+};
+
+// The same for rows gathered through an index (the weight rows of OPSAW):
+// first all index loads, then all row loads, then the LDS stores.
+template <typename T, int U> struct GatherBatch {
+    T value[U];
+    int32_t lds_offset[U];
+
+    __device__ __forceinline__ void load(
+        const T* __restrict__ table,
+        const int32_t* __restrict__ row_index,
+        int32_t table_rows,
+        int32_t stage_stride,
+        int32_t n_rows,
+        int32_t width,
+        int32_t shift,
+        int32_t pass0
+    ) {
+        const int lane = threadIdx.x & (WAVE - 1);
+        const int32_t column = lane & ((1 << shift) - 1);
+        const int32_t row_in_pass = lane >> shift;
+        const int32_t rows_per_pass = WAVE >> shift;
+        int32_t source_row[U];
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const int32_t row = (pass0 + u) * rows_per_pass + row_in_pass;
+            const bool ok = row < n_rows && column < width;
+            const int32_t loaded = row_index[ok ? row : 0];
+            source_row[u] = ok ? loaded : -1;
+            lds_offset[u] = ok ? row * stage_stride + column : -1;
+        }
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            value[u] = load_or_zero(
+                table,
+                static_cast<size_t>(source_row[u]) * width + column,
+                in_bounds(source_row[u], table_rows)
+            );
+        }
+    }
+
+    __device__ __forceinline__ void store(T* __restrict__ stage) const {
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            if (lds_offset[u] >= 0) {
+                stage[lds_offset[u]] = value[u];
+            }
+        }
+    }
+};
+
+// Rows wider than a wavefront (shift > 6): plain loop, one row at a time.
+template <typename T>
+__device__ __forceinline__ void copy_wide_rows_to_lds(
+    T* __restrict__ stage, int32_t stage_stride, const T* __restrict__ source, int32_t n_rows, int32_t width
+) {
+    const int lane = threadIdx.x & (WAVE - 1);
+    for (int32_t row = 0; row < n_rows; row++) {
+        for (int32_t c = lane; c < width; c += WAVE) {
+            stage[row * stage_stride + c] = source[static_cast<size_t>(row) * width + c];
+        }
+    }
+}
+
+// Passes needed to copy n_rows rows when 64 >> shift rows go per pass.
+__device__ __forceinline__ int32_t passes_for(int32_t n_rows, int32_t shift) {
+    const int32_t rows_per_pass = WAVE >> shift;
+    return (n_rows + rows_per_pass - 1) / rows_per_pass; // shift <= 6 here, no division by zero
+}
+
+template <typename T, bool WEIGHTED>
+__global__ __launch_bounds__(WAVE) void vjp_kernel(
     T* __restrict__ grad_A,
     T* __restrict__ grad_B,
     T* __restrict__ edge_W,
@@ -143,115 +317,175 @@ __global__ __launch_bounds__(MAX_THREADS) void vjp_kernel(
     const T* __restrict__ B,
     const T* __restrict__ W,
     const int32_t* __restrict__ indices_W,
-    const int32_t* __restrict__ segments,
+    const int32_t* __restrict__ indices_output,
+    int32_t n_edges,
     int32_t n_output,
-    int32_t n_weights,
     int32_t K,
     int32_t L,
-    int32_t chunk
+    int32_t shift_K,
+    int32_t shift_L
 ) {
+    using M = Mfma<T>;
     extern __shared__ __align__(16) unsigned char lds_bytes[];
-    const int32_t row = blockIdx.x;
-    const int32_t first = segments[row];
-    const int32_t last = segments[n_output + row];
-    if (first < 0) {
-        return; // no edge reads this row of grad_output
-    }
-    const int tid = threadIdx.x;
-    const int nthreads = blockDim.x;
+    const int32_t Ks = odd_stride(K);
+    const int32_t Ls = odd_stride(L);
+    T* g_stage = reinterpret_cast<T*>(lds_bytes);        // [K][Ls]
+    T* a_stage = g_stage + K * Ls;                        // [STAGE_EDGES][Ks]
+    T* b_stage = a_stage + STAGE_EDGES * Ks;              // [STAGE_EDGES][Ls]  B
+    T* w_stage = b_stage + STAGE_EDGES * Ls;              // [STAGE_EDGES][Ls]  W rows (weighted)
 
-    const int32_t g_stride = STAGE_G ? odd_stride(L) : L;
-    T* cursor = reinterpret_cast<T*>(lds_bytes);
-    T* g_stage = cursor;
-    if (STAGE_G) {
-        cursor += static_cast<size_t>(K) * g_stride;
-    }
-    T* a_stage = cursor;
-    cursor += static_cast<size_t>(chunk) * K;
-    T* b_stage = cursor; // B, or B * W when weighted
-    cursor += static_cast<size_t>(chunk) * L;
-    T* w_stage = cursor; // only when weighted
-    if (WEIGHTED) {
-        cursor += static_cast<size_t>(chunk) * L;
-    }
-    T* braw_stage = cursor; // unweighted B, only when weighted
+    const int lane = threadIdx.x;
+    const int sub = lane & 15;
+    const int quarter = lane >> 4;
+    const size_t row_elements = static_cast<size_t>(K) * L;
+    const bool want_S = grad_B != nullptr || (WEIGHTED && edge_W != nullptr);
 
-    const T* g_global = grad_output + static_cast<size_t>(row) * K * L;
-    if (STAGE_G) {
-        for (int32_t i = tid; i < K * L; i += nthreads) {
-            int32_t k = i / L;
-            g_stage[k * g_stride + (i - k * L)] = g_global[i];
-        }
-    }
-    const T* G = STAGE_G ? g_stage : g_global;
+    walk_owned_segments<CHUNK>(
+        indices_output,
+        n_edges,
+        n_output,
+        static_cast<int32_t>(blockIdx.x),
+        [&](int32_t row, int32_t first, int32_t last) {
+            constexpr int U = 8;
+            const bool narrow = shift_K <= 6 && shift_L <= 6;
+            const T* g_source = grad_output + row * row_elements;
+            __syncthreads(); // the previous segment's LDS reads are done
 
-    for (int32_t c0 = first; c0 < last; c0 += chunk) {
-        const int32_t n = min(chunk, last - c0);
-        __syncthreads();
-        const T* a_src = A + static_cast<size_t>(c0) * K;
-        for (int32_t i = tid; i < n * K; i += nthreads) {
-            a_stage[i] = a_src[i];
-        }
-        const T* b_src = B + static_cast<size_t>(c0) * L;
-        for (int32_t i = tid; i < n * L; i += nthreads) {
-            T value = b_src[i];
-            if (WEIGHTED) {
-                int32_t e = i / L;
-                int32_t col = i - e * L;
-                int32_t w_row = indices_W[c0 + e];
-                T weight =
-                    in_bounds(w_row, n_weights) ? W[static_cast<size_t>(w_row) * L + col] : T(0);
-                w_stage[i] = weight;
-                braw_stage[i] = value;
-                value *= weight;
-            }
-            b_stage[i] = value;
-        }
-        __syncthreads();
-
-        if (grad_A != nullptr) {
-            T* dst = grad_A + static_cast<size_t>(c0) * K;
-            for (int32_t i = tid; i < n * K; i += nthreads) {
-                int32_t e = i / K;
-                int32_t k = i - e * K;
-                const T* g_row = G + k * g_stride;
-                const T* b_row = b_stage + e * L;
-                T sum = 0;
-                for (int32_t l = 0; l < L; l++) {
-                    sum += g_row[l] * b_row[l];
+            for (int32_t s0 = first; s0 < last; s0 += STAGE_EDGES) {
+                const int32_t n = min(STAGE_EDGES, last - s0);
+                const T* a_source = A + static_cast<size_t>(s0) * K;
+                const T* b_source = B + static_cast<size_t>(s0) * L;
+                if (s0 != first) {
+                    __syncthreads();
                 }
-                dst[i] = sum;
-            }
-        }
-        if (grad_B != nullptr || (WEIGHTED && edge_W != nullptr)) {
-            for (int32_t i = tid; i < n * L; i += nthreads) {
-                int32_t e = i / L;
-                int32_t l = i - e * L;
-                const T* g_col = G + l;
-                const T* a_row = a_stage + e * K;
-                T sum = 0;
-                for (int32_t k = 0; k < K; k++) {
-                    sum += g_col[k * g_stride] * a_row[k];
-                }
-                if (WEIGHTED) {
-                    if (grad_B != nullptr) {
-                        grad_B[static_cast<size_t>(c0) * L + i] = sum * w_stage[i];
+                if (narrow) {
+                    // first batches of G, A and B: all loads in flight together
+                    RowBatch<T, U> g_batch, a_batch;
+                    RowBatch<T, 2 * U> b_batch;
+                    const bool with_g = s0 == first;
+                    if (with_g) {
+                        g_batch.load(g_source, Ls, K, L, shift_L, 0);
                     }
-                    if (edge_W != nullptr) {
-                        edge_W[static_cast<size_t>(c0) * L + i] = sum * braw_stage[i];
+                    a_batch.load(a_source, Ks, n, K, shift_K, 0);
+                    b_batch.load(b_source, Ls, n, L, shift_L, 0);
+                    if (with_g) {
+                        g_batch.store(g_stage);
+                    }
+                    a_batch.store(a_stage);
+                    b_batch.store(b_stage);
+                    // whatever does not fit the first batch
+                    if (with_g) {
+                        for (int32_t pass = U; pass < passes_for(K, shift_L); pass += U) {
+                            g_batch.load(g_source, Ls, K, L, shift_L, pass);
+                            g_batch.store(g_stage);
+                        }
+                    }
+                    for (int32_t pass = U; pass < passes_for(n, shift_K); pass += U) {
+                        a_batch.load(a_source, Ks, n, K, shift_K, pass);
+                        a_batch.store(a_stage);
+                    }
+                    for (int32_t pass = 2 * U; pass < passes_for(n, shift_L); pass += 2 * U) {
+                        b_batch.load(b_source, Ls, n, L, shift_L, pass);
+                        b_batch.store(b_stage);
                     }
                 } else {
-                    grad_B[static_cast<size_t>(c0) * L + i] = sum;
+                    if (s0 == first) {
+                        copy_wide_rows_to_lds(g_stage, Ls, g_source, K, L);
+                    }
+                    copy_wide_rows_to_lds(a_stage, Ks, a_source, n, K);
+                    copy_wide_rows_to_lds(b_stage, Ls, b_source, n, L);
+                }
+                if (WEIGHTED) {
+                    if (narrow) {
+                        GatherBatch<T, 2 * U> w_batch;
+                        for (int32_t pass = 0; pass < passes_for(n, shift_L); pass += 2 * U) {
+                            w_batch.load(W, indices_W + s0, n_output, Ls, n, L, shift_L, pass);
+                            w_batch.store(w_stage);
+                        }
+                    } else {
+                        for (int32_t r = 0; r < n; r++) {
+                            const int32_t w_row = indices_W[s0 + r];
+                            const bool ok = in_bounds(w_row, n_output);
+                            for (int32_t c = lane; c < L; c += WAVE) {
+                                w_stage[r * Ls + c] =
+                                    ok ? W[static_cast<size_t>(w_row) * L + c] : T(0);
+                            }
+                        }
+                    }
+                }
+                __syncthreads();
+
+                for (int32_t t0 = 0; t0 < n; t0 += 16) {
+                    const int32_t local = t0 + sub;       // operand row = edge within the stage
+                    const bool edge_ok = local < n;
+
+                    if (want_S) {
+                        for (int32_t l0 = 0; l0 < L; l0 += 16) {
+                            const int32_t col = l0 + sub;
+                            typename M::Acc acc = M::zero();
+#pragma unroll 4
+                            for (int32_t kk = 0; kk < K; kk += 4) {
+                                const int32_t k = kk + quarter;
+                                const bool k_ok = k < K;
+                                const T a = load_or_zero(a_stage, local * Ks + k, edge_ok && k_ok);
+                                const T g = load_or_zero(g_stage, k * Ls + col, k_ok && col < L);
+                                acc = M::mma(a, g, acc);
+                            }
+#pragma unroll
+                            for (int r = 0; r < 4; r++) {
+                                const int32_t e_local = t0 + M::row(lane, r);
+                                if (e_local < n && col < L) {
+                                    const size_t at = static_cast<size_t>(s0 + e_local) * L + col;
+                                    if (WEIGHTED) {
+                                        if (grad_B != nullptr) {
+                                            grad_B[at] = acc[r] * w_stage[e_local * Ls + col];
+                                        }
+                                        if (edge_W != nullptr) {
+                                            edge_W[at] = acc[r] * b_stage[e_local * Ls + col];
+                                        }
+                                    } else {
+                                        grad_B[at] = acc[r];
+                                    }
+                                }
+                            }
+                        }
+                    }
+
+                    if (grad_A != nullptr) {
+                        for (int32_t k0 = 0; k0 < K; k0 += 16) {
+                            const int32_t kcol = k0 + sub;
+                            typename M::Acc acc = M::zero();
+#pragma unroll 4
+                            for (int32_t ll = 0; ll < L; ll += 4) {
+                                const int32_t l = ll + quarter;
+                                const bool l_ok = l < L;
+                                T b = load_or_zero(b_stage, local * Ls + l, edge_ok && l_ok);
+                                if (WEIGHTED) {
+                                    b *= load_or_zero(w_stage, local * Ls + l, edge_ok && l_ok);
+                                }
+                                const T g = load_or_zero(g_stage, kcol * Ls + l, kcol < K && l_ok);
+                                acc = M::mma(b, g, acc);
+                            }
+#pragma unroll
+                            for (int r = 0; r < 4; r++) {
+                                const int32_t e_local = t0 + M::row(lane, r);
+                                if (e_local < n && kcol < K) {
+                                    grad_A[static_cast<size_t>(s0 + e_local) * K + kcol] = acc[r];
+                                }
+                            }
+                        }
+                    }
                 }
             }
-        }
-    }
+        },
+        [](int32_t, int32_t) {}
+    );
 }
 
-// An edge whose scatter index lies outside [0, n_output) belongs to no segment:
-// its rows of grad_A / grad_B are then left unwritten (such input is invalid;
-// the reference's device path does not define it either). Nothing is ever read
-// or written out of bounds because of it.
+// An edge whose scatter index lies outside [0, n_output) belongs to no output
+// row: its rows of grad_A / grad_B are then left unwritten (such input is
+// invalid; the reference's device path does not define it either). Nothing is
+// ever read or written out of bounds because of it.
 
 // ---------------------------------------------------------------------------
 // grad_W[w, l] = sum over edges e with PW[e] == w of edge_W[e, l]
@@ -273,17 +507,10 @@ __global__ __launch_bounds__(256) void gather_weights_kernel(
     }
 }
 
-// Edges per LDS chunk such that `per_edge` elements per edge plus `fixed`
-// elements fit the staging budget.
-template <typename T> int32_t pick_chunk(size_t per_edge, size_t fixed) {
-    size_t budget = STAGING_BYTES / sizeof(T);
-    size_t available = budget > fixed ? budget - fixed : 0;
-    size_t chunk = per_edge > 0 ? available / per_edge : 64;
-    chunk = std::min<size_t>(chunk, 64);
-    return static_cast<int32_t>(std::max<size_t>(chunk, 1));
+unsigned blocks_for(int32_t n_edges) {
+    size_t waves = ceil_div(static_cast<size_t>(n_edges), CHUNK);
+    return static_cast<unsigned>(ceil_div(waves, WAVES_PER_BLOCK));
 }
-
-constexpr size_t LDS_LIMIT = 64 * 1024; // stay within the default dynamic-LDS limit
 
 template <typename T, bool WEIGHTED>
 void launch_forward(
@@ -304,33 +531,26 @@ void launch_forward(
         return;
     }
     hipStream_t stream = current_stream();
-    auto* segments = static_cast<int32_t*>(scratch(static_cast<size_t>(n_output) * 2 * sizeof(int32_t)));
-    first_occurrences(indices_output.data, n_edges, n_output, segments, stream);
-
-    const size_t per_edge = static_cast<size_t>(K) + L;
-    if (per_edge * sizeof(T) > LDS_LIMIT) {
-        throw std::runtime_error(
-            std::string(operation) + ": size_A + size_B = " + std::to_string(per_edge) +
-            " is too large for the device kernel (one row of A and B must fit in 64 KiB of LDS)"
-        );
+    if (n_edges == 0) {
+        const size_t count = static_cast<size_t>(n_output) * K * L;
+        unsigned blocks = static_cast<unsigned>(std::min<size_t>(ceil_div(count, 256), 4096));
+        zero_kernel<T><<<blocks, 256, 0, stream>>>(output.data, count);
+        finish_call(operation);
+        return;
     }
-    int32_t chunk = pick_chunk<T>(per_edge, 0);
-    size_t lds = static_cast<size_t>(chunk) * per_edge * sizeof(T);
-    int threads = std::min(MAX_THREADS, round_up_wave(K * L > 0 ? std::min(K * L, MAX_THREADS) : 1));
-
-    forward_kernel<T, WEIGHTED><<<n_output, threads, lds, stream>>>(
-        output.data,
-        A.data,
-        B.data,
-        W,
-        indices_W,
-        segments,
-        n_output,
-        n_output,
-        K,
-        L,
-        chunk
-    );
+    const unsigned blocks = blocks_for(n_edges);
+#define MOPS_LAUNCH_FORWARD(NT)                                                                    \
+    forward_kernel<T, NT, WEIGHTED><<<blocks, BLOCK, 0, stream>>>(                                 \
+        output.data, A.data, B.data, W, indices_W, indices_output.data, n_edges, n_output, K, L    \
+    )
+    if (L <= 16) {
+        MOPS_LAUNCH_FORWARD(1);
+    } else if (L <= 32) {
+        MOPS_LAUNCH_FORWARD(2);
+    } else {
+        MOPS_LAUNCH_FORWARD(4);
+    }
+#undef MOPS_LAUNCH_FORWARD
     finish_call(operation);
 }
 
@@ -360,48 +580,61 @@ void launch_vjp(
     narrow_i32(A.shape[1] * B.shape[1], "size_A * size_B");
     hipStream_t stream = current_stream();
 
-    // scratch: segments | edge_W (weighted, grad_W wanted) | sender buckets
-    const size_t segments_bytes = align256(static_cast<size_t>(n_output) * 2 * sizeof(int32_t));
+    // scratch: edge_W | sender buckets   (only when grad_W is wanted)
     const size_t edge_w_bytes =
         want_W ? align256(static_cast<size_t>(n_edges) * L * sizeof(T)) : 0;
     const size_t buckets_bytes = want_W ? sender_buckets_bytes(n_output, n_edges) : 0;
-    char* workspace = static_cast<char*>(scratch(segments_bytes + edge_w_bytes + buckets_bytes));
-    auto* segments = reinterpret_cast<int32_t*>(workspace);
-    T* edge_W = want_W ? reinterpret_cast<T*>(workspace + segments_bytes) : nullptr;
+    char* workspace =
+        want_W ? static_cast<char*>(scratch(edge_w_bytes + buckets_bytes)) : nullptr;
+    T* edge_W = want_W ? reinterpret_cast<T*>(workspace) : nullptr;
+
+    // degenerate shapes: a gradient that sums over an empty axis is zero
+    if (want_A && L == 0 && n_edges > 0 && K > 0) {
+        const size_t count = static_cast<size_t>(n_edges) * K;
+        zero_kernel<T><<<static_cast<unsigned>(std::min<size_t>(ceil_div(count, 256), 4096)), 256, 0, stream>>>(
+            grad_A.data, count
+        );
+    }
+    if (want_B && K == 0 && n_edges > 0 && L > 0) {
+        const size_t count = static_cast<size_t>(n_edges) * L;
+        zero_kernel<T><<<static_cast<unsigned>(std::min<size_t>(ceil_div(count, 256), 4096)), 256, 0, stream>>>(
+            grad_B.data, count
+        );
+    }
+    if (want_W && K == 0 && n_edges > 0 && L > 0) {
+        const size_t count = static_cast<size_t>(n_edges) * L;
+        zero_kernel<T><<<static_cast<unsigned>(std::min<size_t>(ceil_div(count, 256), 4096)), 256, 0, stream>>>(
+            edge_W, count
+        );
+    }
 
     if (n_output > 0 && n_edges > 0 && K > 0 && L > 0) {
-        first_occurrences(indices_output.data, n_edges, n_output, segments, stream);
-
-        const size_t g_elements = static_cast<size_t>(K) * odd_stride(L);
-        const bool stage_g = g_elements * sizeof(T) <= STAGING_BYTES;
-        const size_t per_edge = static_cast<size_t>(K) + (WEIGHTED ? 3 : 1) * static_cast<size_t>(L);
-        if (per_edge * sizeof(T) > LDS_LIMIT / 2) {
+        const size_t Ks = odd_stride(K), Ls = odd_stride(L);
+        const size_t lds =
+            (K * Ls + STAGE_EDGES * Ks + (WEIGHTED ? 2 : 1) * STAGE_EDGES * Ls) * sizeof(T);
+        if (lds > 64 * 1024) {
             throw std::runtime_error(
-                std::string(operation) + ": size_A and size_B are too large for the device kernel"
+                std::string(operation) + ": size_A * size_B = " + std::to_string(K) + " * " +
+                std::to_string(L) + " is too large for the LDS tile of the device kernel"
             );
         }
-        int32_t chunk = pick_chunk<T>(per_edge, 0);
-        size_t lds = (static_cast<size_t>(chunk) * per_edge + (stage_g ? g_elements : 0)) * sizeof(T);
-        int widest = std::max(K, L) * chunk;
-        int threads = std::min(256, round_up_wave(std::max(widest, 1)));
-
-        if (stage_g) {
-            vjp_kernel<T, WEIGHTED, true><<<n_output, threads, lds, stream>>>(
-                grad_A.data, grad_B.data, edge_W, grad_output.data, A.data, B.data, W, indices_W,
-                segments, n_output, n_output, K, L, chunk
-            );
-        } else {
-            vjp_kernel<T, WEIGHTED, false><<<n_output, threads, lds, stream>>>(
-                grad_A.data, grad_B.data, edge_W, grad_output.data, A.data, B.data, W, indices_W,
-                segments, n_output, n_output, K, L, chunk
-            );
-        }
+        auto log2_ceil = [](int32_t n) {
+            int32_t shift = 0;
+            while ((1 << shift) < n) {
+                shift++;
+            }
+            return shift;
+        };
+        const unsigned waves = static_cast<unsigned>(ceil_div(static_cast<size_t>(n_edges), CHUNK));
+        vjp_kernel<T, WEIGHTED><<<waves, WAVE, lds, stream>>>(
+            grad_A.data, grad_B.data, edge_W, grad_output.data, A.data, B.data, W, indices_W,
+            indices_output.data, n_edges, n_output, K, L, log2_ceil(K), log2_ceil(L)
+        );
     }
 
     if (want_W && n_output > 0 && L > 0) {
-        SenderBuckets buckets = build_sender_buckets(
-            indices_W, n_edges, n_output, workspace + segments_bytes + edge_w_bytes, stream
-        );
+        SenderBuckets buckets =
+            build_sender_buckets(indices_W, n_edges, n_output, workspace + edge_w_bytes, stream);
         int threads = std::min(256, round_up_wave(L));
         gather_weights_kernel<T><<<n_output, threads, 0, stream>>>(grad_W.data, edge_W, buckets, L);
     }
