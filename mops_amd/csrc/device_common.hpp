@@ -24,6 +24,32 @@ __host__ __device__ __forceinline__ int round_up_wave(int n) {
     return (n + WAVE - 1) / WAVE * WAVE;
 }
 
+/// Division of small non-negative integers by a run-time constant without a
+/// divide: the host computes `magic = ceil(2^32 / divisor)` once, the device
+/// takes the high half of a 32x32 multiplication. Exact for all
+/// 0 <= n with n * divisor < 2^32 (checked by the host before it picks a
+/// kernel that uses this). An integer division by a run-time value costs
+/// some thirty instructions on this hardware; index arithmetic of that kind
+/// in front of every element dominated the instruction count of the staging
+/// loops before.
+struct FastDivisor {
+    uint32_t divisor;
+    uint32_t magic;
+
+    __host__ static FastDivisor make(uint32_t divisor) {
+        FastDivisor d;
+        d.divisor = divisor;
+        d.magic = divisor <= 1
+                      ? 0u
+                      : static_cast<uint32_t>(((uint64_t(1) << 32) + divisor - 1) / divisor);
+        return d;
+    }
+
+    __device__ __forceinline__ uint32_t divide(uint32_t n) const {
+        return divisor <= 1 ? n : __umulhi(n, magic);
+    }
+};
+
 /// `pointer[index]` when `ok`, else 0, WITHOUT a branch: the load is always
 /// issued (from element 0 when not ok, which must exist) and the value is
 /// selected afterwards. A conditional load would be compiled to a branch
