@@ -45,6 +45,7 @@
 #include "first_occurrences.hpp"
 #include "index_validation.hpp"
 #include "runtime.hpp"
+#include "sasaw_mfma.hpp"
 #include "sender_buckets.hpp"
 
 namespace mops::amd {
@@ -598,6 +599,19 @@ void sparse_accumulation_scatter_add_with_weights(MOPS_SASAW_PARAMS(MOPS_CXX_FIR
     }
     hipStream_t stream = current_stream();
 
+    const sasaw_mfma::Shape shape{s.n_nodes, s.n_edges, s.nA, s.L, s.N, s.n2, s.n3};
+    if (sasaw_mfma::supports(shape, sizeof(scalar_t))) {
+        const sasaw_mfma::Indices indices{
+            indices_A.data, indices_W_1.data, indices_W_2.data, indices_output_1.data, indices_output_2.data
+        };
+        void* workspace = scratch(sasaw_mfma::workspace_bytes(shape, sizeof(scalar_t)));
+        sasaw_mfma::forward<scalar_t>(
+            output.data, A.data, B.data, C.data, W.data, indices, shape, workspace, stream
+        );
+        finish_call(operation);
+        return;
+    }
+
     const size_t segments_bytes = align256(static_cast<size_t>(s.n_nodes) * 2 * sizeof(int32_t));
     char* workspace = static_cast<char*>(
         scratch(segments_bytes + plan_bytes<scalar_t>(s.N, s.n_cells, s.nA))
@@ -658,6 +672,20 @@ void sparse_accumulation_scatter_add_with_weights_vjp(MOPS_SASAW_VJP_PARAMS(MOPS
 
     const Sizes s = sizes_of(grad_output, A, B, C, W);
     hipStream_t stream = current_stream();
+
+    const sasaw_mfma::Shape shape{s.n_nodes, s.n_edges, s.nA, s.L, s.N, s.n2, s.n3};
+    if (sasaw_mfma::supports(shape, sizeof(scalar_t))) {
+        const sasaw_mfma::Indices indices{
+            indices_A.data, indices_W_1.data, indices_W_2.data, indices_output_1.data, indices_output_2.data
+        };
+        void* workspace = scratch(sasaw_mfma::workspace_bytes(shape, sizeof(scalar_t)));
+        sasaw_mfma::vjp<scalar_t>(
+            grad_A.data, grad_B.data, grad_W.data, grad_output.data, A.data, B.data, C.data, W.data, indices,
+            shape, workspace, stream
+        );
+        finish_call(operation);
+        return;
+    }
 
     const size_t segments_bytes = align256(static_cast<size_t>(s.n_nodes) * 2 * sizeof(int32_t));
     const size_t table_bytes = plan_bytes<scalar_t>(s.N, s.n_cells, s.nA);

@@ -1,0 +1,1062 @@
+// SASAW on the matrix cores of gfx950.
+//
+//   O[PO1[e], PO2[n], :] += C[n] * A[e, PA[n]] * B[e, :] * W[PW1[e], PW2[n], :]
+//
+// (semantics: mops/src/sasaw/cpu.tpp:8-171 of lab-cosmo/mops). For the table
+// shapes of equivariant message passing every index of the coupling table has
+// a handful of values, so the table is first made DENSE,
+//
+//   D[cell, m1] = sum of C[n] over entries with (PO2[n], PW2[n]) == cell, PA[n] == m1
+//   (cell = m3 * n2 + m2),
+//
+// and everything else becomes small matrix products on v_mfma_*_16x16x4:
+//
+//   T[cell, e]     = sum_m1 D[cell, m1] * A[e, m1]                  16 edges at a time
+//   O[i, m3, l]    = sum_e sum_m2 T[(m3, m2), e] * (B[e, l] * W[PW1[e], m2, l])
+//   grad_W[w,m2,l] = sum_e sum_m3 T[(m3, m2), e] * (B[e, l] * G[PO1[e], m3, l])
+//   P_e[m3, l]     = sum_m2 T[(m3, m2), e] * W[PW1[e], m2, l];  grad_B[e, l] = sum_m3 G[i, m3, l] * P_e[m3, l]
+//   U_e[m3, m2]    = sum_l G[i, m3, l] * (B[e, l] * W[PW1[e], m2, l])
+//   grad_A[e, m1]  = sum_cell U_e[cell] * D[cell, m1]              16 edges at a time
+//
+// The forward pass and grad_W are the same contraction with the roles of m2
+// and m3 exchanged, and share their code.
+//
+// The whole call lasts microseconds and every wavefront sees a few dozen
+// edges, so what counts is (a) the number of instructions around every matrix
+// instruction and (b) that no wavefront has much more to do than the others:
+//  - everything that depends only on the lane is computed once per kernel
+//    (byte offsets into blocks, LDS rows); addresses are a uniform base in
+//    scalar registers plus one of those offsets plus an immediate;
+//  - operand arrays are padded with zeros up to fixed loop bounds instead of
+//    being guarded (a matrix instruction on zeros costs what a branch costs);
+//  - forward: a workgroup of four wavefronts owns the receiver segments that
+//    start in its 64 positions of the sorted index and deals their 16-edge
+//    stages out in turn; partial sums meet in LDS in a fixed order;
+//  - grad_A / grad_B: one wavefront per 16 consecutive edges, whatever
+//    segments they belong to;
+//  - grad_W: one wavefront per sender, senders found by sender_gather.hpp.
+// Sums never depend on the launch or on timing: no atomics anywhere.
+#include "sasaw_mfma.hpp"
+
+#include <algorithm>
+#include <stdexcept>
+#include <type_traits>
+
+#include "device_common.hpp"
+#include "mfma.hpp"
+#include "runtime.hpp"
+#include "segment_walk.hpp"
+#include "sender_gather.hpp"
+
+namespace mops::amd::sasaw_mfma {
+namespace {
+
+__host__ __device__ constexpr size_t align16(size_t bytes) { return (bytes + 15) & ~static_cast<size_t>(15); }
+
+constexpr int STAGE = 16;      // edges per matrix tile
+constexpr int MAX_A_STEPS = 4; // nA <= 16
+constexpr int MAX_INDEX = 16;  // n2, n3 <= 16
+constexpr int MAX_L = 64;
+constexpr int T_ROW = STAGE + 1; // LDS row of one cell: 16 edges, one more to spread the banks
+constexpr int TILE_GROUP = 3;    // tiles of 16 cells handled together
+constexpr int STEP_GROUP = 8;    // steps of 4 cells handled together
+constexpr size_t LDS_BUDGET = 64 * 1024;
+
+template <typename T>
+__device__ __forceinline__ T load_at(const T* __restrict__ base, uint32_t byte_offset) {
+    return *reinterpret_cast<const T*>(reinterpret_cast<const char*>(base) + byte_offset);
+}
+
+template <typename T>
+__device__ __forceinline__ void store_at(T* __restrict__ base, uint32_t byte_offset, T value) {
+    *reinterpret_cast<T*>(reinterpret_cast<char*>(base) + byte_offset) = value;
+}
+
+// ---------------------------------------------------------------------------
+// the dense table, laid out as matrix operands and padded with zeros
+
+struct DenseLayout {
+    int32_t n_cells;
+    int32_t n_cell_tiles; // tiles of 16 cells, a multiple of TILE_GROUP
+    int32_t cell_steps;   // steps of 4 cells, a multiple of STEP_GROUP
+    int32_t lds_cells;    // rows of the T area in LDS
+    int32_t zero_cell;    // a row of it that stays zero
+    int32_t dump_cell;    // a row of it nobody reads
+
+    __host__ __device__ int32_t to_cells_slots() const { return n_cell_tiles * MAX_A_STEPS * WAVE; }
+    __host__ __device__ int32_t to_A_slots() const { return cell_steps * WAVE; }
+    __host__ __device__ int32_t t_elements() const { return lds_cells * T_ROW; }
+};
+
+int32_t round_up(int32_t value, int32_t multiple) { return (value + multiple - 1) / multiple * multiple; }
+
+DenseLayout dense_layout(const Shape& s) {
+    DenseLayout d;
+    d.n_cells = s.n3 * s.n2;
+    d.n_cell_tiles = round_up((d.n_cells + 15) / 16, TILE_GROUP);
+    d.cell_steps = round_up((d.n_cells + 3) / 4, STEP_GROUP);
+    const int32_t rows = std::max(16 * d.n_cell_tiles, 4 * d.cell_steps);
+    d.zero_cell = rows;
+    d.dump_cell = rows + 1;
+    d.lds_cells = rows + 2;
+    return d;
+}
+
+constexpr int DENSE_THREADS = 256;
+constexpr int TABLE_TILE = 1024;
+
+// Every thread owns one operand slot and adds up, in ascending entry order,
+// the coefficients of the entries that fall on it.
+//   to_cells[(tile * MAX_A_STEPS + step) * 64 + lane] = D[16 * tile + (lane & 15)][4 * step + (lane >> 4)]
+//   to_A[step * 64 + lane]                            = D[4 * step + (lane >> 4)][lane & 15]
+template <typename T>
+__global__ __launch_bounds__(DENSE_THREADS) void dense_coupling_kernel(
+    T* __restrict__ to_cells,
+    T* __restrict__ to_A,
+    const T* __restrict__ C,
+    const int32_t* __restrict__ PA,
+    const int32_t* __restrict__ PW2,
+    const int32_t* __restrict__ PO2,
+    int32_t N,
+    int32_t nA,
+    int32_t n2,
+    int32_t n3,
+    DenseLayout layout
+) {
+    __shared__ int32_t keys[TABLE_TILE];
+    __shared__ T coefficients[TABLE_TILE];
+
+    const int tid = threadIdx.x;
+    const int32_t slot = blockIdx.x * DENSE_THREADS + tid;
+    const int32_t n_to_cells = layout.to_cells_slots();
+    const int32_t n_slots = n_to_cells + layout.to_A_slots();
+
+    int32_t cell = -1;
+    int32_t m1 = -1;
+    if (slot < n_to_cells) {
+        const int lane = slot & (WAVE - 1);
+        const int32_t tile_step = slot >> 6;
+        cell = 16 * (tile_step / MAX_A_STEPS) + (lane & 15);
+        m1 = 4 * (tile_step % MAX_A_STEPS) + (lane >> 4);
+    } else if (slot < n_slots) {
+        const int32_t local = slot - n_to_cells;
+        const int lane = local & (WAVE - 1);
+        cell = 4 * (local >> 6) + (lane >> 4);
+        m1 = lane & 15;
+    }
+    const int32_t key = (cell >= 0 && cell < layout.n_cells && m1 < nA) ? cell * nA + m1 : -2;
+
+    T sum = T(0);
+    for (int32_t base = 0; base < N; base += TABLE_TILE) {
+        __syncthreads();
+        for (int i = tid; i < TABLE_TILE; i += DENSE_THREADS) {
+            const int32_t n = base + i;
+            int32_t entry_key = -1;
+            T coefficient = T(0);
+            if (n < N) {
+                const int32_t e1 = PA[n];
+                const int32_t e2 = PW2[n];
+                const int32_t e3 = PO2[n];
+                if (in_bounds(e1, nA) && in_bounds(e2, n2) && in_bounds(e3, n3)) {
+                    entry_key = (e3 * n2 + e2) * nA + e1;
+                    coefficient = C[n];
+                }
+            }
+            keys[i] = entry_key;
+            coefficients[i] = coefficient;
+        }
+        __syncthreads();
+        // entries beyond N hold key -1 and match nothing
+        const int32_t count = (min(TABLE_TILE, N - base) + 7) & ~7;
+        for (int32_t i0 = 0; i0 < count; i0 += 8) {
+            int32_t entry_key[8];
+            T coefficient[8];
+#pragma unroll
+            for (int u = 0; u < 8; u++) {
+                entry_key[u] = keys[i0 + u];
+                coefficient[u] = coefficients[i0 + u];
+            }
+#pragma unroll
+            for (int u = 0; u < 8; u++) {
+                sum += entry_key[u] == key ? coefficient[u] : T(0);
+            }
+        }
+    }
+    if (slot < n_to_cells) {
+        to_cells[slot] = sum;
+    } else if (slot < n_slots) {
+        to_A[slot - n_to_cells] = sum;
+    }
+}
+
+// ---------------------------------------------------------------------------
+// pieces shared by the kernels
+
+/// T[cell, k] = sum_m1 D[cell, m1] * A[edge_k, m1] for the (up to) 16 edges
+/// held by lanes 0..15 in `my_edge` (-1: no edge, its column is zero),
+/// written to t_area[cell * T_ROW + k] for every cell of the padded tiles.
+template <typename T>
+__device__ __forceinline__ void coupling_times_A(
+    T* __restrict__ t_area,
+    const T* __restrict__ A,
+    const T* __restrict__ to_cells,
+    int32_t my_edge,
+    int lane,
+    int32_t nA,
+    int32_t n_cell_tiles
+) {
+    using M = Mfma<T>;
+    const int k = lane & 15;
+    const int q = lane >> 4;
+    T a_rows[MAX_A_STEPS];
+#pragma unroll
+    for (int s = 0; s < MAX_A_STEPS; s++) {
+        const int32_t m1 = 4 * s + q;
+        a_rows[s] = load_or_zero(A, static_cast<size_t>(my_edge) * nA + m1, my_edge >= 0 && m1 < nA);
+    }
+    T* my_rows = t_area + M::row(lane, 0) * T_ROW + k;
+    const int row_step = (M::row(0, 1) - M::row(0, 0)) * T_ROW;
+    for (int32_t tile0 = 0; tile0 < n_cell_tiles; tile0 += TILE_GROUP) {
+        const T* group = to_cells + tile0 * MAX_A_STEPS * WAVE + lane;
+        T d[TILE_GROUP][MAX_A_STEPS];
+#pragma unroll
+        for (int g = 0; g < TILE_GROUP; g++) {
+#pragma unroll
+            for (int s = 0; s < MAX_A_STEPS; s++) {
+                d[g][s] = group[(g * MAX_A_STEPS + s) * WAVE];
+            }
+        }
+        T* rows = my_rows + tile0 * 16 * T_ROW;
+#pragma unroll
+        for (int g = 0; g < TILE_GROUP; g++) {
+            typename M::Acc acc = M::zero();
+#pragma unroll
+            for (int s = 0; s < MAX_A_STEPS; s++) {
+                acc = M::mma(d[g][s], a_rows[s], acc);
+            }
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                rows[g * 16 * T_ROW + r * row_step] = acc[r];
+            }
+        }
+    }
+}
+
+// out[o, l] += sum over the edges k of a batch and over c of
+//   T[cell(o, c), k] * B[edge_k, l] * rows[source_k, c, l]
+// (forward: o = m3, c = m2, rows = W, source = sender;
+//  grad_W:  o = m2, c = m3, rows = grad_output, source = receiver).
+template <typename T> struct Contraction {
+    const T* A;    // [n_edges][nA]
+    const T* B;    // [n_edges][L]
+    const T* rows; // [n_blocks][n_red][L]
+    const int32_t* gather_index; // block of `rows` of every edge
+    const T* to_cells;
+    DenseLayout layout;
+    int32_t n_blocks, nA, L, n_out, n_red;
+    int32_t out_cell_stride, red_cell_stride; // cell = o * out_cell_stride + c * red_cell_stride
+};
+
+/// What one lane needs to know for the whole kernel.
+template <typename T, int NT, int RS> struct ContractionLane {
+    uint32_t w_offset[RS][NT]; // bytes into a block of `rows`
+    uint32_t a_offset[RS];     // bytes into the T area
+    uint32_t b_offset[NT];     // bytes into a row of B
+
+    __device__ __forceinline__ void setup(const Contraction<T>& p, int lane) {
+        const int i = lane & 15;
+        const int q = lane >> 4;
+#pragma unroll
+        for (int s = 0; s < RS; s++) {
+            const int32_t c = 4 * s + q;
+            const bool red_ok = c < p.n_red;
+            // lanes without a term read zeros from T and some finite value from `rows`
+            const int32_t cell =
+                red_ok && i < p.n_out ? i * p.out_cell_stride + c * p.red_cell_stride : p.layout.zero_cell;
+            a_offset[s] = cell * T_ROW * sizeof(T);
+#pragma unroll
+            for (int t = 0; t < NT; t++) {
+                const int32_t col = min(16 * t + i, p.L - 1);
+                w_offset[s][t] = ((red_ok ? c : 0) * p.L + col) * sizeof(T);
+            }
+        }
+#pragma unroll
+        for (int t = 0; t < NT; t++) {
+            b_offset[t] = min(16 * t + i, p.L - 1) * sizeof(T);
+        }
+    }
+};
+
+/// One batch of n <= 16 edges (lane k, k + 16, ... hold edge k in `my_edge`).
+/// The right operands of the matrix instructions come straight from global
+/// memory, a few edges ahead of their use, multiplied by the edge's B row on
+/// the way; the left operands are the rows of T in LDS.
+template <typename T, int NT, int RS>
+__device__ __forceinline__ void contract_batch(
+    typename Mfma<T>::Acc (&out)[NT], const Contraction<T>& p, const ContractionLane<T, NT, RS>& mine,
+    T* __restrict__ t_area, int32_t my_edge, int32_t n, int lane
+) {
+    using M = Mfma<T>;
+    constexpr int EB = (NT >= 4 || sizeof(T) == 8) ? 2 : 4; // edges loaded together
+    const int32_t my_source = my_edge >= 0 ? p.gather_index[my_edge] : -1;
+    const uint32_t block_elements = static_cast<uint32_t>(p.n_red) * p.L;
+
+    struct Operands {
+        T w[EB][RS][NT];
+        T scale[EB][NT];
+        bool present[EB];
+    };
+    auto load = [&](Operands& to, int32_t k0) {
+#pragma unroll
+        for (int u = 0; u < EB; u++) {
+            const int32_t k = min(k0 + u, n - 1); // always an edge of the batch
+            const int32_t edge = __builtin_amdgcn_readlane(my_edge, k);
+            const int32_t source = __builtin_amdgcn_readlane(my_source, k);
+            to.present[u] = k0 + u < n && in_bounds(source, p.n_blocks);
+            const T* block =
+                p.rows + static_cast<size_t>(to.present[u] ? source : 0) * block_elements;
+            const T* b_row = p.B + static_cast<size_t>(edge) * p.L;
+#pragma unroll
+            for (int s = 0; s < RS; s++) {
+#pragma unroll
+                for (int t = 0; t < NT; t++) {
+                    to.w[u][s][t] = load_at(block, mine.w_offset[s][t]);
+                }
+            }
+#pragma unroll
+            for (int t = 0; t < NT; t++) {
+                to.scale[u][t] = load_at(b_row, mine.b_offset[t]);
+            }
+        }
+    };
+    auto multiply = [&](const Operands& from, int32_t k0) {
+        T a[EB][RS];
+        const uint32_t first_column = k0 * sizeof(T);
+#pragma unroll
+        for (int s = 0; s < RS; s++) {
+            const uint32_t at = mine.a_offset[s] + first_column;
+#pragma unroll
+            for (int u = 0; u < EB; u++) {
+                a[u][s] = load_at(t_area, at + u * static_cast<uint32_t>(sizeof(T)));
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < EB; u++) {
+            if (from.present[u]) {
+#pragma unroll
+                for (int s = 0; s < RS; s++) {
+#pragma unroll
+                    for (int t = 0; t < NT; t++) {
+                        out[t] = M::mma(a[u][s], from.w[u][s][t] * from.scale[u][t], out[t]);
+                    }
+                }
+            }
+        }
+    };
+
+    Operands first;
+    Operands second;
+    load(first, 0); // in flight while T is computed
+    wave_sync();    // earlier reads of the T area are over
+    coupling_times_A<T>(t_area, p.A, p.to_cells, my_edge, lane, p.nA, p.layout.n_cell_tiles);
+    wave_sync();
+    for (int32_t k0 = 0; k0 < n; k0 += 2 * EB) {
+        if (k0 + EB < n) {
+            load(second, k0 + EB);
+        }
+        multiply(first, k0);
+        if (k0 + 2 * EB < n) {
+            load(first, k0 + 2 * EB);
+        }
+        if (k0 + EB < n) {
+            multiply(second, k0 + EB);
+        }
+    }
+}
+
+template <typename T, int NT>
+__device__ __forceinline__ void store_block(
+    T* __restrict__ target, const typename Mfma<T>::Acc (&acc)[NT], int32_t n_out, int32_t L, int lane
+) {
+    using M = Mfma<T>;
+    const int i = lane & 15;
+#pragma unroll
+    for (int t = 0; t < NT; t++) {
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const int32_t row = M::row(lane, r);
+            const int32_t col = 16 * t + i;
+            if (row < n_out && col < L) {
+                target[row * L + col] = acc[t][r];
+            }
+        }
+    }
+}
+
+/// The row of the T area that must hold zeros before the first use.
+template <typename T>
+__device__ __forceinline__ void clear_zero_row(T* __restrict__ t_area, const DenseLayout& layout, int lane) {
+    if (lane < T_ROW) {
+        t_area[layout.zero_cell * T_ROW + lane] = T(0);
+    }
+}
+
+// ---------------------------------------------------------------------------
+// forward pass
+
+/// Wavefronts per workgroup (their T areas share 64 KB of LDS) ...
+template <typename T> constexpr int forward_waves() { return sizeof(T) == 4 ? 4 : 2; }
+/// ... and positions of the sorted index per workgroup, 16 per wavefront.
+template <typename T> constexpr int forward_chunk() { return STAGE * forward_waves<T>(); }
+
+template <typename T, int NT, int RS>
+__global__ __launch_bounds__(forward_waves<T>() * WAVE) void forward_kernel(
+    T* __restrict__ output, const int32_t* __restrict__ receivers, int32_t n_edges, const Contraction<T> p
+) {
+    using M = Mfma<T>;
+    constexpr int FORWARD_WAVES = forward_waves<T>();
+    constexpr int FORWARD_CHUNK = forward_chunk<T>();
+    extern __shared__ __align__(16) char lds_raw[];
+    const int lane = threadIdx.x & (WAVE - 1);
+    const int wave = threadIdx.x >> 6;
+    const int i = lane & 15;
+    T* t_area = reinterpret_cast<T*>(lds_raw) + wave * p.layout.t_elements();
+    // partial sums of the wavefronts: [rank][NT][4][64]
+    T* meeting = reinterpret_cast<T*>(lds_raw) + FORWARD_WAVES * p.layout.t_elements();
+    const size_t row_elements = static_cast<size_t>(p.n_out) * p.L;
+
+    ContractionLane<T, NT, RS> mine;
+    mine.setup(p, lane);
+    clear_zero_row(t_area, p.layout, lane);
+
+    int32_t stages_before = 0; // 16-edge stages dealt out so far, the same in every wavefront
+    walk_owned_segments<FORWARD_CHUNK>(
+        receivers, n_edges, p.n_blocks, blockIdx.x,
+        [&](int32_t node, int32_t first, int32_t last) {
+            const int32_t n_stages = (last - first + STAGE - 1) / STAGE;
+            typename M::Acc acc[NT];
+#pragma unroll
+            for (int t = 0; t < NT; t++) {
+                acc[t] = M::zero();
+            }
+            // stage number `st` goes to wavefront (stages_before + st) % FORWARD_WAVES
+            const int32_t rank = (wave - stages_before) & (FORWARD_WAVES - 1);
+            for (int32_t st = rank; st < n_stages; st += FORWARD_WAVES) {
+                const int32_t s0 = first + st * STAGE;
+                const int32_t n = min(STAGE, last - s0);
+                contract_batch<T, NT, RS>(acc, p, mine, t_area, i < n ? s0 + i : -1, n, lane);
+            }
+            const int32_t participants = min(n_stages, FORWARD_WAVES);
+            if (participants > 1) {
+                if (rank > 0 && rank < participants) {
+#pragma unroll
+                    for (int t = 0; t < NT; t++) {
+#pragma unroll
+                        for (int r = 0; r < 4; r++) {
+                            meeting[((rank * NT + t) * 4 + r) * WAVE + lane] = acc[t][r];
+                        }
+                    }
+                }
+                __syncthreads();
+                if (rank == 0) {
+                    for (int32_t other = 1; other < participants; other++) {
+#pragma unroll
+                        for (int t = 0; t < NT; t++) {
+#pragma unroll
+                            for (int r = 0; r < 4; r++) {
+                                acc[t][r] += meeting[((other * NT + t) * 4 + r) * WAVE + lane];
+                            }
+                        }
+                    }
+                }
+                __syncthreads();
+            }
+            if (rank == 0) {
+                store_block<T, NT>(output + node * row_elements, acc, p.n_out, p.L, lane);
+            }
+            stages_before += n_stages;
+        },
+        [&](int32_t begin, int32_t end) {
+            T* target = output + begin * row_elements;
+            const size_t count = (end - begin) * row_elements;
+            for (size_t at = threadIdx.x; at < count; at += FORWARD_WAVES * WAVE) {
+                target[at] = T(0);
+            }
+        }
+    );
+}
+
+// ---------------------------------------------------------------------------
+// grad_W: one wavefront per sender
+
+/// Wavefronts (= senders) per workgroup.
+template <typename T> constexpr int senders_per_group() { return sizeof(T) == 4 ? 6 : 4; }
+
+template <typename T, int NT, int RS>
+__global__ __launch_bounds__(senders_per_group<T>() * WAVE) void weight_gradient_kernel(
+    T* __restrict__ grad_W, const int32_t* __restrict__ senders, int32_t n_edges, bool aligned_senders,
+    const Contraction<T> p
+) {
+    using M = Mfma<T>;
+    constexpr int SENDERS_PER_GROUP = senders_per_group<T>();
+    using Gather = SenderGather<SENDERS_PER_GROUP>;
+    extern __shared__ __align__(16) char lds_raw[];
+    typename Gather::Storage& gather = *reinterpret_cast<typename Gather::Storage*>(lds_raw);
+    const int lane = threadIdx.x & (WAVE - 1);
+    const int wave = threadIdx.x >> 6;
+    T* t_area = reinterpret_cast<T*>(lds_raw + align16(sizeof(typename Gather::Storage))) +
+                wave * p.layout.t_elements();
+    const int32_t node0 = blockIdx.x * SENDERS_PER_GROUP;
+    const int32_t node = node0 + wave;
+
+    ContractionLane<T, NT, RS> mine;
+    mine.setup(p, lane);
+    clear_zero_row(t_area, p.layout, lane);
+    typename M::Acc acc[NT];
+#pragma unroll
+    for (int t = 0; t < NT; t++) {
+        acc[t] = M::zero();
+    }
+    auto on_stage = [&](int32_t my_edge, int32_t n) {
+        contract_batch<T, NT, RS>(acc, p, mine, t_area, my_edge, n, lane);
+    };
+    if (aligned_senders) {
+        Gather::template run<4>(gather, senders, n_edges, node0, p.n_blocks, on_stage);
+    } else {
+        Gather::template run<1>(gather, senders, n_edges, node0, p.n_blocks, on_stage);
+    }
+    if (node < p.n_blocks) {
+        store_block<T, NT>(grad_W + static_cast<size_t>(node) * p.n_out * p.L, acc, p.n_out, p.L, lane);
+    }
+}
+
+// ---------------------------------------------------------------------------
+// grad_A and grad_B: one wavefront per 16 consecutive edges
+
+template <typename T> struct EdgeGradArgs {
+    T* grad_A; // may be null
+    T* grad_B; // may be null
+    const T* G; // grad_output [n_nodes][n3][L]
+    const T* A;
+    const T* B;
+    const T* W;
+    const int32_t* receivers;
+    const int32_t* senders;
+    const T* to_cells;
+    const T* to_A;
+    DenseLayout layout;
+    int32_t n_edges, n_nodes, nA, L, n2, n3;
+    int32_t Ls;        // LDS stride of one row of W and of B
+    bool vector_loads; // W may be read 128 bits at a time
+    FastDivisor by_items, by_lvec, by_L; // n2 * L / vec, L / vec, L
+};
+
+constexpr int EDGE_BATCH = 4; // edges whose W blocks are in LDS together
+
+template <typename T, int NT, int M2S>
+__global__ __launch_bounds__(WAVE) void edge_gradients_kernel(const EdgeGradArgs<T> p) {
+    using M = Mfma<T>;
+    constexpr int L_STEPS = 4 * NT;
+    constexpr uint32_t ELEMENT = sizeof(T);
+    extern __shared__ __align__(16) char lds_raw[];
+    T* t_area = reinterpret_cast<T*>(lds_raw);   // T, then U, of the 16 edges
+    T* w_lds = t_area + p.layout.t_elements();   // [EDGE_BATCH][n2][Ls]
+    T* b_lds = w_lds + EDGE_BATCH * p.n2 * p.Ls; // [EDGE_BATCH][Ls]
+    T* partial_lds = b_lds + EDGE_BATCH * p.Ls;  // [EDGE_BATCH][NT][64]
+    const int32_t lds_elements = p.layout.t_elements() + EDGE_BATCH * (p.n2 + 1) * p.Ls;
+
+    const int lane = threadIdx.x;
+    const int i = lane & 15;
+    const int q = lane >> 4;
+    const bool want_A = p.grad_A != nullptr;
+    const bool want_B = p.grad_B != nullptr;
+
+    const int32_t chunk_begin = blockIdx.x * STAGE;
+    const int32_t n = min(STAGE, p.n_edges - chunk_begin);
+    const int32_t my_edge = i < n ? chunk_begin + i : -1;
+    const int32_t my_source = my_edge >= 0 ? p.senders[my_edge] : -1;
+    const int32_t my_node = my_edge >= 0 ? p.receivers[my_edge] : -1;
+
+    // padding of the LDS arrays is read (and multiplied by zeros): make it finite
+    for (int32_t at = lane; at < lds_elements; at += WAVE) {
+        t_area[at] = T(0);
+    }
+
+    // ---- what depends on the lane only
+    // left operand rows of T for P = T_e * W_e: lane (m3 = i, m2 = 4 s + q)
+    uint32_t t_offset[M2S];
+    // right operand W_e[m2 = 4 s + q][l = 16 t + i], t as immediate
+    uint32_t w_by_column[EDGE_BATCH][M2S];
+#pragma unroll
+    for (int s = 0; s < M2S; s++) {
+        const int32_t m2 = 4 * s + q;
+        const bool ok = m2 < p.n2;
+        t_offset[s] = (ok && i < p.n3 ? i * p.n2 + m2 : p.layout.zero_cell) * T_ROW * ELEMENT;
+#pragma unroll
+        for (int kw = 0; kw < EDGE_BATCH; kw++) {
+            w_by_column[kw][s] = ((kw * p.n2 + (ok ? m2 : 0)) * p.Ls + i) * ELEMENT;
+        }
+    }
+    // right operand of U = G * Z^T: lane (m2 = i, l = 4 s + q), s as immediate
+    uint32_t w_by_row[EDGE_BATCH];
+    uint32_t b_by_row[EDGE_BATCH];
+#pragma unroll
+    for (int kw = 0; kw < EDGE_BATCH; kw++) {
+        w_by_row[kw] = ((kw * p.n2 + (i < p.n2 ? i : 0)) * p.Ls + q) * ELEMENT;
+        b_by_row[kw] = (kw * p.Ls + q) * ELEMENT;
+    }
+    // where this lane's elements of U go: U[m3 = D row][m2 = i] of edge k
+    uint32_t u_offset[4];
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+        const int32_t m3 = M::row(lane, r);
+        u_offset[r] = (m3 < p.n3 && i < p.n2 ? m3 * p.n2 + i : p.layout.dump_cell) * T_ROW * ELEMENT;
+    }
+    // left operand of grad_A = U * D: lane (edge = i, cell = 4 step + q), step as immediate
+    const uint32_t u_by_edge = (q * T_ROW + i) * ELEMENT;
+
+    __syncthreads();
+    if (want_B) {
+        coupling_times_A<T>(t_area, p.A, p.to_cells, my_edge, lane, p.nA, p.layout.n_cell_tiles);
+    }
+
+    // G of the receiver of the current edge, as operands
+    int32_t current_node = -1;
+    T g_rows[NT][4];   // G[m3 = D row of this lane][l = column of this lane]
+    T g_left[L_STEPS]; // lane (m3 = i, l = 4 s + q)
+#pragma unroll
+    for (int t = 0; t < NT; t++) {
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            g_rows[t][r] = T(0);
+        }
+    }
+#pragma unroll
+    for (int s = 0; s < L_STEPS; s++) {
+        g_left[s] = T(0);
+    }
+
+    const uint32_t items_per_edge = p.by_items.divisor;
+    const uint32_t lvecs = p.by_lvec.divisor;
+    const int32_t block_elements = p.n2 * p.L;
+
+    for (int32_t k0 = 0; k0 < n; k0 += EDGE_BATCH) {
+        const int32_t n_batch = min(EDGE_BATCH, n - k0);
+        __syncthreads(); // the previous batch is no longer read
+        // ---- W blocks and B rows of the batch into LDS
+        if (p.vector_loads) {
+            typedef T Vec __attribute__((ext_vector_type(4)));
+            constexpr int ROUND = 5;
+            const uint32_t total = static_cast<uint32_t>(n_batch) * items_per_edge;
+            for (uint32_t base = 0; base < total; base += ROUND * WAVE) {
+                Vec loaded[ROUND];
+                uint32_t where[ROUND];
+                bool ok[ROUND];
+#pragma unroll
+                for (int u = 0; u < ROUND; u++) {
+                    const uint32_t item = base + u * WAVE + lane;
+                    ok[u] = item < total;
+                    const uint32_t safe = ok[u] ? item : 0;
+                    const uint32_t kw = p.by_items.divide(safe);
+                    const uint32_t rest = safe - kw * items_per_edge;
+                    const uint32_t row = p.by_lvec.divide(rest);
+                    const uint32_t lv = rest - row * lvecs;
+                    const int32_t source = __shfl(my_source, k0 + static_cast<int>(kw));
+                    const bool valid = ok[u] && in_bounds(source, p.n_nodes);
+                    const size_t from = valid ? static_cast<size_t>(source) * block_elements + rest * 4 : 0;
+                    const Vec value = *reinterpret_cast<const Vec*>(p.W + from);
+                    loaded[u] = valid ? value : Vec(T(0));
+                    where[u] = (kw * p.n2 + row) * p.Ls + lv * 4;
+                }
+#pragma unroll
+                for (int u = 0; u < ROUND; u++) {
+                    if (ok[u]) {
+#pragma unroll
+                        for (int v = 0; v < 4; v++) {
+                            w_lds[where[u] + v] = loaded[u][v];
+                        }
+                    }
+                }
+            }
+        } else {
+            const uint32_t total = static_cast<uint32_t>(n_batch) * items_per_edge;
+            // all lanes stay in the loop: the shuffle reads lanes that would
+            // otherwise have left it
+            for (uint32_t base = 0; base < total; base += WAVE) {
+                const uint32_t item = base + lane;
+                const bool ok = item < total;
+                const uint32_t safe = ok ? item : 0;
+                const uint32_t kw = p.by_items.divide(safe);
+                const uint32_t rest = safe - kw * items_per_edge;
+                const uint32_t row = p.by_lvec.divide(rest);
+                const uint32_t l = rest - row * lvecs;
+                const int32_t source = __shfl(my_source, k0 + static_cast<int>(kw));
+                const bool valid = ok && in_bounds(source, p.n_nodes);
+                const T value =
+                    load_or_zero(p.W, static_cast<size_t>(source) * block_elements + rest, valid);
+                if (ok) {
+                    w_lds[(kw * p.n2 + row) * p.Ls + l] = value;
+                }
+            }
+        }
+        {
+            const T* from = p.B + static_cast<size_t>(chunk_begin + k0) * p.L;
+            const uint32_t count = static_cast<uint32_t>(n_batch) * p.L;
+            for (uint32_t at = lane; at < count; at += WAVE) {
+                const uint32_t kw = p.by_L.divide(at);
+                b_lds[kw * p.Ls + (at - kw * p.L)] = from[at];
+            }
+        }
+        __syncthreads();
+
+        const uint32_t first_column = k0 * ELEMENT;
+#pragma unroll
+        for (int kw = 0; kw < EDGE_BATCH; kw++) {
+            if (kw >= n_batch) {
+                continue;
+            }
+            const int32_t node = __builtin_amdgcn_readlane(my_node, min(k0 + kw, STAGE - 1));
+            if (node != current_node) {
+                current_node = node;
+                const bool valid = in_bounds(node, p.n_nodes);
+                const T* g_block = p.G + static_cast<size_t>(valid ? node : 0) * p.n3 * p.L;
+#pragma unroll
+                for (int t = 0; t < NT; t++) {
+#pragma unroll
+                    for (int r = 0; r < 4; r++) {
+                        const int32_t m3 = M::row(lane, r);
+                        const int32_t col = 16 * t + i;
+                        g_rows[t][r] = load_or_zero(g_block, m3 * p.L + col, valid && m3 < p.n3 && col < p.L);
+                    }
+                }
+#pragma unroll
+                for (int s = 0; s < L_STEPS; s++) {
+                    const int32_t l = 4 * s + q;
+                    g_left[s] = load_or_zero(g_block, i * p.L + l, valid && i < p.n3 && l < p.L);
+                }
+            }
+            const uint32_t column = first_column + kw * ELEMENT;
+            if (want_B) {
+                // P[m3, l] = sum_m2 T[(m3, m2), k] * W[m2, l]; grad_B[l] = sum_m3 G[m3, l] P[m3, l]
+                typename M::Acc product[NT];
+#pragma unroll
+                for (int t = 0; t < NT; t++) {
+                    product[t] = M::zero();
+                }
+#pragma unroll
+                for (int s = 0; s < M2S; s++) {
+                    const T left = load_at(t_area, t_offset[s] + column);
+#pragma unroll
+                    for (int t = 0; t < NT; t++) {
+                        const T right = load_at(w_lds, w_by_column[kw][s] + t * 16 * ELEMENT);
+                        product[t] = M::mma(left, right, product[t]);
+                    }
+                }
+#pragma unroll
+                for (int t = 0; t < NT; t++) {
+                    T partial = T(0);
+#pragma unroll
+                    for (int r = 0; r < 4; r++) {
+                        partial += product[t][r] * g_rows[t][r];
+                    }
+                    partial_lds[(kw * NT + t) * WAVE + lane] = partial;
+                }
+            }
+            if (want_A) {
+                // U[m3, m2] = sum_l G[m3, l] * B[k, l] * W[m2, l]
+                typename M::Acc even = M::zero();
+                typename M::Acc odd = M::zero();
+#pragma unroll
+                for (int s = 0; s < L_STEPS; s += 2) {
+                    const T z0 = load_at(w_lds, w_by_row[kw] + s * 4 * ELEMENT) *
+                                 load_at(b_lds, b_by_row[kw] + s * 4 * ELEMENT);
+                    const T z1 = load_at(w_lds, w_by_row[kw] + (s + 1) * 4 * ELEMENT) *
+                                 load_at(b_lds, b_by_row[kw] + (s + 1) * 4 * ELEMENT);
+                    even = M::mma(g_left[s], z0, even);
+                    odd = M::mma(g_left[s + 1], z1, odd);
+                }
+                // T of this edge is no longer needed: its column takes U
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    store_at(t_area, u_offset[r] + column, even[r] + odd[r]);
+                }
+            }
+        }
+        if (want_B) {
+            __syncthreads();
+            // the four quarters of the wavefront finish one edge each
+#pragma unroll
+            for (int t = 0; t < NT; t++) {
+                T sum = T(0);
+#pragma unroll
+                for (int g = 0; g < 4; g++) {
+                    sum += partial_lds[(q * NT + t) * WAVE + g * 16 + i];
+                }
+                const int32_t col = 16 * t + i;
+                if (q < n_batch && col < p.L) {
+                    p.grad_B[static_cast<size_t>(chunk_begin + k0 + q) * p.L + col] = sum;
+                }
+            }
+        }
+    }
+
+    if (want_A) {
+        __syncthreads();
+        // grad_A[k, m1] = sum_cell U[k, cell] * D[cell, m1]
+        typename M::Acc even = M::zero();
+        typename M::Acc odd = M::zero();
+        const T* table = p.to_A + lane;
+        for (int32_t step0 = 0; step0 < p.layout.cell_steps; step0 += STEP_GROUP) {
+            T left[STEP_GROUP];
+            T right[STEP_GROUP];
+            const uint32_t at = u_by_edge + step0 * 4 * T_ROW * ELEMENT;
+#pragma unroll
+            for (int u = 0; u < STEP_GROUP; u++) {
+                left[u] = load_at(t_area, at + u * 4 * T_ROW * ELEMENT);
+                right[u] = table[(step0 + u) * WAVE];
+            }
+#pragma unroll
+            for (int u = 0; u < STEP_GROUP; u += 2) {
+                even = M::mma(left[u], right[u], even);
+                odd = M::mma(left[u + 1], right[u + 1], odd);
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const int32_t k = M::row(lane, r);
+            if (k < n && i < p.nA) {
+                p.grad_A[static_cast<size_t>(chunk_begin + k) * p.nA + i] = even[r] + odd[r];
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// host side
+
+template <typename T> struct DenseBuffers {
+    T* to_cells;
+    T* to_A;
+};
+
+size_t dense_bytes(const DenseLayout& layout, size_t element_size) {
+    return align256(static_cast<size_t>(layout.to_cells_slots()) * element_size) +
+           align256(static_cast<size_t>(layout.to_A_slots()) * element_size);
+}
+
+template <typename T>
+DenseBuffers<T> enqueue_dense(
+    void* workspace, const DenseLayout& layout, const T* C, const Indices& indices, const Shape& s,
+    hipStream_t stream
+) {
+    DenseBuffers<T> buffers;
+    char* base = static_cast<char*>(workspace);
+    buffers.to_cells = reinterpret_cast<T*>(base);
+    buffers.to_A = reinterpret_cast<T*>(base + align256(static_cast<size_t>(layout.to_cells_slots()) * sizeof(T)));
+    const int32_t slots = layout.to_cells_slots() + layout.to_A_slots();
+    dense_coupling_kernel<T><<<(slots + DENSE_THREADS - 1) / DENSE_THREADS, DENSE_THREADS, 0, stream>>>(
+        buffers.to_cells, buffers.to_A, C, indices.A, indices.W_2, indices.output_2, s.N, s.nA, s.n2, s.n3,
+        layout
+    );
+    MOPS_HIP_CHECK(hipGetLastError());
+    return buffers;
+}
+
+int tiles_for(int32_t L) { return L <= 32 ? 2 : 4; }
+
+size_t t_area_bytes(const Shape& s, size_t element_size) {
+    return static_cast<size_t>(dense_layout(s).t_elements()) * element_size;
+}
+
+size_t forward_lds(const Shape& s, size_t element_size) {
+    const size_t waves = element_size == 4 ? forward_waves<float>() : forward_waves<double>();
+    return waves * t_area_bytes(s, element_size) + waves * tiles_for(s.L) * 4 * WAVE * element_size;
+}
+
+size_t weight_gradient_lds(const Shape& s, size_t element_size) {
+    return element_size == 4
+               ? align16(sizeof(SenderGather<senders_per_group<float>()>::Storage)) +
+                     senders_per_group<float>() * t_area_bytes(s, element_size)
+               : align16(sizeof(SenderGather<senders_per_group<double>()>::Storage)) +
+                     senders_per_group<double>() * t_area_bytes(s, element_size);
+}
+
+/// Rows of W in LDS: at least the 16 * NT columns the operands touch, and two
+/// more so that lanes walking down a column of 4-byte elements spread over
+/// the banks.
+int32_t weight_row_stride(const Shape& s) { return 16 * tiles_for(s.L) + 2; }
+
+size_t edge_gradients_lds(const Shape& s, size_t element_size) {
+    return t_area_bytes(s, element_size) +
+           (static_cast<size_t>(EDGE_BATCH) * (s.n2 + 1) * weight_row_stride(s) +
+            static_cast<size_t>(EDGE_BATCH) * tiles_for(s.L) * WAVE) *
+               element_size;
+}
+
+bool aligned_for_vectors(const void* pointer, size_t element_size) {
+    return reinterpret_cast<uintptr_t>(pointer) % (4 * element_size) == 0;
+}
+
+template <typename T>
+Contraction<T> contraction(
+    const T* A, const T* B, const T* rows, const int32_t* gather_index, const T* to_cells,
+    const DenseLayout& layout, const Shape& s, int32_t n_out, int32_t n_red, int32_t out_cell_stride,
+    int32_t red_cell_stride
+) {
+    Contraction<T> c{};
+    c.A = A;
+    c.B = B;
+    c.rows = rows;
+    c.gather_index = gather_index;
+    c.to_cells = to_cells;
+    c.layout = layout;
+    c.n_blocks = s.n_nodes;
+    c.nA = s.nA;
+    c.L = s.L;
+    c.n_out = n_out;
+    c.n_red = n_red;
+    c.out_cell_stride = out_cell_stride;
+    c.red_cell_stride = red_cell_stride;
+    return c;
+}
+
+/// Calls `launch(tiles, steps)` with the two shape parameters the kernels are
+/// compiled for as integral constants.
+template <typename Launch> void with_shape_constants(int tiles, int steps, Launch&& launch) {
+    auto with_steps = [&](auto tiles_constant) {
+        switch (steps) {
+        case 1:
+            launch(tiles_constant, std::integral_constant<int, 1>{});
+            break;
+        case 2:
+            launch(tiles_constant, std::integral_constant<int, 2>{});
+            break;
+        case 3:
+            launch(tiles_constant, std::integral_constant<int, 3>{});
+            break;
+        default:
+            launch(tiles_constant, std::integral_constant<int, 4>{});
+            break;
+        }
+    };
+    if (tiles == 2) {
+        with_steps(std::integral_constant<int, 2>{});
+    } else {
+        with_steps(std::integral_constant<int, 4>{});
+    }
+}
+
+} // namespace
+
+bool supports(const Shape& s, size_t element_size) {
+    if (s.n_nodes < 1 || s.n_edges < 1 || s.N < 1) {
+        return false;
+    }
+    if (s.nA < 1 || s.nA > 4 * MAX_A_STEPS || s.n2 < 1 || s.n2 > MAX_INDEX || s.n3 < 1 ||
+        s.n3 > MAX_INDEX || s.L < 1 || s.L > MAX_L) {
+        return false;
+    }
+    return forward_lds(s, element_size) <= LDS_BUDGET && weight_gradient_lds(s, element_size) <= LDS_BUDGET &&
+           edge_gradients_lds(s, element_size) <= LDS_BUDGET;
+}
+
+size_t workspace_bytes(const Shape& s, size_t element_size) {
+    return dense_bytes(dense_layout(s), element_size);
+}
+
+template <typename T>
+void forward(
+    T* output, const T* A, const T* B, const T* C, const T* W, const Indices& indices,
+    const Shape& s, void* workspace, hipStream_t stream
+) {
+    const DenseLayout layout = dense_layout(s);
+    const DenseBuffers<T> dense = enqueue_dense<T>(workspace, layout, C, indices, s, stream);
+    const Contraction<T> c =
+        contraction<T>(A, B, W, indices.W_1, dense.to_cells, layout, s, s.n3, s.n2, s.n2, 1);
+    const int32_t grid = (s.n_edges + forward_chunk<T>() - 1) / forward_chunk<T>();
+    const size_t lds = forward_lds(s, sizeof(T));
+    with_shape_constants(tiles_for(s.L), (s.n2 + 3) / 4, [&](auto tiles, auto steps) {
+        forward_kernel<T, decltype(tiles)::value, decltype(steps)::value>
+            <<<grid, forward_waves<T>() * WAVE, lds, stream>>>(output, indices.output_1, s.n_edges, c);
+    });
+    MOPS_HIP_CHECK(hipGetLastError());
+}
+
+template <typename T>
+void vjp(
+    T* grad_A, T* grad_B, T* grad_W, const T* grad_output, const T* A, const T* B, const T* C,
+    const T* W, const Indices& indices, const Shape& s, void* workspace, hipStream_t stream
+) {
+    const DenseLayout layout = dense_layout(s);
+    const DenseBuffers<T> dense = enqueue_dense<T>(workspace, layout, C, indices, s, stream);
+    const int tiles = tiles_for(s.L);
+
+    if (grad_A != nullptr || grad_B != nullptr) {
+        const bool vectors = s.L % 4 == 0 && aligned_for_vectors(W, sizeof(T));
+        const int vec = vectors ? 4 : 1;
+        EdgeGradArgs<T> args{};
+        args.grad_A = grad_A;
+        args.grad_B = grad_B;
+        args.G = grad_output;
+        args.A = A;
+        args.B = B;
+        args.W = W;
+        args.receivers = indices.output_1;
+        args.senders = indices.W_1;
+        args.to_cells = dense.to_cells;
+        args.to_A = dense.to_A;
+        args.layout = layout;
+        args.n_edges = s.n_edges;
+        args.n_nodes = s.n_nodes;
+        args.nA = s.nA;
+        args.L = s.L;
+        args.n2 = s.n2;
+        args.n3 = s.n3;
+        args.Ls = weight_row_stride(s);
+        args.vector_loads = vectors;
+        args.by_items = FastDivisor::make(s.n2 * s.L / vec);
+        args.by_lvec = FastDivisor::make(s.L / vec);
+        args.by_L = FastDivisor::make(s.L);
+        const int32_t grid = (s.n_edges + STAGE - 1) / STAGE;
+        const size_t lds = edge_gradients_lds(s, sizeof(T));
+        with_shape_constants(tiles, (s.n2 + 3) / 4, [&](auto tiles_constant, auto steps) {
+            edge_gradients_kernel<T, decltype(tiles_constant)::value, decltype(steps)::value>
+                <<<grid, WAVE, lds, stream>>>(args);
+        });
+        MOPS_HIP_CHECK(hipGetLastError());
+    }
+
+    if (grad_W != nullptr) {
+        const Contraction<T> c = contraction<T>(
+            A, B, grad_output, indices.output_1, dense.to_cells, layout, s, s.n2, s.n3, 1, s.n2
+        );
+        constexpr int SENDERS_PER_GROUP = senders_per_group<T>();
+        const int32_t grid = (s.n_nodes + SENDERS_PER_GROUP - 1) / SENDERS_PER_GROUP;
+        const size_t lds = weight_gradient_lds(s, sizeof(T));
+        const bool aligned = aligned_for_vectors(indices.W_1, sizeof(int32_t));
+        with_shape_constants(tiles, (s.n3 + 3) / 4, [&](auto tiles_constant, auto steps) {
+            weight_gradient_kernel<T, decltype(tiles_constant)::value, decltype(steps)::value>
+                <<<grid, SENDERS_PER_GROUP * WAVE, lds, stream>>>(grad_W, indices.W_1, s.n_edges, aligned, c);
+        });
+        MOPS_HIP_CHECK(hipGetLastError());
+    }
+}
+
+template void forward<float>(
+    float*, const float*, const float*, const float*, const float*, const Indices&, const Shape&, void*,
+    hipStream_t
+);
+template void forward<double>(
+    double*, const double*, const double*, const double*, const double*, const Indices&, const Shape&,
+    void*, hipStream_t
+);
+template void vjp<float>(
+    float*, float*, float*, const float*, const float*, const float*, const float*, const float*,
+    const Indices&, const Shape&, void*, hipStream_t
+);
+template void vjp<double>(
+    double*, double*, double*, const double*, const double*, const double*, const double*, const double*,
+    const Indices&, const Shape&, void*, hipStream_t
+);
+
+} // namespace mops::amd::sasaw_mfma
