@@ -192,28 +192,33 @@ __global__ __launch_bounds__(DENSE_THREADS) void dense_coupling_kernel(
 // ---------------------------------------------------------------------------
 // pieces shared by the kernels
 
-/// T[cell, k] = sum_m1 D[cell, m1] * A[edge_k, m1] for the (up to) 16 edges
-/// held by lanes 0..15 in `my_edge` (-1: no edge, its column is zero),
-/// written to t_area[cell * T_ROW + k] for every cell of the padded tiles.
+/// Row of A of the edge held by this lane's column (lane & 15), as right
+/// operand of T = D * A^T; zeros without an edge (`my_edge` -1).
 template <typename T>
-__device__ __forceinline__ void coupling_times_A(
-    T* __restrict__ t_area,
-    const T* __restrict__ A,
-    const T* __restrict__ to_cells,
-    int32_t my_edge,
-    int lane,
-    int32_t nA,
-    int32_t n_cell_tiles
+__device__ __forceinline__ void load_A_rows(
+    T (&a_rows)[MAX_A_STEPS], const T* __restrict__ A, int32_t my_edge, int lane, int32_t nA
 ) {
-    using M = Mfma<T>;
-    const int k = lane & 15;
     const int q = lane >> 4;
-    T a_rows[MAX_A_STEPS];
 #pragma unroll
     for (int s = 0; s < MAX_A_STEPS; s++) {
         const int32_t m1 = 4 * s + q;
         a_rows[s] = load_or_zero(A, static_cast<size_t>(my_edge) * nA + m1, my_edge >= 0 && m1 < nA);
     }
+}
+
+/// T[cell, k] = sum_m1 D[cell, m1] * A[edge_k, m1] for the (up to) 16 edges
+/// whose rows of A are in `a_rows`, written to t_area[cell * T_ROW + k] for
+/// every cell of the padded tiles.
+template <typename T>
+__device__ __forceinline__ void coupling_times_A(
+    T* __restrict__ t_area,
+    const T (&a_rows)[MAX_A_STEPS],
+    const T* __restrict__ to_cells,
+    int lane,
+    int32_t n_cell_tiles
+) {
+    using M = Mfma<T>;
+    const int k = lane & 15;
     T* my_rows = t_area + M::row(lane, 0) * T_ROW + k;
     const int row_step = (M::row(0, 1) - M::row(0, 0)) * T_ROW;
     for (int32_t tile0 = 0; tile0 < n_cell_tiles; tile0 += TILE_GROUP) {
@@ -255,6 +260,7 @@ template <typename T> struct Contraction {
     DenseLayout layout;
     int32_t n_blocks, nA, L, n_out, n_red;
     int32_t out_cell_stride, red_cell_stride; // cell = o * out_cell_stride + c * red_cell_stride
+    bool vector_rows; // NT neighbouring elements of `rows` and of B may be loaded at once
 };
 
 /// What one lane needs to know for the whole kernel.
@@ -276,118 +282,165 @@ template <typename T, int NT, int RS> struct ContractionLane {
             a_offset[s] = cell * T_ROW * sizeof(T);
 #pragma unroll
             for (int t = 0; t < NT; t++) {
-                const int32_t col = min(16 * t + i, p.L - 1);
-                w_offset[s][t] = ((red_ok ? c : 0) * p.L + col) * sizeof(T);
+                w_offset[s][t] = ((red_ok ? c : 0) * p.L + column(p, i, t)) * sizeof(T);
             }
         }
 #pragma unroll
         for (int t = 0; t < NT; t++) {
-            b_offset[t] = min(16 * t + i, p.L - 1) * sizeof(T);
+            b_offset[t] = column(p, i, t) * sizeof(T);
         }
+    }
+
+    /// Column l of the feature dimension that column i of matrix tile t stands
+    /// for: l = NT * i + t, so that one lane's NT columns are neighbours in
+    /// memory. Columns beyond L are redirected to existing ones (and never
+    /// stored).
+    static __device__ __forceinline__ int32_t column(const Contraction<T>& p, int i, int t) {
+        if (p.vector_rows) {
+            return min(NT * i, p.L - NT) + t;
+        }
+        return min(NT * i + t, p.L - 1);
     }
 };
 
-/// One batch of n <= 16 edges (lane k, k + 16, ... hold edge k in `my_edge`).
-/// The right operands of the matrix instructions come straight from global
-/// memory, a few edges ahead of their use, multiplied by the edge's B row on
-/// the way; the left operands are the rows of T in LDS.
-template <typename T, int NT, int RS>
-__device__ __forceinline__ void contract_batch(
-    typename Mfma<T>::Acc (&out)[NT], const Contraction<T>& p, const ContractionLane<T, NT, RS>& mine,
-    T* __restrict__ t_area, int32_t my_edge, int32_t n, int lane
-) {
-    using M = Mfma<T>;
-    constexpr int EB = (NT >= 4 || sizeof(T) == 8) ? 2 : 4; // edges loaded together
-    const int32_t my_source = my_edge >= 0 ? p.gather_index[my_edge] : -1;
-    const uint32_t block_elements = static_cast<uint32_t>(p.n_red) * p.L;
+/// Two independent sets of accumulators, used in turn: consecutive matrix
+/// instructions on one accumulator wait for each other.
+template <typename T, int NT> struct Accumulators {
+    typename Mfma<T>::Acc part[2][NT];
 
-    struct Operands {
-        T w[EB][RS][NT];
-        T scale[EB][NT];
-        bool present[EB];
-    };
-    auto load = [&](Operands& to, int32_t k0) {
+    __device__ __forceinline__ void clear() {
 #pragma unroll
-        for (int u = 0; u < EB; u++) {
-            const int32_t k = min(k0 + u, n - 1); // always an edge of the batch
-            const int32_t edge = __builtin_amdgcn_readlane(my_edge, k);
-            const int32_t source = __builtin_amdgcn_readlane(my_source, k);
-            to.present[u] = k0 + u < n && in_bounds(source, p.n_blocks);
-            const T* block =
-                p.rows + static_cast<size_t>(to.present[u] ? source : 0) * block_elements;
-            const T* b_row = p.B + static_cast<size_t>(edge) * p.L;
-#pragma unroll
-            for (int s = 0; s < RS; s++) {
-#pragma unroll
-                for (int t = 0; t < NT; t++) {
-                    to.w[u][s][t] = load_at(block, mine.w_offset[s][t]);
-                }
-            }
+        for (int h = 0; h < 2; h++) {
 #pragma unroll
             for (int t = 0; t < NT; t++) {
+                part[h][t] = Mfma<T>::zero();
+            }
+        }
+    }
+    __device__ __forceinline__ T total(int t, int r) const { return part[0][t][r] + part[1][t][r]; }
+};
+
+/// One batch of n <= 16 edges (lane k, k + 16, ... hold edge k in `my_edge`
+/// and its block of `rows` in `my_source`; both -1 beyond n).
+/// The right operands of the matrix instructions come straight from global
+/// memory, all edges of the batch in flight together, multiplied by the
+/// edge's B row on the way; the left operands are the rows of T in LDS.
+template <typename T, int NT, int RS>
+__device__ __forceinline__ void contract_batch(
+    Accumulators<T, NT>& out, const Contraction<T>& p, const ContractionLane<T, NT, RS>& mine,
+    T* __restrict__ t_area, int32_t my_edge, int32_t my_source, int32_t n, int lane
+) {
+    using M = Mfma<T>;
+    typedef T Vec __attribute__((ext_vector_type(NT)));
+    // Edges whose operands are in flight together: a round trip to memory
+    // costs about as much as the arithmetic of all 16 edges, so as many as
+    // the registers hold (RS * NT + NT values per edge).
+    constexpr int EB = (sizeof(T) == 8 ? 4 : 8) / (NT >= 4 ? 2 : 1);
+    const uint32_t block_elements = static_cast<uint32_t>(p.n_red) * p.L;
+    // Nothing below is conditional: lanes 0..15 without an edge (or with a
+    // source out of range) get a zero column of T, and their operand loads are
+    // redirected to an edge that exists, so their products vanish.
+    const bool usable = my_edge >= 0 && in_bounds(my_source, p.n_blocks);
+    const int32_t edge_or_none = usable ? my_edge : -1;
+    const int32_t fallback_edge = __builtin_amdgcn_readfirstlane(my_edge);
+    const int32_t load_edge = usable ? my_edge : fallback_edge;
+    const int32_t load_source = usable ? my_source : 0;
+
+    struct Operands {
+        Vec w[EB][RS];
+        Vec scale[EB];
+    };
+    auto load_one = [&](Operands& to, int32_t k0, int u, auto vectors) {
+        const int32_t k = min(k0 + u, STAGE - 1);
+        const int32_t edge = __builtin_amdgcn_readlane(load_edge, k);
+        const int32_t source = __builtin_amdgcn_readlane(load_source, k);
+        const T* block = p.rows + static_cast<size_t>(source) * block_elements;
+        const T* b_row = p.B + static_cast<size_t>(edge) * p.L;
+        if constexpr (decltype(vectors)::value) {
+#pragma unroll
+            for (int s = 0; s < RS; s++) {
+                to.w[u][s] =
+                    *reinterpret_cast<const Vec*>(reinterpret_cast<const char*>(block) + mine.w_offset[s][0]);
+            }
+            to.scale[u] =
+                *reinterpret_cast<const Vec*>(reinterpret_cast<const char*>(b_row) + mine.b_offset[0]);
+        } else {
+#pragma unroll
+            for (int t = 0; t < NT; t++) {
+#pragma unroll
+                for (int s = 0; s < RS; s++) {
+                    to.w[u][s][t] = load_at(block, mine.w_offset[s][t]);
+                }
                 to.scale[u][t] = load_at(b_row, mine.b_offset[t]);
             }
         }
     };
-    auto multiply = [&](const Operands& from, int32_t k0) {
-        T a[EB][RS];
-        const uint32_t first_column = k0 * sizeof(T);
-#pragma unroll
-        for (int s = 0; s < RS; s++) {
-            const uint32_t at = mine.a_offset[s] + first_column;
+    auto load = [&](Operands& to, int32_t k0) {
+        if (p.vector_rows) {
 #pragma unroll
             for (int u = 0; u < EB; u++) {
-                a[u][s] = load_at(t_area, at + u * static_cast<uint32_t>(sizeof(T)));
+                load_one(to, k0, u, std::true_type{});
             }
+        } else {
+#pragma unroll
+            for (int u = 0; u < EB; u++) {
+                load_one(to, k0, u, std::false_type{});
+            }
+        }
+    };
+    auto multiply = [&](const Operands& from, int32_t k0) {
+        uint32_t a_base[RS];
+#pragma unroll
+        for (int s = 0; s < RS; s++) {
+            a_base[s] = mine.a_offset[s] + k0 * static_cast<uint32_t>(sizeof(T));
         }
 #pragma unroll
         for (int u = 0; u < EB; u++) {
-            if (from.present[u]) {
+            T a[RS];
 #pragma unroll
-                for (int s = 0; s < RS; s++) {
+            for (int s = 0; s < RS; s++) {
+                a[s] = load_at(t_area, a_base[s] + u * static_cast<uint32_t>(sizeof(T)));
+            }
 #pragma unroll
-                    for (int t = 0; t < NT; t++) {
-                        out[t] = M::mma(a[u][s], from.w[u][s][t] * from.scale[u][t], out[t]);
-                    }
+            for (int s = 0; s < RS; s++) {
+                const Vec right = from.w[u][s] * from.scale[u];
+#pragma unroll
+                for (int t = 0; t < NT; t++) {
+                    out.part[u & 1][t] = M::mma(a[s], right[t], out.part[u & 1][t]);
                 }
             }
         }
     };
 
-    Operands first;
-    Operands second;
-    load(first, 0); // in flight while T is computed
-    wave_sync();    // earlier reads of the T area are over
-    coupling_times_A<T>(t_area, p.A, p.to_cells, my_edge, lane, p.nA, p.layout.n_cell_tiles);
+    T a_rows[MAX_A_STEPS];
+    load_A_rows<T>(a_rows, p.A, edge_or_none, lane, p.nA); // first in the queue: T needs them first
+    Operands operands;
+    load(operands, 0);
+    wave_sync(); // earlier reads of the T area are over
+    coupling_times_A<T>(t_area, a_rows, p.to_cells, lane, p.layout.n_cell_tiles);
     wave_sync();
-    for (int32_t k0 = 0; k0 < n; k0 += 2 * EB) {
-        if (k0 + EB < n) {
-            load(second, k0 + EB);
-        }
-        multiply(first, k0);
-        if (k0 + 2 * EB < n) {
-            load(first, k0 + 2 * EB);
-        }
-        if (k0 + EB < n) {
-            multiply(second, k0 + EB);
-        }
+    multiply(operands, 0);
+    for (int32_t k0 = EB; k0 < n; k0 += EB) {
+        load(operands, k0);
+        multiply(operands, k0);
     }
 }
 
-template <typename T, int NT>
+/// Writes tile element (row, column i of tile t) to target[row * L + NT * i + t].
+template <typename T, int NT, typename Value>
 __device__ __forceinline__ void store_block(
-    T* __restrict__ target, const typename Mfma<T>::Acc (&acc)[NT], int32_t n_out, int32_t L, int lane
+    T* __restrict__ target, Value&& value, int32_t n_out, int32_t L, int lane
 ) {
     using M = Mfma<T>;
     const int i = lane & 15;
 #pragma unroll
-    for (int t = 0; t < NT; t++) {
+    for (int r = 0; r < 4; r++) {
+        const int32_t row = M::row(lane, r);
 #pragma unroll
-        for (int r = 0; r < 4; r++) {
-            const int32_t row = M::row(lane, r);
-            const int32_t col = 16 * t + i;
+        for (int t = 0; t < NT; t++) {
+            const int32_t col = NT * i + t;
             if (row < n_out && col < L) {
-                target[row * L + col] = acc[t][r];
+                target[row * L + col] = value(t, r);
             }
         }
     }
@@ -409,70 +462,126 @@ template <typename T> constexpr int forward_waves() { return sizeof(T) == 4 ? 4 
 /// ... and positions of the sorted index per workgroup, 16 per wavefront.
 template <typename T> constexpr int forward_chunk() { return STAGE * forward_waves<T>(); }
 
+/// Segments whose partial sums wait in LDS before the wavefronts meet.
+constexpr int ROUND_SEGMENTS = 2;
+
 template <typename T, int NT, int RS>
 __global__ __launch_bounds__(forward_waves<T>() * WAVE) void forward_kernel(
     T* __restrict__ output, const int32_t* __restrict__ receivers, int32_t n_edges, const Contraction<T> p
 ) {
-    using M = Mfma<T>;
     constexpr int FORWARD_WAVES = forward_waves<T>();
     constexpr int FORWARD_CHUNK = forward_chunk<T>();
+    constexpr int TILE = NT * 4 * WAVE; // elements of one wavefront's partial sums
     extern __shared__ __align__(16) char lds_raw[];
     const int lane = threadIdx.x & (WAVE - 1);
     const int wave = threadIdx.x >> 6;
     const int i = lane & 15;
     T* t_area = reinterpret_cast<T*>(lds_raw) + wave * p.layout.t_elements();
-    // partial sums of the wavefronts: [rank][NT][4][64]
+    // partial sums: [segment of the round][rank][NT][4][64]
     T* meeting = reinterpret_cast<T*>(lds_raw) + FORWARD_WAVES * p.layout.t_elements();
     const size_t row_elements = static_cast<size_t>(p.n_out) * p.L;
+
+    // the senders of this workgroup's positions, asked for before anything
+    // is known about the segments
+    const int32_t chunk_begin = blockIdx.x * FORWARD_CHUNK;
+    const int32_t chunk_position = chunk_begin + lane;
+    const int32_t chunk_source =
+        lane < FORWARD_CHUNK && chunk_position < n_edges ? p.gather_index[chunk_position] : -1;
 
     ContractionLane<T, NT, RS> mine;
     mine.setup(p, lane);
     clear_zero_row(t_area, p.layout, lane);
 
     int32_t stages_before = 0; // 16-edge stages dealt out so far, the same in every wavefront
+    int32_t waiting = 0;       // segments of the current round
+    int32_t waiting_node[ROUND_SEGMENTS];
+    int32_t waiting_participants[ROUND_SEGMENTS];
+
+    // All wavefronts meet; wavefront j adds up, in rank order, the partial
+    // sums of the j-th waiting segment and writes its output row.
+    auto meet = [&]() {
+        __syncthreads();
+#pragma unroll
+        for (int segment = 0; segment < ROUND_SEGMENTS; segment++) {
+            if (segment < waiting && (segment % FORWARD_WAVES) == wave) {
+                const T* slots = meeting + segment * FORWARD_WAVES * TILE;
+                T sum[NT][4];
+#pragma unroll
+                for (int t = 0; t < NT; t++) {
+#pragma unroll
+                    for (int r = 0; r < 4; r++) {
+                        sum[t][r] = slots[(t * 4 + r) * WAVE + lane];
+                    }
+                }
+                for (int32_t rank = 1; rank < waiting_participants[segment]; rank++) {
+#pragma unroll
+                    for (int t = 0; t < NT; t++) {
+#pragma unroll
+                        for (int r = 0; r < 4; r++) {
+                            sum[t][r] += slots[rank * TILE + (t * 4 + r) * WAVE + lane];
+                        }
+                    }
+                }
+                store_block<T, NT>(
+                    output + waiting_node[segment] * row_elements, [&](int t, int r) { return sum[t][r]; },
+                    p.n_out, p.L, lane
+                );
+            }
+        }
+        __syncthreads();
+        waiting = 0;
+    };
+
     walk_owned_segments<FORWARD_CHUNK>(
         receivers, n_edges, p.n_blocks, blockIdx.x,
         [&](int32_t node, int32_t first, int32_t last) {
             const int32_t n_stages = (last - first + STAGE - 1) / STAGE;
-            typename M::Acc acc[NT];
-#pragma unroll
-            for (int t = 0; t < NT; t++) {
-                acc[t] = M::zero();
-            }
+            Accumulators<T, NT> acc;
+            acc.clear();
             // stage number `st` goes to wavefront (stages_before + st) % FORWARD_WAVES
             const int32_t rank = (wave - stages_before) & (FORWARD_WAVES - 1);
             for (int32_t st = rank; st < n_stages; st += FORWARD_WAVES) {
                 const int32_t s0 = first + st * STAGE;
                 const int32_t n = min(STAGE, last - s0);
-                contract_batch<T, NT, RS>(acc, p, mine, t_area, i < n ? s0 + i : -1, n, lane);
+                const int32_t my_edge = i < n ? s0 + i : -1;
+                const int32_t offset = s0 + i - chunk_begin; // >= 0: owned segments start in the chunk
+                const bool at_hand = i < n && offset < FORWARD_CHUNK;
+                int32_t my_source = __shfl(chunk_source, at_hand ? offset : 0);
+                if (!at_hand) {
+                    my_source = i < n ? p.gather_index[my_edge] : -1;
+                }
+                contract_batch<T, NT, RS>(acc, p, mine, t_area, my_edge, my_source, n, lane);
             }
             const int32_t participants = min(n_stages, FORWARD_WAVES);
-            if (participants > 1) {
-                if (rank > 0 && rank < participants) {
+            if (participants == 1) {
+                if (rank == 0) {
+                    store_block<T, NT>(
+                        output + node * row_elements, [&](int t, int r) { return acc.total(t, r); }, p.n_out,
+                        p.L, lane
+                    );
+                }
+            } else {
+                if (rank < participants) {
+                    T* slot = meeting + (waiting * FORWARD_WAVES + rank) * TILE;
 #pragma unroll
                     for (int t = 0; t < NT; t++) {
 #pragma unroll
                         for (int r = 0; r < 4; r++) {
-                            meeting[((rank * NT + t) * 4 + r) * WAVE + lane] = acc[t][r];
+                            slot[(t * 4 + r) * WAVE + lane] = acc.total(t, r);
                         }
                     }
                 }
-                __syncthreads();
-                if (rank == 0) {
-                    for (int32_t other = 1; other < participants; other++) {
 #pragma unroll
-                        for (int t = 0; t < NT; t++) {
-#pragma unroll
-                            for (int r = 0; r < 4; r++) {
-                                acc[t][r] += meeting[((other * NT + t) * 4 + r) * WAVE + lane];
-                            }
-                        }
+                for (int segment = 0; segment < ROUND_SEGMENTS; segment++) {
+                    if (segment == waiting) {
+                        waiting_node[segment] = node;
+                        waiting_participants[segment] = participants;
                     }
                 }
-                __syncthreads();
-            }
-            if (rank == 0) {
-                store_block<T, NT>(output + node * row_elements, acc, p.n_out, p.L, lane);
+                waiting++;
+                if (waiting == ROUND_SEGMENTS) {
+                    meet();
+                }
             }
             stages_before += n_stages;
         },
@@ -484,6 +593,9 @@ __global__ __launch_bounds__(forward_waves<T>() * WAVE) void forward_kernel(
             }
         }
     );
+    if (waiting > 0) {
+        meet();
+    }
 }
 
 // ---------------------------------------------------------------------------
@@ -497,7 +609,6 @@ __global__ __launch_bounds__(senders_per_group<T>() * WAVE) void weight_gradient
     T* __restrict__ grad_W, const int32_t* __restrict__ senders, int32_t n_edges, bool aligned_senders,
     const Contraction<T> p
 ) {
-    using M = Mfma<T>;
     constexpr int SENDERS_PER_GROUP = senders_per_group<T>();
     using Gather = SenderGather<SENDERS_PER_GROUP>;
     extern __shared__ __align__(16) char lds_raw[];
@@ -512,13 +623,11 @@ __global__ __launch_bounds__(senders_per_group<T>() * WAVE) void weight_gradient
     ContractionLane<T, NT, RS> mine;
     mine.setup(p, lane);
     clear_zero_row(t_area, p.layout, lane);
-    typename M::Acc acc[NT];
-#pragma unroll
-    for (int t = 0; t < NT; t++) {
-        acc[t] = M::zero();
-    }
+    Accumulators<T, NT> acc;
+    acc.clear();
     auto on_stage = [&](int32_t my_edge, int32_t n) {
-        contract_batch<T, NT, RS>(acc, p, mine, t_area, my_edge, n, lane);
+        const int32_t my_source = my_edge >= 0 ? p.gather_index[my_edge] : -1;
+        contract_batch<T, NT, RS>(acc, p, mine, t_area, my_edge, my_source, n, lane);
     };
     if (aligned_senders) {
         Gather::template run<4>(gather, senders, n_edges, node0, p.n_blocks, on_stage);
@@ -526,7 +635,10 @@ __global__ __launch_bounds__(senders_per_group<T>() * WAVE) void weight_gradient
         Gather::template run<1>(gather, senders, n_edges, node0, p.n_blocks, on_stage);
     }
     if (node < p.n_blocks) {
-        store_block<T, NT>(grad_W + static_cast<size_t>(node) * p.n_out * p.L, acc, p.n_out, p.L, lane);
+        store_block<T, NT>(
+            grad_W + static_cast<size_t>(node) * p.n_out * p.L, [&](int t, int r) { return acc.total(t, r); },
+            p.n_out, p.L, lane
+        );
     }
 }
 
@@ -617,7 +729,9 @@ __global__ __launch_bounds__(WAVE) void edge_gradients_kernel(const EdgeGradArgs
 
     __syncthreads();
     if (want_B) {
-        coupling_times_A<T>(t_area, p.A, p.to_cells, my_edge, lane, p.nA, p.layout.n_cell_tiles);
+        T a_rows[MAX_A_STEPS];
+        load_A_rows<T>(a_rows, p.A, my_edge, lane, p.nA);
+        coupling_times_A<T>(t_area, a_rows, p.to_cells, lane, p.layout.n_cell_tiles);
     }
 
     // G of the receiver of the current edge, as operands
@@ -870,7 +984,8 @@ size_t t_area_bytes(const Shape& s, size_t element_size) {
 
 size_t forward_lds(const Shape& s, size_t element_size) {
     const size_t waves = element_size == 4 ? forward_waves<float>() : forward_waves<double>();
-    return waves * t_area_bytes(s, element_size) + waves * tiles_for(s.L) * 4 * WAVE * element_size;
+    return waves * t_area_bytes(s, element_size) +
+           ROUND_SEGMENTS * waves * tiles_for(s.L) * 4 * WAVE * element_size;
 }
 
 size_t weight_gradient_lds(const Shape& s, size_t element_size) {
@@ -917,6 +1032,9 @@ Contraction<T> contraction(
     c.n_red = n_red;
     c.out_cell_stride = out_cell_stride;
     c.red_cell_stride = red_cell_stride;
+    const size_t vector_bytes = tiles_for(s.L) * sizeof(T);
+    c.vector_rows = s.L % tiles_for(s.L) == 0 && reinterpret_cast<uintptr_t>(rows) % vector_bytes == 0 &&
+                    reinterpret_cast<uintptr_t>(B) % vector_bytes == 0;
     return c;
 }
 
