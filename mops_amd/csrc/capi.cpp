@@ -128,3 +128,16 @@ extern "C" int mops_amd_first_occurrences(
     mops::amd::finish_call("first_occurrences");
     MOPS_CATCH_EXCEPTIONS_END
 }
+
+extern "C" int mops_amd_kernel_timing(int enable) {
+    return mops::amd::set_kernel_timing(enable != 0) ? 1 : 0;
+}
+
+extern "C" int mops_amd_kernel_time(double* total_milliseconds, int64_t* launches) {
+    MOPS_CATCH_EXCEPTIONS_BEGIN
+    if (total_milliseconds == nullptr || launches == nullptr) {
+        throw std::runtime_error("mops_amd_kernel_time: both result pointers must be given");
+    }
+    mops::amd::collect_kernel_time(total_milliseconds, launches);
+    MOPS_CATCH_EXCEPTIONS_END
+}

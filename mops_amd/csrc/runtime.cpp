@@ -2,6 +2,8 @@
 
 #include <cstdlib>
 #include <limits>
+#include <utility>
+#include <vector>
 
 namespace mops::amd {
 
@@ -24,7 +26,23 @@ struct ThreadState {
     size_t capacity = 0;
     int device = -1;
     hipStream_t block_stream = nullptr;
+
+    // kernel timing
+    bool timing = false;
+    std::vector<std::pair<hipEvent_t, hipEvent_t>> recorded;
+    std::vector<hipEvent_t> spare;
 };
+
+hipEvent_t take_event(ThreadState& st) {
+    if (!st.spare.empty()) {
+        hipEvent_t event = st.spare.back();
+        st.spare.pop_back();
+        return event;
+    }
+    hipEvent_t event = nullptr;
+    MOPS_HIP_CHECK(hipEventCreate(&event));
+    return event;
+}
 
 ThreadState& state() {
     // Deliberately never destroyed: at thread or process exit the HIP runtime
@@ -53,6 +71,50 @@ void finish_call(const char* operation) {
     if (st.synchronous) {
         check_hip(hipStreamSynchronize(st.stream), operation);
     }
+}
+
+MainKernelTimer::MainKernelTimer(hipStream_t stream) : stream_(stream) {
+    auto& st = state();
+    if (!st.timing) {
+        return;
+    }
+    hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+    MOPS_HIP_CHECK(hipStreamIsCapturing(stream, &capture));
+    if (capture != hipStreamCaptureStatusNone) {
+        return;
+    }
+    hipEvent_t start = take_event(st);
+    stop_ = take_event(st);
+    MOPS_HIP_CHECK(hipEventRecord(start, stream));
+    st.recorded.emplace_back(start, stop_);
+}
+
+MainKernelTimer::~MainKernelTimer() {
+    if (stop_ != nullptr) {
+        (void)hipEventRecord(stop_, stream_);
+    }
+}
+
+bool set_kernel_timing(bool value) {
+    bool previous = state().timing;
+    state().timing = value;
+    return previous;
+}
+
+void collect_kernel_time(double* milliseconds, int64_t* launches) {
+    auto& st = state();
+    double total = 0.0;
+    for (auto& pair : st.recorded) {
+        MOPS_HIP_CHECK(hipEventSynchronize(pair.second));
+        float elapsed = 0.0f;
+        MOPS_HIP_CHECK(hipEventElapsedTime(&elapsed, pair.first, pair.second));
+        total += elapsed;
+        st.spare.push_back(pair.first);
+        st.spare.push_back(pair.second);
+    }
+    *milliseconds = total;
+    *launches = static_cast<int64_t>(st.recorded.size());
+    st.recorded.clear();
 }
 
 void* scratch(size_t bytes) {

@@ -42,6 +42,28 @@ void finish_call(const char* operation);
 /// block at the same time.
 void* scratch(size_t bytes);
 
+/// Device time of an operation's main kernel, for benchmarks that want the
+/// duration of one kernel and not of the whole call. While a thread has
+/// kernel timing on (set_kernel_timing), every MainKernelTimer in scope of a
+/// launch records a pair of HIP events around it on the stream it is launched
+/// on; collect_kernel_time waits for them and adds the intervals up. Streams
+/// that are being captured into a graph are left alone.
+class MainKernelTimer {
+public:
+    explicit MainKernelTimer(hipStream_t stream);
+    ~MainKernelTimer();
+    MainKernelTimer(const MainKernelTimer&) = delete;
+    MainKernelTimer& operator=(const MainKernelTimer&) = delete;
+
+private:
+    hipStream_t stream_;
+    hipEvent_t stop_ = nullptr;
+};
+bool set_kernel_timing(bool value);
+/// Sum (milliseconds) and number of the intervals recorded since the last
+/// call on this thread.
+void collect_kernel_time(double* milliseconds, int64_t* launches);
+
 /// ceil(a / b) for positive b.
 inline size_t ceil_div(size_t a, size_t b) { return (a + b - 1) / b; }
 

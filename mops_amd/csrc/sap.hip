@@ -705,6 +705,7 @@ void sparse_accumulation_of_products(MOPS_SAP_PARAMS(MOPS_CXX_FIRST, MOPS_CXX_NE
 
     const int waves = pick_waves(n_blocks, nO);
     const size_t lds = (tile_elements + (use_products ? product_elements : 0)) * sizeof(scalar_t);
+    MainKernelTimer timer(stream);
     if (use_products) {
         forward_kernel<scalar_t, true><<<static_cast<unsigned>(n_blocks), waves * WAVE, lds, stream>>>(
             output.data, A.data, B.data, table, n_rows, FastDivisor::make(nA), FastDivisor::make(nB),
@@ -776,6 +777,7 @@ void sparse_accumulation_of_products_vjp(MOPS_SAP_VJP_PARAMS(MOPS_CXX_FIRST, MOP
     // gradient is computed alongside.
     const int waves = pick_waves(n_blocks, (want_A ? nA : 0) + (want_B ? nB : 0));
     const size_t lds = tile_elements * sizeof(scalar_t);
+    MainKernelTimer timer(stream);
     vjp_kernel<scalar_t><<<static_cast<unsigned>(n_blocks), waves * WAVE, lds, stream>>>(
         grad_A.data, grad_B.data, grad_output.data, A.data, B.data, by_A, by_B, n_rows,
         FastDivisor::make(nA), FastDivisor::make(nB), FastDivisor::make(nO)
