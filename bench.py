@@ -258,6 +258,13 @@ def main():
     parser.add_argument("--warmup", type=int, default=100)
     parser.add_argument("--cpu-seconds", type=float, default=10.0)
     parser.add_argument("--no-per-op", action="store_true", help="only the headline workload")
+    parser.add_argument(
+        "--profile",
+        choices=["hpe", "sap", "opsa", "opsaw", "sasaw", "all"],
+        help="for rocprofv3: run 50 eager forward+vjp calls of the operation(s) at the BASELINE "
+        "shapes (all their dtypes) and 20 element-wise passes over 64 MiB (read 64 MiB, write 64 MiB) as a yardstick for the HBM "
+        "counters, print nothing, exit",
+    )
     args = parser.parse_args()
 
     if args.gpus != 1:
@@ -279,6 +286,22 @@ def main():
     bind_library_to_torch_stream(device)
     oracle = support.oracle_library()
     configs = build_configs()
+
+    if args.profile:
+        for _, op_name, _, op_case in configs:
+            if args.profile in (op_name, "all"):
+                w = DeviceWorkload(op_name, op_case, device)
+                for _ in range(50):
+                    w.step()
+                torch.cuda.synchronize()
+                del w
+                torch.cuda.empty_cache()
+        source = torch.empty(64 * 1024 * 1024 // 4, dtype=torch.float32, device=device).normal_()
+        target = torch.empty_like(source)
+        for _ in range(20):
+            torch.mul(source, 2.0, out=target)  # reads 64 MiB, writes 64 MiB
+        torch.cuda.synchronize()
+        return
 
     # ---------------- headline: c1 SAP f32, forward + vjp -------------------
     # The K timed steps are replays of HIP graphs that hold `steps_per_graph`
