@@ -364,15 +364,13 @@ def main():
             torch.cuda.empty_cache()
 
     # ---------------- roofline of the dominant kernel -----------------------
-    # forward: sort_table_kernel<float> then forward_kernel<float, true>;
-    # vjp: sort_table_kernel<float> then vjp_kernel<float> (mops_amd/csrc/sap.hip).
-    # The main kernel of each is timed on its own, with HIP events recorded by
-    # the library on the stream the kernel runs on.
+    # At this shape each call is one kernel (mops_amd/csrc/sap_mfma.hip), timed
+    # with HIP events recorded by the library on the stream the kernel runs on.
     library = bind_library_to_torch_stream(device)
     kernels = {}
     for kind, function, name in (
-        ("forward", workload.forward, "mops::amd::(anonymous namespace)::forward_kernel<float, true>"),
-        ("vjp", workload.vjp, "mops::amd::(anonymous namespace)::vjp_kernel<float>"),
+        ("forward", workload.forward, "mops::amd::sap_mfma::(anonymous namespace)::forward_kernel<float, 2, 2>"),
+        ("vjp", workload.vjp, "mops::amd::sap_mfma::(anonymous namespace)::vjp_kernel<float, 5>"),
     ):
         seconds, launches = main_kernel_time(library, function, 400)
         kernels[kind] = (seconds, launches, name)

@@ -44,6 +44,7 @@
 #include "device_common.hpp"
 #include "index_validation.hpp"
 #include "runtime.hpp"
+#include "sap_mfma.hpp"
 
 namespace mops::amd {
 namespace {
@@ -678,6 +679,13 @@ void sparse_accumulation_of_products(MOPS_SAP_PARAMS(MOPS_CXX_FIRST, MOPS_CXX_NE
         return;
     }
     hipStream_t stream = current_stream();
+    const sap_mfma::Shape dense_shape{n_rows, nA, nB, nO, n_products};
+    if (sap_mfma::supports_forward(dense_shape, sizeof(scalar_t))) {
+        const sap_mfma::Table dense_table{C.data, indices_A.data, indices_B.data, indices_output.data};
+        sap_mfma::forward<scalar_t>(output.data, A.data, B.data, dense_table, dense_shape, stream);
+        finish_call(operation);
+        return;
+    }
     const size_t n_blocks = ceil_div(static_cast<size_t>(n_rows), ROWS);
     const size_t tile_elements = (static_cast<size_t>(nA) + nB + nO) * ROW_STRIDE + ROWS;
     const size_t product_elements = static_cast<size_t>(nA) * nB * ROWS;
@@ -744,6 +752,15 @@ void sparse_accumulation_of_products_vjp(MOPS_SAP_VJP_PARAMS(MOPS_CXX_FIRST, MOP
         return;
     }
     hipStream_t stream = current_stream();
+    const sap_mfma::Shape dense_shape{n_rows, nA, nB, nO, n_products};
+    if (sap_mfma::supports_vjp(dense_shape, sizeof(scalar_t))) {
+        const sap_mfma::Table dense_table{C.data, indices_A.data, indices_B.data, indices_output.data};
+        sap_mfma::vjp<scalar_t>(
+            grad_A.data, grad_B.data, grad_output.data, A.data, B.data, dense_table, dense_shape, stream
+        );
+        finish_call(operation);
+        return;
+    }
     const size_t n_blocks = ceil_div(static_cast<size_t>(n_rows), ROWS);
     const size_t tile_elements =
         (static_cast<size_t>(nO) + 2 * (static_cast<size_t>(nA) + nB)) * ROW_STRIDE + ROWS;
