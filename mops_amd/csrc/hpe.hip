@@ -92,6 +92,94 @@ __global__ __launch_bounds__(256) void forward_kernel(
 }
 
 // ---------------------------------------------------------------------------
+// forward with the order known at compile time: factors and the values they
+// select in registers, the next monomial fetched while the current one is
+// multiplied, and the partial sums of the groups combined by a fixed tree
+// (shuffles inside a wavefront, then the wavefronts in order) instead of one
+// thread walking over all of them. R is a power of two.
+// ---------------------------------------------------------------------------
+template <typename T, int ORDER>
+__global__ __launch_bounds__(256) void forward_ordered_kernel(
+    T* __restrict__ output,
+    const T* __restrict__ A,
+    const T* __restrict__ C,
+    const int32_t* __restrict__ P,
+    int32_t n_rows,
+    int32_t nA,
+    int32_t n_monomials,
+    int32_t R
+) {
+    extern __shared__ __align__(16) unsigned char lds_bytes[];
+    T* a_stage = reinterpret_cast<T*>(lds_bytes);
+    T* partial = a_stage + static_cast<size_t>(nA) * R;
+
+    const int tid = threadIdx.x;
+    const int G = blockDim.x / R;
+    const int r = tid % R;
+    const int g = tid / R;
+    const int32_t row0 = blockIdx.x * R;
+    const int32_t rows = min(R, n_rows - row0);
+
+    const T* a_src = A + static_cast<size_t>(row0) * nA;
+    for (int32_t i = tid; i < rows * nA; i += blockDim.x) {
+        int32_t row = i / nA;
+        a_stage[(i - row * nA) * R + row] = a_src[i];
+    }
+    __syncthreads();
+
+    struct Monomial {
+        int32_t factor[ORDER > 0 ? ORDER : 1];
+        T coefficient;
+    };
+    auto fetch = [&](Monomial& to, int32_t j) {
+        const int32_t safe = min(j, n_monomials - 1);
+        const int32_t* factors = P + static_cast<size_t>(safe) * ORDER;
+#pragma unroll
+        for (int k = 0; k < ORDER; k++) {
+            to.factor[k] = factors[k];
+        }
+        to.coefficient = C[safe];
+    };
+    T sum = T(0);
+    if (r < rows && n_monomials > 0) {
+        Monomial next;
+        fetch(next, g);
+        for (int32_t j = g; j < n_monomials; j += G) {
+            const Monomial now = next;
+            fetch(next, j + G);
+            T product = now.coefficient;
+#pragma unroll
+            for (int k = 0; k < ORDER; k++) {
+                product *= in_bounds(now.factor[k], nA) ? a_stage[now.factor[k] * R + r] : T(0);
+            }
+            sum += product;
+        }
+    }
+    // lanes with the same r inside a wavefront, then the wavefronts
+    for (int offset = WAVE / 2; offset >= R; offset >>= 1) {
+        sum += __shfl_xor(sum, offset);
+    }
+    const int wave = tid / WAVE;
+    const int lane = tid % WAVE;
+    if (R <= WAVE) {
+        if (lane < R) {
+            partial[wave * R + lane] = sum;
+        }
+    } else {
+        partial[g * R + r] = sum;
+    }
+    __syncthreads();
+    const int copies = R <= WAVE ? static_cast<int>(blockDim.x) / WAVE : G;
+    if (tid < rows) {
+        T total = T(0);
+        for (int copy = 0; copy < copies; copy++) {
+            total += partial[copy * R + tid];
+        }
+        output[row0 + tid] = total;
+    }
+}
+
+// ---------------------------------------------------------------------------
 // vjp. One wavefront per workgroup. LDS: a[nA][R] accumulator[G][nA][R]
 // Thread (r, g) adds its monomials' terms into its private accumulator row
 // set; afterwards the G copies are added in group order.
@@ -150,6 +238,105 @@ __global__ __launch_bounds__(WAVE) void vjp_kernel(
                     term *= in_bounds(feature, nA) ? a_stage[feature * R + r] : T(0);
                 }
                 mine[target * R] += term;
+            }
+        }
+    }
+    __syncthreads();
+
+    T* dst = grad_A + static_cast<size_t>(row0) * nA;
+    for (int32_t i = tid; i < rows * nA; i += WAVE) {
+        int32_t row = i / nA;
+        int32_t feature = i - row * nA;
+        T total = T(0);
+        for (int group = 0; group < G; group++) {
+            total += accumulator[(static_cast<size_t>(group) * nA + feature) * R + row];
+        }
+        dst[i] = total;
+    }
+}
+
+// ---------------------------------------------------------------------------
+// vjp with the order known at compile time: same layout as vjp_kernel, but a
+// monomial's factors, the values they select and the K partial products
+// (prefix * suffix, 3 K multiplications instead of K^2) live in registers, and
+// the factors of the next monomial are fetched while the current one is used.
+// ---------------------------------------------------------------------------
+template <typename T, int ORDER>
+__global__ __launch_bounds__(WAVE) void vjp_ordered_kernel(
+    T* __restrict__ grad_A,
+    const T* __restrict__ grad_output,
+    const T* __restrict__ A,
+    const T* __restrict__ C,
+    const int32_t* __restrict__ P,
+    int32_t n_rows,
+    int32_t nA,
+    int32_t n_monomials,
+    int32_t R
+) {
+    extern __shared__ __align__(16) unsigned char lds_bytes[];
+    T* a_stage = reinterpret_cast<T*>(lds_bytes);
+    T* accumulator = a_stage + static_cast<size_t>(nA) * R;
+
+    const int tid = threadIdx.x;
+    const int G = WAVE / R;
+    const int r = tid % R;
+    const int g = tid / R;
+    const int32_t row0 = blockIdx.x * R;
+    const int32_t rows = min(R, n_rows - row0);
+
+    const T* a_src = A + static_cast<size_t>(row0) * nA;
+    for (int32_t i = tid; i < rows * nA; i += WAVE) {
+        int32_t row = i / nA;
+        a_stage[(i - row * nA) * R + row] = a_src[i];
+    }
+    for (int32_t i = tid; i < G * nA * R; i += WAVE) {
+        accumulator[i] = T(0);
+    }
+    __syncthreads();
+
+    if (r < rows) {
+        T* mine = accumulator + static_cast<size_t>(g) * nA * R + r;
+        const T upstream = grad_output[row0 + r];
+        struct Monomial {
+            int32_t factor[ORDER];
+            T coefficient;
+        };
+        auto fetch = [&](Monomial& to, int32_t j) {
+            const int32_t safe = min(j, n_monomials - 1);
+            const int32_t* factors = P + static_cast<size_t>(safe) * ORDER;
+#pragma unroll
+            for (int k = 0; k < ORDER; k++) {
+                to.factor[k] = factors[k];
+            }
+            to.coefficient = C[safe];
+        };
+        Monomial next;
+        fetch(next, g);
+        for (int32_t j = g; j < n_monomials; j += G) {
+            const Monomial now = next;
+            fetch(next, j + G);
+            T value[ORDER];
+            bool valid[ORDER];
+#pragma unroll
+            for (int k = 0; k < ORDER; k++) {
+                valid[k] = in_bounds(now.factor[k], nA);
+                value[k] = valid[k] ? a_stage[now.factor[k] * R + r] : T(0);
+            }
+            // term[f] = base * prod_{k != f} value[k], multiplied left to right
+            T prefix[ORDER];
+            prefix[0] = now.coefficient * upstream;
+#pragma unroll
+            for (int k = 1; k < ORDER; k++) {
+                prefix[k] = prefix[k - 1] * value[k - 1];
+            }
+            T suffix = T(1);
+#pragma unroll
+            for (int f = ORDER - 1; f >= 0; f--) {
+                const T term = prefix[f] * suffix;
+                suffix *= value[f];
+                if (valid[f]) {
+                    mine[now.factor[f] * R] += term;
+                }
             }
         }
     }
@@ -281,9 +468,39 @@ void homogeneous_polynomial_evaluation(MOPS_HPE_PARAMS(MOPS_CXX_FIRST, MOPS_CXX_
     if (R > 0) {
         size_t lds = (static_cast<size_t>(nA) * R + THREADS) * sizeof(scalar_t);
         unsigned blocks = static_cast<unsigned>(ceil_div(static_cast<size_t>(n_rows), R));
-        forward_kernel<scalar_t><<<blocks, THREADS, lds, stream>>>(
-            output.data, A.data, C.data, indices_A.data, n_rows, nA, n_monomials, order, R
-        );
+#define MOPS_LAUNCH_ORDERED(ORDER)                                                                  \
+    forward_ordered_kernel<scalar_t, ORDER><<<blocks, THREADS, lds, stream>>>(                     \
+        output.data, A.data, C.data, indices_A.data, n_rows, nA, n_monomials, R                    \
+    )
+        switch (order) {
+        case 0:
+            MOPS_LAUNCH_ORDERED(0);
+            break;
+        case 1:
+            MOPS_LAUNCH_ORDERED(1);
+            break;
+        case 2:
+            MOPS_LAUNCH_ORDERED(2);
+            break;
+        case 3:
+            MOPS_LAUNCH_ORDERED(3);
+            break;
+        case 4:
+            MOPS_LAUNCH_ORDERED(4);
+            break;
+        case 5:
+            MOPS_LAUNCH_ORDERED(5);
+            break;
+        case 6:
+            MOPS_LAUNCH_ORDERED(6);
+            break;
+        default:
+            forward_kernel<scalar_t><<<blocks, THREADS, lds, stream>>>(
+                output.data, A.data, C.data, indices_A.data, n_rows, nA, n_monomials, order, R
+            );
+            break;
+        }
+#undef MOPS_LAUNCH_ORDERED
     } else {
         unsigned blocks = static_cast<unsigned>(ceil_div(static_cast<size_t>(n_rows), THREADS));
         forward_global_kernel<scalar_t><<<blocks, THREADS, 0, stream>>>(
@@ -328,10 +545,37 @@ void homogeneous_polynomial_evaluation_vjp(MOPS_HPE_VJP_PARAMS(MOPS_CXX_FIRST, M
     if (R > 0) {
         size_t lds = accumulator_bytes + static_cast<size_t>(nA) * R * sizeof(scalar_t);
         unsigned blocks = static_cast<unsigned>(ceil_div(static_cast<size_t>(n_rows), R));
-        vjp_kernel<scalar_t><<<blocks, WAVE, lds, stream>>>(
-            grad_A.data, grad_output.data, A.data, C.data, indices_A.data, n_rows, nA, n_monomials,
-            order, R
-        );
+#define MOPS_LAUNCH_ORDERED(ORDER)                                                                  \
+    vjp_ordered_kernel<scalar_t, ORDER><<<blocks, WAVE, lds, stream>>>(                            \
+        grad_A.data, grad_output.data, A.data, C.data, indices_A.data, n_rows, nA, n_monomials, R  \
+    )
+        switch (n_monomials > 0 ? order : 0) {
+        case 1:
+            MOPS_LAUNCH_ORDERED(1);
+            break;
+        case 2:
+            MOPS_LAUNCH_ORDERED(2);
+            break;
+        case 3:
+            MOPS_LAUNCH_ORDERED(3);
+            break;
+        case 4:
+            MOPS_LAUNCH_ORDERED(4);
+            break;
+        case 5:
+            MOPS_LAUNCH_ORDERED(5);
+            break;
+        case 6:
+            MOPS_LAUNCH_ORDERED(6);
+            break;
+        default:
+            vjp_kernel<scalar_t><<<blocks, WAVE, lds, stream>>>(
+                grad_A.data, grad_output.data, A.data, C.data, indices_A.data, n_rows, nA, n_monomials,
+                order, R
+            );
+            break;
+        }
+#undef MOPS_LAUNCH_ORDERED
     } else {
         unsigned blocks = static_cast<unsigned>(ceil_div(static_cast<size_t>(n_rows), 256));
         vjp_global_kernel<scalar_t><<<blocks, 256, 0, stream>>>(

@@ -42,6 +42,7 @@
 #include "runtime.hpp"
 #include "segment_walk.hpp"
 #include "sender_buckets.hpp"
+#include "sender_gather.hpp"
 
 namespace mops::amd {
 namespace {
@@ -507,6 +508,73 @@ __global__ __launch_bounds__(256) void gather_weights_kernel(
     }
 }
 
+// The same sum without any list in global memory: the workgroup's eight
+// wavefronts find the edges of their eight senders by one pass over the
+// sender index (sender_gather.hpp) and add the rows up, sixteen loads in
+// flight. Used when a row of W fits one value per lane and register.
+constexpr int GATHER_SENDERS = 8;
+constexpr int GATHER_COLUMNS = 4; // values of a row per lane
+
+template <typename T>
+__global__ __launch_bounds__(GATHER_SENDERS* WAVE) void sum_by_sender_kernel(
+    T* __restrict__ grad_W, const T* __restrict__ edge_W, const int32_t* __restrict__ senders,
+    int32_t n_edges, int32_t n_nodes, int32_t L, bool aligned_senders
+) {
+    using Gather = SenderGather<GATHER_SENDERS>;
+    __shared__ typename Gather::Storage storage;
+    const int lane = threadIdx.x & (WAVE - 1);
+    const int wave = threadIdx.x >> 6;
+    const int32_t node0 = blockIdx.x * GATHER_SENDERS;
+    T sum[GATHER_COLUMNS];
+    uint32_t column[GATHER_COLUMNS];
+#pragma unroll
+    for (int c = 0; c < GATHER_COLUMNS; c++) {
+        sum[c] = T(0);
+        column[c] = min(lane + c * WAVE, L - 1);
+    }
+    auto on_stage = [&](int32_t my_edge, int32_t n) {
+        T values[Gather::STAGE][GATHER_COLUMNS];
+#pragma unroll
+        for (int k = 0; k < Gather::STAGE; k++) {
+            // lanes beyond n hold -1: read row 0 and leave it out of the sum
+            const int32_t edge = max(__builtin_amdgcn_readlane(my_edge, k), 0);
+            const T* row = edge_W + static_cast<size_t>(edge) * L;
+#pragma unroll
+            for (int c = 0; c < GATHER_COLUMNS; c++) {
+                if (c * WAVE < L) {
+                    values[k][c] = row[column[c]];
+                }
+            }
+        }
+#pragma unroll
+        for (int k = 0; k < Gather::STAGE; k++) {
+            if (k < n) {
+#pragma unroll
+                for (int c = 0; c < GATHER_COLUMNS; c++) {
+                    if (c * WAVE < L) {
+                        sum[c] += values[k][c];
+                    }
+                }
+            }
+        }
+    };
+    if (aligned_senders) {
+        Gather::template run<4>(storage, senders, n_edges, node0, n_nodes, on_stage);
+    } else {
+        Gather::template run<1>(storage, senders, n_edges, node0, n_nodes, on_stage);
+    }
+    const int32_t node = node0 + wave;
+    if (node < n_nodes) {
+#pragma unroll
+        for (int c = 0; c < GATHER_COLUMNS; c++) {
+            const int32_t l = lane + c * WAVE;
+            if (l < L) {
+                grad_W[static_cast<size_t>(node) * L + l] = sum[c];
+            }
+        }
+    }
+}
+
 unsigned blocks_for(int32_t n_edges) {
     size_t waves = ceil_div(static_cast<size_t>(n_edges), CHUNK);
     return static_cast<unsigned>(ceil_div(waves, WAVES_PER_BLOCK));
@@ -583,7 +651,9 @@ void launch_vjp(
     // scratch: edge_W | sender buckets   (only when grad_W is wanted)
     const size_t edge_w_bytes =
         want_W ? align256(static_cast<size_t>(n_edges) * L * sizeof(T)) : 0;
-    const size_t buckets_bytes = want_W ? sender_buckets_bytes(n_output, n_edges) : 0;
+    const bool gather_in_kernel = L <= GATHER_COLUMNS * WAVE && n_edges > 0;
+    const size_t buckets_bytes =
+        want_W && !gather_in_kernel ? sender_buckets_bytes(n_output, n_edges) : 0;
     char* workspace =
         want_W ? static_cast<char*>(scratch(edge_w_bytes + buckets_bytes)) : nullptr;
     T* edge_W = want_W ? reinterpret_cast<T*>(workspace) : nullptr;
@@ -632,7 +702,13 @@ void launch_vjp(
         );
     }
 
-    if (want_W && n_output > 0 && L > 0) {
+    if (want_W && n_output > 0 && L > 0 && gather_in_kernel) {
+        const bool aligned = reinterpret_cast<uintptr_t>(indices_W) % 16 == 0;
+        const unsigned blocks = static_cast<unsigned>(ceil_div(static_cast<size_t>(n_output), GATHER_SENDERS));
+        sum_by_sender_kernel<T><<<blocks, GATHER_SENDERS * WAVE, 0, stream>>>(
+            grad_W.data, edge_W, indices_W, n_edges, n_output, L, aligned
+        );
+    } else if (want_W && n_output > 0 && L > 0) {
         SenderBuckets buckets =
             build_sender_buckets(indices_W, n_edges, n_output, workspace + edge_w_bytes, stream);
         int threads = std::min(256, round_up_wave(L));

@@ -128,42 +128,39 @@ template <int NW> struct SenderGather {
                         values[u][0] = ok ? values[u][0] : -1;
                     }
                 }
+                // Matches are rare (one lane in a few hundred), so they are
+                // handled one at a time by the whole wavefront: a uniform loop
+                // over the lanes that found something, in lane (= edge) order.
                 int consumed = 0;
 #pragma unroll
                 for (int u = 0; u < BATCH; u++) {
                     if (full || unit + u >= unit_end) {
                         continue;
                     }
-                    bool match[VEC];
-                    bool any_match = false;
+                    uint32_t found = 0; // bit c: component c names one of our nodes
 #pragma unroll
                     for (int c = 0; c < VEC; c++) {
-                        match[c] = in_bounds(values[u][c] - node0, served);
-                        any_match |= match[c];
+                        found |= in_bounds(values[u][c] - node0, served) ? (1u << c) : 0u;
                     }
-                    if (__ballot(any_match) != 0) {
-                        int32_t before = 0;
-                        int32_t total = 0;
+                    unsigned long long finders = __ballot(found != 0);
+                    if (count + VEC * __popcll(finders) > CAPACITY) {
+                        full = true;
+                        continue;
+                    }
+                    while (finders != 0) {
+                        const int finder = __ffsll(static_cast<long long>(finders)) - 1;
+                        finders &= finders - 1;
+                        const uint32_t bits = __builtin_amdgcn_readlane(found, finder);
 #pragma unroll
                         for (int c = 0; c < VEC; c++) {
-                            const unsigned long long mask = __ballot(match[c]);
-                            before += __popcll(mask & below);
-                            total += __popcll(mask);
-                        }
-                        if (count + total > CAPACITY) {
-                            full = true;
-                            continue;
-                        }
-                        int32_t slot = count + before;
-#pragma unroll
-                        for (int c = 0; c < VEC; c++) {
-                            if (match[c]) {
-                                lds.edges[wave][slot] = (unit + u) * UNIT + lane * VEC + c;
-                                lds.which[wave][slot] = static_cast<uint8_t>(values[u][c] - node0);
-                                slot++;
+                            if (bits & (1u << c)) {
+                                const int32_t value = __builtin_amdgcn_readlane(values[u][c], finder);
+                                // every lane writes the same value to the same place
+                                lds.edges[wave][count] = (unit + u) * UNIT + finder * VEC + c;
+                                lds.which[wave][count] = static_cast<uint8_t>(value - node0);
+                                count++;
                             }
                         }
-                        count += total;
                     }
                     consumed = u + 1;
                 }
