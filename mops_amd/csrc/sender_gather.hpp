@@ -96,6 +96,8 @@ template <int NW> struct SenderGather {
             }
         };
 
+        // the wavefront of the last slice also looks after the last n_edges % 4 positions
+        bool tail_done = VEC != 4 || wave != NW - 1;
         bool more = true;
         while (more) {
             // ---- scan my slice until it ends or my list is full
@@ -115,13 +117,9 @@ template <int NW> struct SenderGather {
                         values[u][1] = whole ? loaded.y : -1;
                         values[u][2] = whole ? loaded.z : -1;
                         values[u][3] = whole ? loaded.w : -1;
-                        if (!whole && unit + u < unit_end) {
-                            // the last few positions of the index
-#pragma unroll
-                            for (int c = 0; c < 4; c++) {
-                                values[u][c] = position + c < n_edges ? senders[position + c] : -1;
-                            }
-                        }
+                        // (the last n_edges % 4 positions are looked at below:
+                        // a conditional load here would make every load of the
+                        // batch wait for the one before)
                     } else {
                         const bool ok = unit + u < unit_end && position < n_edges;
                         values[u][0] = load_or_zero(senders, position, ok);
@@ -166,9 +164,23 @@ template <int NW> struct SenderGather {
                 }
                 unit += consumed;
             }
+            if (VEC == 4 && !tail_done && unit >= unit_end && !full) {
+                // the positions after the last whole group of four
+                if (count + 3 <= CAPACITY) {
+                    for (int32_t position = n_edges & ~3; position < n_edges; position++) {
+                        const int32_t value = senders[position];
+                        if (in_bounds(value - node0, served)) {
+                            lds.edges[wave][count] = position;
+                            lds.which[wave][count] = static_cast<uint8_t>(value - node0);
+                            count++;
+                        }
+                    }
+                    tail_done = true;
+                }
+            }
             if (lane == 0) {
                 lds.counts[wave] = count;
-                lds.resume[wave] = unit < unit_end ? 1 : 0;
+                lds.resume[wave] = (unit < unit_end || !tail_done) ? 1 : 0;
             }
             __syncthreads();
 

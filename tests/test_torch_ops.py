@@ -1,0 +1,84 @@
+"""torch.ops.mops.*: schemas (as mops-torch/src/register.cpp of the reference), values, autograd."""
+import numpy as np
+import pytest
+import torch
+
+import mops_amd.torch  # noqa: F401  (registers the operators)
+from tests import support
+
+SCHEMAS = {
+    "homogeneous_polynomial_evaluation": "mops::homogeneous_polynomial_evaluation(Tensor A, Tensor C, Tensor indices_A) -> Tensor",
+    "outer_product_scatter_add": "mops::outer_product_scatter_add(Tensor A, Tensor B, Tensor indices_output, int output_size) -> Tensor",
+    "sparse_accumulation_of_products": "mops::sparse_accumulation_of_products(Tensor A, Tensor B, Tensor C, Tensor indices_A, Tensor indices_B, Tensor indices_output, int output_size) -> Tensor",
+    "outer_product_scatter_add_with_weights": "mops::outer_product_scatter_add_with_weights(Tensor A, Tensor B, Tensor W, Tensor indices_W, Tensor indices_output) -> Tensor",
+    "sparse_accumulation_scatter_add_with_weights": "mops::sparse_accumulation_scatter_add_with_weights(Tensor A, Tensor B, Tensor C, Tensor W, Tensor indices_A, Tensor indices_W_1, Tensor indices_W_2, Tensor indices_output_1, Tensor indices_output_2, int output_size) -> Tensor",
+}  # fmt: skip
+
+SMALL = {
+    "hpe": lambda d: support.hpe_case(11, d, I=9, nA=5, J=12, K=3),
+    "sap": lambda d: support.sap_case(12, d, I=70, nA=4, nB=3, K=15, nO=5),
+    "opsa": lambda d: support.opsa_case(13, d, J=50, K=3, L=4, n_out=6, allow_empty=True),
+    "opsaw": lambda d: support.opsaw_case(14, d, E=50, K=3, L=4, n_nodes=6, allow_empty=True),
+    "sasaw": lambda d: support.sasaw_case(15, d, E=40, nA=3, L=4, n_nodes=5, n2=3, n3=4, N=11, allow_empty=True),
+}  # fmt: skip
+
+
+def arguments(op, case):
+    """Arguments of torch.ops.mops.<op> in schema order."""
+    tensors = [case[name] for name in support.OPS[op].inputs]
+    if op in ("sap", "opsa", "sasaw"):
+        tensors.append(case["output_size"])
+    return tensors
+
+
+def test_schemas_match_the_reference():
+    for name, schema in SCHEMAS.items():
+        assert str(getattr(torch.ops.mops, name).default._schema) == schema
+
+
+def test_host_tensors_are_refused():
+    case = SMALL["opsa"](np.float64)
+    tensors = [torch.from_numpy(v) if isinstance(v, np.ndarray) else v for v in arguments("opsa", case)]
+    with pytest.raises(RuntimeError, match="device path only"):
+        torch.ops.mops.outer_product_scatter_add(*tensors)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [np.float32, np.float64], ids=["f32", "f64"])
+@pytest.mark.parametrize("op", list(SMALL))
+def test_operator_values(oracle, device, op, dtype):
+    case = SMALL[op](dtype)
+    expected = support.cpu_forward(oracle, op, case)
+    on_device = support.to_device(case, device)
+    operator = getattr(torch.ops.mops, support.OPS[op].function)
+    actual = operator(*arguments(op, on_device))
+    support.assert_close(actual.cpu().numpy(), expected, dtype, op)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("op", list(SMALL))
+def test_operator_gradients(oracle, device, op):
+    """Backward of the operator = the oracle's vjp; and torch's own finite-difference gradcheck."""
+    case = SMALL[op](np.float64)
+    expected = support.cpu_vjp(oracle, op, case)
+    on_device = support.to_device(case, device)
+    spec = support.OPS[op]
+    for name in spec.differentiable:
+        on_device[name].requires_grad_(True)
+    operator = getattr(torch.ops.mops, spec.function)
+    output = operator(*arguments(op, on_device))
+    output.backward(on_device["grad_output"])
+    for name in spec.differentiable:
+        support.assert_close(on_device[name].grad.cpu().numpy(), expected[name], np.float64, f"{op} grad_{name}")
+    for name in spec.differentiable:
+        on_device[name].grad = None
+    assert torch.autograd.gradcheck(operator, arguments(op, on_device), fast_mode=True)
+
+
+@pytest.mark.gpu
+def test_only_requested_gradients_are_computed(device):
+    case = support.to_device(SMALL["opsaw"](np.float64), device)
+    case["B"].requires_grad_(True)
+    output = torch.ops.mops.outer_product_scatter_add_with_weights(*arguments("opsaw", case))
+    output.sum().backward()
+    assert case["B"].grad is not None and case["A"].grad is None and case["W"].grad is None
