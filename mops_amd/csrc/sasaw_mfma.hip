@@ -335,7 +335,7 @@ __device__ __forceinline__ void contract_batch(
     // Edges whose operands are in flight together: a round trip to memory
     // costs about as much as the arithmetic of all 16 edges, so as many as
     // the registers hold (RS * NT + NT values per edge).
-    constexpr int EB = (sizeof(T) == 8 ? 4 : 8) / (NT >= 4 ? 2 : 1);
+    constexpr int EB = 4 / (NT >= 4 ? 2 : 1);
     const uint32_t block_elements = static_cast<uint32_t>(p.n_red) * p.L;
     // Nothing below is conditional: lanes 0..15 without an edge (or with a
     // source out of range) get a zero column of T, and their operand loads are
@@ -463,7 +463,7 @@ template <typename T> constexpr int forward_waves() { return sizeof(T) == 4 ? 4 
 template <typename T> constexpr int forward_chunk() { return STAGE * forward_waves<T>(); }
 
 /// Segments whose partial sums wait in LDS before the wavefronts meet.
-constexpr int ROUND_SEGMENTS = 2;
+template <typename T> constexpr int round_segments() { return sizeof(T) == 4 ? 2 : 1; }
 
 template <typename T, int NT, int RS>
 __global__ __launch_bounds__(forward_waves<T>() * WAVE) void forward_kernel(
@@ -471,6 +471,7 @@ __global__ __launch_bounds__(forward_waves<T>() * WAVE) void forward_kernel(
 ) {
     constexpr int FORWARD_WAVES = forward_waves<T>();
     constexpr int FORWARD_CHUNK = forward_chunk<T>();
+    constexpr int ROUND_SEGMENTS = round_segments<T>();
     constexpr int TILE = NT * 4 * WAVE; // elements of one wavefront's partial sums
     extern __shared__ __align__(16) char lds_raw[];
     const int lane = threadIdx.x & (WAVE - 1);
@@ -985,7 +986,8 @@ size_t t_area_bytes(const Shape& s, size_t element_size) {
 size_t forward_lds(const Shape& s, size_t element_size) {
     const size_t waves = element_size == 4 ? forward_waves<float>() : forward_waves<double>();
     return waves * t_area_bytes(s, element_size) +
-           ROUND_SEGMENTS * waves * tiles_for(s.L) * 4 * WAVE * element_size;
+           (element_size == 4 ? round_segments<float>() : round_segments<double>()) * waves * tiles_for(s.L) * 4 *
+               WAVE * element_size;
 }
 
 size_t weight_gradient_lds(const Shape& s, size_t element_size) {
