@@ -458,7 +458,7 @@ __device__ __forceinline__ void clear_zero_row(T* __restrict__ t_area, const Den
 // forward pass
 
 /// Wavefronts per workgroup (their T areas share 64 KB of LDS) ...
-template <typename T> constexpr int forward_waves() { return sizeof(T) == 4 ? 4 : 2; }
+template <typename T> constexpr int forward_waves() { return 2; }
 /// ... and positions of the sorted index per workgroup, 16 per wavefront.
 template <typename T> constexpr int forward_chunk() { return STAGE * forward_waves<T>(); }
 
@@ -603,7 +603,7 @@ __global__ __launch_bounds__(forward_waves<T>() * WAVE) void forward_kernel(
 // grad_W: one wavefront per sender
 
 /// Wavefronts (= senders) per workgroup.
-template <typename T> constexpr int senders_per_group() { return sizeof(T) == 4 ? 6 : 4; }
+template <typename T> constexpr int senders_per_group() { return 4; }
 
 template <typename T, int NT, int RS>
 __global__ __launch_bounds__(senders_per_group<T>() * WAVE) void weight_gradient_kernel(
