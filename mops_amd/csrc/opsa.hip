@@ -508,6 +508,192 @@ __global__ __launch_bounds__(256) void gather_weights_kernel(
     }
 }
 
+// ---------------------------------------------------------------------------
+// vjp for moderate feature counts (K <= 32, L <= 64), the shapes of the
+// reference's benchmarks: the gradients are per EDGE, so nothing has to follow
+// the segments. A wavefront takes 16 consecutive edges, whatever receivers
+// they have: it knows which rows of A, B (and W) it needs before it has seen
+// any index, all its loads go straight from global memory into matrix
+// operands (no LDS), and for every receiver among its edges it multiplies the
+// rows of that receiver (the others zeroed) with the receiver's grad_output:
+//
+//   grad_A[e, k] = sum_l (B * W)[e, l] * gO[node, k, l]     16 x L times L x K
+//   grad_B[e, l] = sum_k A[e, k] * gO[node, k, l] (* W)     16 x K times K x L
+//
+// Rows of the result belong to one edge each, so the products for different
+// receivers add up in the same accumulators. Two dependent round trips to
+// memory (index, then grad_output), every wavefront the same amount of work.
+// ---------------------------------------------------------------------------
+template <typename T, int KT, int NT, bool WEIGHTED>
+__global__ __launch_bounds__(WAVE) void edge_rows_vjp_kernel(
+    T* __restrict__ grad_A,
+    T* __restrict__ grad_B,
+    T* __restrict__ edge_W,
+    const T* __restrict__ grad_output,
+    const T* __restrict__ A,
+    const T* __restrict__ B,
+    const T* __restrict__ W,
+    const int32_t* __restrict__ indices_W,
+    const int32_t* __restrict__ indices_output,
+    int32_t n_edges,
+    int32_t n_output,
+    int32_t K,
+    int32_t L
+) {
+    using M = Mfma<T>;
+    constexpr int K_STEPS = 4 * KT;
+    constexpr int L_STEPS = 4 * NT;
+    const int lane = threadIdx.x;
+    const int i = lane & 15;
+    const int q = lane >> 4;
+    const int32_t first_edge = blockIdx.x * 16;
+    const int32_t n = min(16, n_edges - first_edge);
+    const int32_t my_edge = i < n ? first_edge + i : -1;
+    const bool want_A = grad_A != nullptr;
+    const bool want_B = grad_B != nullptr;
+    const bool want_W = WEIGHTED && edge_W != nullptr;
+
+    const int32_t my_node = my_edge >= 0 ? indices_output[my_edge] : -1;
+    int32_t my_sender = 0;
+    if constexpr (WEIGHTED) {
+        my_sender = my_edge >= 0 ? indices_W[my_edge] : -1;
+    }
+    const bool sender_ok = !WEIGHTED || in_bounds(my_sender, n_output);
+
+    // left operands: lane (row = edge i, reduction index 4 s + q)
+    T b_left[L_STEPS]; // (B * W)[e, l]
+    T a_left[K_STEPS]; // A[e, k]
+#pragma unroll
+    for (int s = 0; s < L_STEPS; s++) {
+        const int32_t l = 4 * s + q;
+        const bool ok = my_edge >= 0 && l < L;
+        b_left[s] = load_or_zero(B, static_cast<size_t>(my_edge) * L + l, ok && want_A);
+        if constexpr (WEIGHTED) {
+            b_left[s] *= load_or_zero(W, static_cast<size_t>(my_sender) * L + l, ok && want_A && sender_ok);
+        }
+    }
+#pragma unroll
+    for (int s = 0; s < K_STEPS; s++) {
+        const int32_t k = 4 * s + q;
+        a_left[s] = load_or_zero(A, static_cast<size_t>(my_edge) * K + k, my_edge >= 0 && k < K && (want_B || want_W));
+    }
+
+    typename M::Acc acc_A[KT];
+    typename M::Acc acc_B[NT];
+#pragma unroll
+    for (int t = 0; t < KT; t++) {
+        acc_A[t] = M::zero();
+    }
+#pragma unroll
+    for (int t = 0; t < NT; t++) {
+        acc_B[t] = M::zero();
+    }
+
+    const int32_t l_steps = (L + 3) >> 2;
+    const int32_t k_steps = (K + 3) >> 2;
+    // the receivers among my edges, in ascending order (the index is sorted)
+    int32_t node = __builtin_amdgcn_readfirstlane(my_node);
+    while (node >= 0) {
+        if (in_bounds(node, n_output)) {
+            const bool mine = my_node == node;
+            const T* block = grad_output + static_cast<size_t>(node) * K * L;
+            if (want_A) {
+                // right operand: lane (column k = 16 t + i, reduction index l = 4 s + q)
+                T right[L_STEPS][KT];
+#pragma unroll
+                for (int s = 0; s < L_STEPS; s++) {
+                    const int32_t l = 4 * s + q;
+#pragma unroll
+                    for (int t = 0; t < KT; t++) {
+                        const int32_t k = 16 * t + i;
+                        right[s][t] = load_or_zero(block, k * L + l, k < K && l < L);
+                    }
+                }
+#pragma unroll
+                for (int s = 0; s < L_STEPS; s++) {
+                    if (s < l_steps) {
+                        const T left = mine ? b_left[s] : T(0);
+#pragma unroll
+                        for (int t = 0; t < KT; t++) {
+                            acc_A[t] = M::mma(left, right[s][t], acc_A[t]);
+                        }
+                    }
+                }
+            }
+            if (want_B || want_W) {
+                // right operand: lane (column l = 16 t + i, reduction index k = 4 s + q)
+                T right[K_STEPS][NT];
+#pragma unroll
+                for (int s = 0; s < K_STEPS; s++) {
+                    const int32_t k = 4 * s + q;
+#pragma unroll
+                    for (int t = 0; t < NT; t++) {
+                        const int32_t l = 16 * t + i;
+                        right[s][t] = load_or_zero(block, k * L + l, k < K && l < L);
+                    }
+                }
+#pragma unroll
+                for (int s = 0; s < K_STEPS; s++) {
+                    if (s < k_steps) {
+                        const T left = mine ? a_left[s] : T(0);
+#pragma unroll
+                        for (int t = 0; t < NT; t++) {
+                            acc_B[t] = M::mma(left, right[s][t], acc_B[t]);
+                        }
+                    }
+                }
+            }
+        }
+        const unsigned long long later = __ballot(lane < n && my_node > node);
+        node = later == 0 ? -1 : __builtin_amdgcn_readlane(my_node, __ffsll(static_cast<long long>(later)) - 1);
+    }
+
+    // accumulators: lane (column = 16 t + i, rows = edges M::row(lane, r))
+    if (want_A) {
+#pragma unroll
+        for (int t = 0; t < KT; t++) {
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                const int32_t row = M::row(lane, r);
+                const int32_t k = 16 * t + i;
+                if (row < n && k < K) {
+                    grad_A[static_cast<size_t>(first_edge + row) * K + k] = acc_A[t][r];
+                }
+            }
+        }
+    }
+    if (want_B || want_W) {
+#pragma unroll
+        for (int t = 0; t < NT; t++) {
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                const int32_t row = M::row(lane, r);
+                const int32_t l = 16 * t + i;
+                const bool ok = row < n && l < L;
+                const size_t at = static_cast<size_t>(first_edge + row) * L + l;
+                if constexpr (WEIGHTED) {
+                    const int32_t sender = __shfl(my_sender, row);
+                    const bool gather = ok && in_bounds(sender, n_output);
+                    if (want_B) {
+                        const T weight = load_or_zero(W, static_cast<size_t>(sender) * L + l, gather);
+                        if (ok) {
+                            grad_B[at] = acc_B[t][r] * weight;
+                        }
+                    }
+                    if (want_W) {
+                        const T b = load_or_zero(B, at, ok);
+                        if (ok) {
+                            edge_W[at] = acc_B[t][r] * b;
+                        }
+                    }
+                } else if (ok) {
+                    grad_B[at] = acc_B[t][r];
+                }
+            }
+        }
+    }
+}
+
 // The same sum without any list in global memory: the workgroup's eight
 // wavefronts find the edges of their eight senders by one pass over the
 // sender index (sender_gather.hpp) and add the rows up, sixteen loads in
@@ -696,10 +882,39 @@ void launch_vjp(
             return shift;
         };
         const unsigned waves = static_cast<unsigned>(ceil_div(static_cast<size_t>(n_edges), CHUNK));
-        vjp_kernel<T, WEIGHTED><<<waves, WAVE, lds, stream>>>(
-            grad_A.data, grad_B.data, edge_W, grad_output.data, A.data, B.data, W, indices_W,
-            indices_output.data, n_edges, n_output, K, L, log2_ceil(K), log2_ceil(L)
-        );
+        if (K <= 32 && L <= 64) {
+            const unsigned groups = static_cast<unsigned>(ceil_div(static_cast<size_t>(n_edges), 16));
+            MainKernelTimer timer(stream);
+#define MOPS_LAUNCH_ROWS(KT, NT)                                                                   \
+    edge_rows_vjp_kernel<T, KT, NT, WEIGHTED><<<groups, WAVE, 0, stream>>>(                        \
+        grad_A.data, grad_B.data, edge_W, grad_output.data, A.data, B.data, W, indices_W,          \
+        indices_output.data, n_edges, n_output, K, L                                               \
+    )
+            if (K <= 16) {
+                if (L <= 16) {
+                    MOPS_LAUNCH_ROWS(1, 1);
+                } else if (L <= 32) {
+                    MOPS_LAUNCH_ROWS(1, 2);
+                } else {
+                    MOPS_LAUNCH_ROWS(1, 4);
+                }
+            } else {
+                if (L <= 16) {
+                    MOPS_LAUNCH_ROWS(2, 1);
+                } else if (L <= 32) {
+                    MOPS_LAUNCH_ROWS(2, 2);
+                } else {
+                    MOPS_LAUNCH_ROWS(2, 4);
+                }
+            }
+#undef MOPS_LAUNCH_ROWS
+        } else {
+            MainKernelTimer timer(stream);
+            vjp_kernel<T, WEIGHTED><<<waves, WAVE, lds, stream>>>(
+                grad_A.data, grad_B.data, edge_W, grad_output.data, A.data, B.data, W, indices_W,
+                indices_output.data, n_edges, n_output, K, L, log2_ceil(K), log2_ceil(L)
+            );
+        }
     }
 
     if (want_W && n_output > 0 && L > 0 && gather_in_kernel) {
