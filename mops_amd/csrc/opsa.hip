@@ -578,6 +578,27 @@ __global__ __launch_bounds__(WAVE) void edge_rows_vjp_kernel(
         a_left[s] = load_or_zero(A, static_cast<size_t>(my_edge) * K + k, my_edge >= 0 && k < K && (want_B || want_W));
     }
 
+    // factors of the results, per accumulator element (row = edge, column l = 16 t + i):
+    // asked for now, needed after the matrix products
+    T weight_out[NT][4];
+    T b_out[NT][4];
+    if constexpr (WEIGHTED) {
+#pragma unroll
+        for (int t = 0; t < NT; t++) {
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                const int32_t row = M::row(lane, r);
+                const int32_t l = 16 * t + i;
+                const bool ok = row < n && l < L;
+                const int32_t sender = __shfl(my_sender, row);
+                weight_out[t][r] = load_or_zero(
+                    W, static_cast<size_t>(sender) * L + l, ok && want_B && in_bounds(sender, n_output)
+                );
+                b_out[t][r] = load_or_zero(B, static_cast<size_t>(first_edge + row) * L + l, ok && want_W);
+            }
+        }
+    }
+
     typename M::Acc acc_A[KT];
     typename M::Acc acc_B[NT];
 #pragma unroll
@@ -672,19 +693,11 @@ __global__ __launch_bounds__(WAVE) void edge_rows_vjp_kernel(
                 const bool ok = row < n && l < L;
                 const size_t at = static_cast<size_t>(first_edge + row) * L + l;
                 if constexpr (WEIGHTED) {
-                    const int32_t sender = __shfl(my_sender, row);
-                    const bool gather = ok && in_bounds(sender, n_output);
-                    if (want_B) {
-                        const T weight = load_or_zero(W, static_cast<size_t>(sender) * L + l, gather);
-                        if (ok) {
-                            grad_B[at] = acc_B[t][r] * weight;
-                        }
+                    if (want_B && ok) {
+                        grad_B[at] = acc_B[t][r] * weight_out[t][r];
                     }
-                    if (want_W) {
-                        const T b = load_or_zero(B, at, ok);
-                        if (ok) {
-                            edge_W[at] = acc_B[t][r] * b;
-                        }
+                    if (want_W && ok) {
+                        edge_W[at] = acc_B[t][r] * b_out[t][r];
                     }
                 } else if (ok) {
                     grad_B[at] = acc_B[t][r];
