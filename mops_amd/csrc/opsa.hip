@@ -731,27 +731,32 @@ __global__ __launch_bounds__(GATHER_SENDERS* WAVE) void sum_by_sender_kernel(
         sum[c] = T(0);
         column[c] = min(lane + c * WAVE, L - 1);
     }
+    // rows in flight at a time: what 64 registers per lane hold
+    constexpr int ROWS = sizeof(T) == 8 ? Gather::STAGE / 2 : Gather::STAGE;
     auto on_stage = [&](int32_t my_edge, int32_t n) {
-        T values[Gather::STAGE][GATHER_COLUMNS];
+#pragma unroll 1 // one group of rows after the other, or the registers run out
+        for (int k0 = 0; k0 < Gather::STAGE; k0 += ROWS) {
+            T values[ROWS][GATHER_COLUMNS];
 #pragma unroll
-        for (int k = 0; k < Gather::STAGE; k++) {
-            // lanes beyond n hold -1: read row 0 and leave it out of the sum
-            const int32_t edge = max(__builtin_amdgcn_readlane(my_edge, k), 0);
-            const T* row = edge_W + static_cast<size_t>(edge) * L;
-#pragma unroll
-            for (int c = 0; c < GATHER_COLUMNS; c++) {
-                if (c * WAVE < L) {
-                    values[k][c] = row[column[c]];
-                }
-            }
-        }
-#pragma unroll
-        for (int k = 0; k < Gather::STAGE; k++) {
-            if (k < n) {
+            for (int k = 0; k < ROWS; k++) {
+                // lanes beyond n hold -1: read row 0 and leave it out of the sum
+                const int32_t edge = max(__builtin_amdgcn_readlane(my_edge, k0 + k), 0);
+                const T* row = edge_W + static_cast<size_t>(edge) * L;
 #pragma unroll
                 for (int c = 0; c < GATHER_COLUMNS; c++) {
                     if (c * WAVE < L) {
-                        sum[c] += values[k][c];
+                        values[k][c] = row[column[c]];
+                    }
+                }
+            }
+#pragma unroll
+            for (int k = 0; k < ROWS; k++) {
+                if (k0 + k < n) {
+#pragma unroll
+                    for (int c = 0; c < GATHER_COLUMNS; c++) {
+                        if (c * WAVE < L) {
+                            sum[c] += values[k][c];
+                        }
                     }
                 }
             }

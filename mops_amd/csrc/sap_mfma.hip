@@ -231,12 +231,15 @@ __device__ __forceinline__ void build_operands(
                     last = smallest;
                 }
             }
-            const int32_t index[3] = {entries.index_A[e], entries.index_B[e], entries.index_O[e]};
+            // (selects, not an array indexed by role: that would live in scratch memory)
+            auto index = [&](int role) {
+                return role == 0 ? entries.index_A[e] : (role == 1 ? entries.index_B[e] : entries.index_O[e]);
+            };
 #pragma unroll
             for (int w = 0; w < TARGETS; w++) {
                 if (targets[w].operand != nullptr) {
                     targets[w].operand[targets[w].shape.slot(
-                        index[targets[w].role[0]], index[targets[w].role[1]], index[targets[w].role[2]]
+                        index(targets[w].role[0]), index(targets[w].role[1]), index(targets[w].role[2])
                     )] = sum;
                 }
             }
