@@ -37,10 +37,11 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0  # MI355X, published
 ROTATE_BYTES = 320 * 1024 * 1024  # > 256 MB Infinity Cache
-# HBM bytes per launch of the main SAP f32 kernels from rocprofv3 --pmc runs
-# (FETCH_SIZE, WRITE_SIZE; see profiles/); None until measured for the
-# current kernels.
-MEASURED_TRAFFIC_BYTES = {"forward": None, "vjp": None}
+# HBM bytes per launch of the main SAP f32 kernels from two rocprofv3 --pmc
+# runs (profiles/all_ops_baseline_shapes_hbm_traffic.txt): FETCH_SIZE x 1.9993
+# (the factor a 64 MiB element-wise pass gives) + WRITE_SIZE x 1.0, in KiB.
+# forward: 1742.5 and 2500.0; vjp: 3099.8 and 2500.0.
+MEASURED_TRAFFIC_BYTES = {"forward": 6127000, "vjp": 8906000}
 
 
 def nbytes(arrays):
@@ -365,7 +366,10 @@ def main():
 
     # ---------------- roofline of the dominant kernel -----------------------
     # At this shape each call is one kernel (mops_amd/csrc/sap_mfma.hip), timed
-    # with HIP events recorded by the library on the stream the kernel runs on.
+    # with a pair of HIP events that the library records around every launch on
+    # the stream the kernel runs on (the pair itself costs about 1 us, which is
+    # inside the figure; consecutive eager calls from Python cannot be used, the
+    # interpreter needs longer per call than the kernel runs).
     library = bind_library_to_torch_stream(device)
     kernels = {}
     for kind, function, name in (
