@@ -15,6 +15,8 @@
 //   opsa / opsa_vjp        mops/src/opsa/cpu.tpp:9-53, 55-112
 //   opsaw / opsaw_vjp      mops/src/opsaw/cpu.tpp:9-54, 57-131
 //   sasaw / sasaw_vjp      mops/src/sasaw/cpu.tpp:8-72, 75-171
+//   hpe / sap / opsa _vjp_vjp   mops/src/hpe/cpu.tpp:275-539, sap/cpu.tpp:257-541,
+//                               opsa/cpu.tpp:114-246
 // The loop structure is the reference's: HPE and SAP re-lay the batch axis
 // into blocks of `lanes` rows ([block][feature][lane], lanes = 256 bits /
 // element size) and run an OpenMP loop over blocks with a serial remainder;
@@ -28,7 +30,9 @@
 // share code with it -- dense einsum / index_add formulations in numpy,
 // order-0 and order-1 polynomials, single-segment inputs that reduce to a
 // matrix product, finite differences and the adjoint identity for every vjp,
-// and empty segments. The compiled reference itself is not available to this
+// and empty segments; the second-order functions against central differences
+// of the (pinned) vjps through the adjoint identity, and against torch's double
+// backward of the dense formulations (golden vectors). The compiled reference itself is not available to this
 // build (it needs a CMake-generated header), so "equal to the reference" is
 // established through those mathematical pins, not by running it.
 //
@@ -250,6 +254,73 @@ void homogeneous_polynomial_evaluation_vjp(MOPS_HPE_VJP_PARAMS(MOPS_CXX_FIRST, M
     g.store(grad_A.data);
 }
 
+// Second-order functions (mops/src/hpe/cpu.tpp:275-460, sap/cpu.tpp:257-541,
+// opsa/cpu.tpp:114-246): the vjp of the vjp. Inputs are those of the vjp plus
+// the cotangents of its outputs (grad_grad_*); outputs are the cotangents of
+// grad_output (grad_grad_output) and of A, B (grad_*_2). They are written row
+// by row here (the reference blocks the batch axis as above, which changes
+// which rows share a vector register but not the order of any row's sums):
+// monomials / table entries / bucket members in ascending order, and inside
+// one of them the grad_grad_A term before the grad_grad_B term. A cotangent
+// that is not given counts as zero; the reference reads through the null
+// pointer in HPE in that case (hpe/cpu.tpp:367-388), which is not followed.
+template <typename scalar_t>
+void homogeneous_polynomial_evaluation_vjp_vjp(MOPS_HPE_VJP_VJP_PARAMS(MOPS_CXX_FIRST, MOPS_CXX_NEXT)) {
+    using T = scalar_t;
+    const size_t n = A.shape[0], nA = A.shape[1];
+    const size_t J = indices_A.shape[0], K = indices_A.shape[1];
+    if (K > 10) {
+        throw std::runtime_error(
+            "Only up to polynomial order 10 is supported at the moment. Please contact the "
+            "developers for more"
+        );
+    }
+    const bool have = grad_grad_A.data != nullptr;
+    const bool want_O = grad_grad_output.data != nullptr, want_A = grad_A_2.data != nullptr;
+    const int32_t* P = indices_A.data;
+#pragma omp parallel for
+    for (size_t i = 0; i < n; i++) {
+        const T* a = A.data + i * nA;
+        const T* gg = have ? grad_grad_A.data + i * nA : nullptr;
+        if (want_O) {
+            T sum = T(0);
+            for (size_t j = 0; have && j < J; j++) {
+                for (size_t f = 0; f < K; f++) {
+                    T term = C.data[j] * gg[P[j * K + f]];
+                    for (size_t k = 0; k < K; k++) {
+                        if (k != f) {
+                            term *= a[P[j * K + k]];
+                        }
+                    }
+                    sum += term;
+                }
+            }
+            grad_grad_output.data[i] = sum;
+        }
+        if (want_A) {
+            T* out = grad_A_2.data + i * nA;
+            std::fill(out, out + nA, T(0));
+            for (size_t j = 0; have && j < J; j++) {
+                const T base = C.data[j] * grad_output.data[i];
+                for (size_t f2 = 0; f2 < K; f2++) {
+                    for (size_t f = 0; f < K; f++) {
+                        if (f == f2) {
+                            continue;
+                        }
+                        T term = base * gg[P[j * K + f]];
+                        for (size_t k = 0; k < K; k++) {
+                            if (k != f && k != f2) {
+                                term *= a[P[j * K + k]];
+                            }
+                        }
+                        out[P[j * K + f2]] += term;
+                    }
+                }
+            }
+        }
+    }
+}
+
 // ---------------------------------------------------------------- SAP -------
 template <typename scalar_t>
 void sparse_accumulation_of_products(MOPS_SAP_PARAMS(MOPS_CXX_FIRST, MOPS_CXX_NEXT)) {
@@ -357,6 +428,56 @@ void sparse_accumulation_of_products_vjp(MOPS_SAP_VJP_PARAMS(MOPS_CXX_FIRST, MOP
     }
 }
 
+template <typename scalar_t>
+void sparse_accumulation_of_products_vjp_vjp(MOPS_SAP_VJP_VJP_PARAMS(MOPS_CXX_FIRST, MOPS_CXX_NEXT)) {
+    using T = scalar_t;
+    const size_t n = A.shape[0], nA = A.shape[1], nB = B.shape[1], nO = grad_output.shape[1];
+    const size_t K = C.shape[0];
+    const bool have_A = grad_grad_A.data != nullptr, have_B = grad_grad_B.data != nullptr;
+    const bool want_O = grad_grad_output.data != nullptr;
+    const bool want_A = grad_A_2.data != nullptr, want_B = grad_B_2.data != nullptr;
+    const int32_t *PA = indices_A.data, *PB = indices_B.data, *PO = indices_output.data;
+#pragma omp parallel for
+    for (size_t i = 0; i < n; i++) {
+        const T* a = A.data + i * nA;
+        const T* b = B.data + i * nB;
+        const T* g = grad_output.data + i * nO;
+        const T* gga = have_A ? grad_grad_A.data + i * nA : nullptr;
+        const T* ggb = have_B ? grad_grad_B.data + i * nB : nullptr;
+        T* ggo = want_O ? grad_grad_output.data + i * nO : nullptr;
+        T* ga2 = want_A ? grad_A_2.data + i * nA : nullptr;
+        T* gb2 = want_B ? grad_B_2.data + i * nB : nullptr;
+        if (want_O) {
+            std::fill(ggo, ggo + nO, T(0));
+        }
+        if (want_A) {
+            std::fill(ga2, ga2 + nA, T(0));
+        }
+        if (want_B) {
+            std::fill(gb2, gb2 + nB, T(0));
+        }
+        for (size_t k = 0; k < K; k++) {
+            const T c = C.data[k];
+            if (have_A) {
+                if (want_O) {
+                    ggo[PO[k]] += c * gga[PA[k]] * b[PB[k]];
+                }
+                if (want_B) {
+                    gb2[PB[k]] += c * gga[PA[k]] * g[PO[k]];
+                }
+            }
+            if (have_B) {
+                if (want_O) {
+                    ggo[PO[k]] += c * ggb[PB[k]] * a[PA[k]];
+                }
+                if (want_A) {
+                    ga2[PA[k]] += c * ggb[PB[k]] * g[PO[k]];
+                }
+            }
+        }
+    }
+}
+
 // --------------------------------------------------------------- OPSA -------
 template <typename scalar_t>
 void outer_product_scatter_add(MOPS_OPSA_PARAMS(MOPS_CXX_FIRST, MOPS_CXX_NEXT)) {
@@ -408,6 +529,61 @@ void outer_product_scatter_add_vjp(MOPS_OPSA_VJP_PARAMS(MOPS_CXX_FIRST, MOPS_CXX
                 }
                 if (want_B) {
                     grad_B.data[j * L + l] += g[k * L + l] * a[k];
+                }
+            }
+        }
+    }
+}
+
+template <typename scalar_t>
+void outer_product_scatter_add_vjp_vjp(MOPS_OPSA_VJP_VJP_PARAMS(MOPS_CXX_FIRST, MOPS_CXX_NEXT)) {
+    using T = scalar_t;
+    const size_t J = A.shape[0], K = A.shape[1], L = B.shape[1], n_out = grad_output.shape[0];
+    const bool have_A = grad_grad_A.data != nullptr, have_B = grad_grad_B.data != nullptr;
+    const bool want_O = grad_grad_output.data != nullptr;
+    const bool want_A = grad_A_2.data != nullptr, want_B = grad_B_2.data != nullptr;
+    if (want_A) {
+        std::fill(grad_A_2.data, grad_A_2.data + J * K, T(0));
+    }
+    if (want_B) {
+        std::fill(grad_B_2.data, grad_B_2.data + J * L, T(0));
+    }
+    if (want_O) {
+        std::fill(grad_grad_output.data, grad_grad_output.data + n_out * K * L, T(0));
+    }
+    Buckets buckets = bucket_rows(indices_output.data, J, n_out);
+#pragma omp parallel for
+    for (size_t i = 0; i < n_out; i++) {
+        T* ggo = want_O ? grad_grad_output.data + i * K * L : nullptr;
+        const T* g = grad_output.data + i * K * L;
+        for (size_t p = buckets.begin[i]; p < buckets.begin[i + 1]; p++) {
+            const size_t j = buckets.rows[p];
+            const T* a = A.data + j * K;
+            const T* b = B.data + j * L;
+            if (have_A) {
+                const T* gga = grad_grad_A.data + j * K;
+                for (size_t k = 0; k < K; k++) {
+                    for (size_t l = 0; l < L; l++) {
+                        if (want_O) {
+                            ggo[k * L + l] += gga[k] * b[l];
+                        }
+                        if (want_B) {
+                            grad_B_2.data[j * L + l] += gga[k] * g[k * L + l];
+                        }
+                    }
+                }
+            }
+            if (have_B) {
+                const T* ggb = grad_grad_B.data + j * L;
+                for (size_t k = 0; k < K; k++) {
+                    for (size_t l = 0; l < L; l++) {
+                        if (want_O) {
+                            ggo[k * L + l] += ggb[l] * a[k];
+                        }
+                        if (want_A) {
+                            grad_A_2.data[j * K + k] += ggb[l] * g[k * L + l];
+                        }
+                    }
                 }
             }
         }
@@ -568,6 +744,9 @@ void sparse_accumulation_scatter_add_with_weights_vjp(MOPS_SASAW_VJP_PARAMS(MOPS
     }
 }
 
+// No second-order function exists for the two weighted operations
+// (mops/src/opsaw/cpu.tpp:133-150, mops/src/sasaw/cpu.tpp:173-194: "Not implemented").
+
 } // namespace oracle
 
 // ---- C entry points ---------------------------------------------------------
@@ -629,6 +808,9 @@ ORACLE_C_DEFINE_BOTH(outer_product_scatter_add_with_weights, MOPS_OPSAW_PARAMS)
 ORACLE_C_DEFINE_BOTH(outer_product_scatter_add_with_weights_vjp, MOPS_OPSAW_VJP_PARAMS)
 ORACLE_C_DEFINE_BOTH(sparse_accumulation_scatter_add_with_weights, MOPS_SASAW_PARAMS)
 ORACLE_C_DEFINE_BOTH(sparse_accumulation_scatter_add_with_weights_vjp, MOPS_SASAW_VJP_PARAMS)
+ORACLE_C_DEFINE_BOTH(homogeneous_polynomial_evaluation_vjp_vjp, MOPS_HPE_VJP_VJP_PARAMS)
+ORACLE_C_DEFINE_BOTH(sparse_accumulation_of_products_vjp_vjp, MOPS_SAP_VJP_VJP_PARAMS)
+ORACLE_C_DEFINE_BOTH(outer_product_scatter_add_vjp_vjp, MOPS_OPSA_VJP_VJP_PARAMS)
 
 ORACLE_EXPORT const char* mops_oracle_get_last_error_message(void) { return LAST_ERROR.c_str(); }
 

@@ -8,7 +8,10 @@ by code that shares nothing with the oracle or the HIP kernels:
 * outputs: dense float64 formulations written with `torch.einsum` /
   `index_add_` (the definitions quoted in the docstrings below);
 * gradients: `torch.autograd.grad` of those formulations against the stored
-  `grad_output` (float64), i.e. torch's differentiation rules, not ours.
+  `grad_output` (float64), i.e. torch's differentiation rules, not ours;
+* second order (HPE, SAP, OPSA, the operations that have a vjp_vjp): the
+  stored cotangents `grad_grad_*` are contracted with those gradients and
+  differentiated once more by torch with respect to `grad_output`, A and B.
 
 Inputs are float64 values that are exactly representable in float32
 (multiples of 1/64), so the same fixture serves both precisions; expected
@@ -138,10 +141,32 @@ def main():
         rng = np.random.default_rng(sum(name.encode()) * 7919)
         grad_output = grid(rng, tuple(output.shape))
         wanted = [tensors[key] for key in DIFFERENTIABLE[op]]
-        if output.requires_grad and output.numel() > 0 and all(t.numel() > 0 for t in wanted):
-            gradients = torch.autograd.grad(output, wanted, torch.from_numpy(grad_output), allow_unused=True)
+        upstream = torch.from_numpy(grad_output).requires_grad_(True)
+        live = output.requires_grad and output.numel() > 0 and all(t.numel() > 0 for t in wanted)
+        if live:
+            gradients = torch.autograd.grad(output, wanted, upstream, allow_unused=True, create_graph=True)
         else:
             gradients = [torch.zeros_like(t) for t in wanted]
+        if op in ("hpe", "sap", "opsa"):
+            cotangents = [grid(rng, tuple(t.shape)) for t in wanted]
+            contracted = sum(
+                (torch.from_numpy(c) * g).sum() for c, g in zip(cotangents, gradients) if g is not None
+            )
+            targets = [upstream] + wanted
+            if live and isinstance(contracted, torch.Tensor) and contracted.requires_grad:
+                second = torch.autograd.grad(contracted, targets, allow_unused=True)
+            else:
+                second = [None] * len(targets)
+            second = [torch.zeros_like(t) if g is None else g.detach().clone() for t, g in zip(targets, second)]
+            for g in second:
+                # torch differentiates prod() through a division: what should be an exact
+                # zero (second derivative of an order-1 polynomial) comes out as ~1e-16
+                g[g.abs() < 1e-12] = 0.0
+            for key, c in zip(DIFFERENTIABLE[op], cotangents):
+                arrays[f"{name}/in/grad_grad_{key}"] = c
+            arrays[f"{name}/out/grad_grad_output"] = second[0].detach().numpy()
+            for key, g in zip(DIFFERENTIABLE[op], second[1:]):
+                arrays[f"{name}/out/grad_{key}_2"] = g.detach().numpy()
         for key, value in case.items():
             arrays[f"{name}/in/{key}"] = np.asarray(value)
         arrays[f"{name}/in/grad_output"] = grad_output

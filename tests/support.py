@@ -272,6 +272,64 @@ def cpu_vjp(library, op, case, wanted=None):
     return dict(zip(op.differentiable, gradients))
 
 
+SECOND_ORDER = ["hpe", "sap", "opsa"]  # operations that have a vjp_vjp
+
+
+def add_cotangents(case, op, seed=99):
+    """Adds grad_grad_<input> (cotangents of the vjp's outputs) to ``case``."""
+    rng = np.random.default_rng(seed)
+    for name in OPS[op].differentiable:
+        case["grad_grad_" + name] = rng.normal(size=case[name].shape).astype(case[name].dtype)
+    return case
+
+
+def _vjp_vjp_arguments(op, case, have, wanted, empty_like):
+    """ABI order: grad_grad_output, grad_<x>_2 ..., grad_grad_<x> ..., grad_output, inputs."""
+    have = op.differentiable if have is None else have
+    wanted = ["grad_output"] + op.differentiable if wanted is None else wanted
+    outputs = {"grad_output": empty_like(case["grad_output"]) if "grad_output" in wanted else None}
+    for name in op.differentiable:
+        outputs[name] = empty_like(case[name]) if name in wanted else None
+    cotangents = [case["grad_grad_" + name] if name in have else None for name in op.differentiable]
+    arguments = (
+        [outputs["grad_output"]]
+        + [outputs[name] for name in op.differentiable]
+        + cotangents
+        + [case["grad_output"]]
+        + [case[name] for name in op.inputs]
+    )
+    return outputs, arguments
+
+
+def cpu_vjp_vjp(library, op, case, have=None, wanted=None):
+    """Second-order function; returns {"grad_output": grad_grad_output, input name: grad_<name>_2}.
+
+    ``have``: the inputs whose cotangent grad_grad_<name> is passed (others null);
+    ``wanted``: which of "grad_output" and the input names are computed.
+    """
+    op = OPS[op]
+    outputs, arguments = _vjp_vjp_arguments(
+        op, case, have, wanted, lambda x: np.full(x.shape, np.nan, dtype=x.dtype)
+    )
+    library.call(op.function + "_vjp_vjp", *arguments)
+    return outputs
+
+
+def hip_vjp_vjp(op, case_on_device, have=None, wanted=None):
+    import torch
+
+    from mops_amd._c_lib import device_library
+
+    op = OPS[op]
+    outputs, arguments = _vjp_vjp_arguments(
+        op, case_on_device, have, wanted, lambda x: torch.full_like(x, float("nan"))
+    )
+    library = device_library()
+    _bind_stream(library, case_on_device["A"].device)
+    library.call(op.function + "_vjp_vjp", *arguments)
+    return outputs
+
+
 def to_device(case, device):
     import torch
 

@@ -61,6 +61,11 @@ def test_oracle_against_golden(oracle, name, dtype):
     gradients = support.cpu_vjp(oracle, op, case)
     for key in OPS[op].differentiable:
         assert_close(gradients[key], expected["grad_" + key], dtype, f"{name} grad_{key}", 4.0)
+    if op in support.SECOND_ORDER:
+        second = support.cpu_vjp_vjp(oracle, op, case)
+        assert_close(second["grad_output"], expected["grad_grad_output"], dtype, f"{name} grad_grad_output", 8.0)
+        for key in OPS[op].differentiable:
+            assert_close(second[key], expected[f"grad_{key}_2"], dtype, f"{name} grad_{key}_2", 8.0)
 
 
 @pytest.mark.gpu
@@ -75,3 +80,10 @@ def test_hip_against_golden(device, name, dtype):
     gradients = support.hip_vjp(op, case)
     for key in OPS[op].differentiable:
         assert_close(gradients[key].cpu().numpy(), expected["grad_" + key], dtype, f"{name} grad_{key}", 4.0)
+    if op in support.SECOND_ORDER:
+        second = support.hip_vjp_vjp(op, case)
+        assert_close(
+            second["grad_output"].cpu().numpy(), expected["grad_grad_output"], dtype, f"{name} grad_grad_output", 8.0
+        )
+        for key in OPS[op].differentiable:
+            assert_close(second[key].cpu().numpy(), expected[f"grad_{key}_2"], dtype, f"{name} grad_{key}_2", 8.0)

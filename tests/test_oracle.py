@@ -10,6 +10,9 @@ term, a swapped index or a transposed operand fails at least one of them:
   segment = one matrix product, identity-like tables);
 * every vjp against central finite differences of the oracle's own forward
   and against the adjoint identity <vjp(g), dx> = <g, J dx> using linearity;
+* the second-order functions (vjp_vjp of HPE, SAP, OPSA) against central
+  differences of the pinned vjps, against the forward pass by linearity, and
+  with absent cotangents against zero cotangents;
 * empty segments give exact zeros; unsorted scatter indices are accepted;
 * the committed golden vectors (tests/golden).
 """
@@ -220,3 +223,70 @@ def test_first_occurrences_definition(oracle):
     oracle.cdll.mops_oracle_first_occurrences(index.ctypes.data, len(index), 6, out.ctypes.data)
     assert out[:6].tolist() == [-1, 0, -1, -1, 2, -1]
     assert out[6:].tolist() == [-1, 2, -1, -1, 3, -1]
+
+
+# --------------------------------------------------------------------------
+# second order: the vjp of the vjp
+# --------------------------------------------------------------------------
+def _contracted_vjp(oracle, op, case):
+    """s(grad_output, A, B) = sum over inputs of <grad_grad_x, vjp_x>, in float64."""
+    gradients = cpu_vjp(oracle, op, case)
+    return sum(np.sum(case["grad_grad_" + name] * gradients[name]) for name in OPS[op].differentiable)
+
+
+@pytest.mark.parametrize("op", support.SECOND_ORDER)
+def test_vjp_vjp_matches_finite_differences_of_the_vjp(oracle, op):
+    """grad_grad_output, grad_A_2, grad_B_2 are the derivatives of
+    s = <grad_grad_A, grad_A> + <grad_grad_B, grad_B> with respect to
+    grad_output, A and B; s is evaluated with the (pinned) vjp."""
+    case = support.add_cotangents(SMALL[op](5, np.float64), op)
+    second = support.cpu_vjp_vjp(oracle, op, case)
+    h = 1e-6
+    rng = np.random.default_rng(13)
+    for name in ["grad_output"] + OPS[op].differentiable:
+        x = case[name]
+        assert second[name].shape == x.shape
+        for _ in range(12):
+            position = tuple(rng.integers(0, s) for s in x.shape)
+            saved = x[position]
+            x[position] = saved + h
+            plus = _contracted_vjp(oracle, op, case)
+            x[position] = saved - h
+            minus = _contracted_vjp(oracle, op, case)
+            x[position] = saved
+            numeric = (plus - minus) / (2 * h)
+            analytic = second[name][position]
+            assert abs(numeric - analytic) <= 2e-6 * max(1.0, abs(numeric)), (op, name, position)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("op", ["sap", "opsa"])
+def test_grad_grad_output_is_two_forward_passes(oracle, op, dtype):
+    """Bilinear operations: grad_grad_output = f(grad_grad_A, B) + f(A, grad_grad_B)."""
+    case = support.add_cotangents(SMALL[op](6, dtype), op)
+    second = support.cpu_vjp_vjp(oracle, op, case)
+    first = dict(case, A=case["grad_grad_A"])
+    other = dict(case, B=case["grad_grad_B"])
+    expected = cpu_forward(oracle, op, first).astype(np.float64) + cpu_forward(oracle, op, other)
+    assert_close(second["grad_output"], expected, dtype, op, 4.0)
+
+
+@pytest.mark.parametrize("op", support.SECOND_ORDER)
+def test_vjp_vjp_absent_cotangents_and_skipped_outputs(oracle, op):
+    case = support.add_cotangents(SMALL[op](7, np.float64), op)
+    everything = support.cpu_vjp_vjp(oracle, op, case)
+    names = OPS[op].differentiable
+    # an absent cotangent counts as zero
+    for absent in names:
+        have = [n for n in names if n != absent]
+        zeroed = dict(case)
+        zeroed["grad_grad_" + absent] = np.zeros_like(case["grad_grad_" + absent])
+        expected = support.cpu_vjp_vjp(oracle, op, zeroed)
+        actual = support.cpu_vjp_vjp(oracle, op, case, have=have)
+        for key in expected:
+            assert np.array_equal(actual[key], expected[key]), (op, absent, key)
+    # every output can be computed alone and gives the same values
+    for alone in ["grad_output"] + names:
+        actual = support.cpu_vjp_vjp(oracle, op, case, wanted=[alone])
+        assert np.array_equal(actual[alone], everything[alone]), (op, alone)
+        assert all(value is None for key, value in actual.items() if key != alone)
