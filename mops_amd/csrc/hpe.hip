@@ -28,6 +28,7 @@
 #include "checks.hpp"
 #include "device_common.hpp"
 #include "index_validation.hpp"
+#include "elementwise.hpp"
 #include "runtime.hpp"
 
 namespace mops::amd {
@@ -430,6 +431,198 @@ __global__ __launch_bounds__(256) void vjp_global_kernel(
     }
 }
 
+// ---------------------------------------------------------------------------
+// Second order: the vjp of the vjp (semantics of mops/src/hpe/cpu.tpp:275-539).
+//
+//   grad_grad_O[i]      = sum_j C[j] sum_f gg[i, P[j, f]] prod_{k != f} A[i, P[j, k]]
+//   grad_A_2[i, P[j,f2]] += gO[i] C[j] sum_{f != f2} gg[i, P[j, f]] prod_{k != f, f2} A[i, P[j, k]]
+//
+// with gg = grad_grad_A. Same work split as vjp_kernel: one wavefront per
+// workgroup, thread (r, g) walks the monomials j = g, g + G, ... of row r and
+// adds into private accumulators in LDS, which are then combined in group
+// order. LDS: a[nA][R] gg[nA][R] accumulator[G][nA][R] partial[G][R].
+// Either output may be null.
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(WAVE) void vjp_vjp_kernel(
+    T* __restrict__ grad_grad_output,
+    T* __restrict__ grad_A_2,
+    const T* __restrict__ grad_grad_A,
+    const T* __restrict__ grad_output,
+    const T* __restrict__ A,
+    const T* __restrict__ C,
+    const int32_t* __restrict__ P,
+    int32_t n_rows,
+    int32_t nA,
+    int32_t n_monomials,
+    int32_t order,
+    int32_t R
+) {
+    extern __shared__ __align__(16) unsigned char lds_bytes[];
+    T* a_stage = reinterpret_cast<T*>(lds_bytes);
+    T* gg_stage = a_stage + static_cast<size_t>(nA) * R;
+    T* accumulator = gg_stage + static_cast<size_t>(nA) * R;
+    T* partial = accumulator + static_cast<size_t>(nA) * WAVE;
+
+    const int tid = threadIdx.x;
+    const int G = WAVE / R;
+    const int r = tid % R;
+    const int g = tid / R;
+    const int32_t row0 = blockIdx.x * R;
+    const int32_t rows = min(R, n_rows - row0);
+    const bool want_O = grad_grad_output != nullptr;
+    const bool want_A = grad_A_2 != nullptr;
+
+    const T* a_src = A + static_cast<size_t>(row0) * nA;
+    const T* gg_src = grad_grad_A + static_cast<size_t>(row0) * nA;
+    for (int32_t i = tid; i < rows * nA; i += WAVE) {
+        const int32_t row = i / nA;
+        a_stage[(i - row * nA) * R + row] = a_src[i];
+        gg_stage[(i - row * nA) * R + row] = gg_src[i];
+    }
+    for (int32_t i = tid; i < nA * WAVE; i += WAVE) {
+        accumulator[i] = T(0);
+    }
+    __syncthreads();
+
+    T sum = T(0);
+    if (r < rows) {
+        T* mine = accumulator + static_cast<size_t>(g) * nA * R + r;
+        const T upstream = grad_output[row0 + r];
+        auto value_of = [&](const T* stage, int32_t feature) {
+            return in_bounds(feature, nA) ? stage[feature * R + r] : T(0);
+        };
+        for (int32_t j = g; j < n_monomials; j += G) {
+            const int32_t* factors = P + static_cast<size_t>(j) * order;
+            const T coefficient = C[j];
+            if (want_O) {
+                for (int32_t f = 0; f < order; f++) {
+                    T term = coefficient * value_of(gg_stage, factors[f]);
+                    for (int32_t k = 0; k < order; k++) {
+                        if (k != f) {
+                            term *= value_of(a_stage, factors[k]);
+                        }
+                    }
+                    sum += term;
+                }
+            }
+            if (want_A) {
+                const T base = coefficient * upstream;
+                for (int32_t f2 = 0; f2 < order; f2++) {
+                    const int32_t target = factors[f2];
+                    if (!in_bounds(target, nA)) {
+                        continue;
+                    }
+                    T total = T(0);
+                    for (int32_t f = 0; f < order; f++) {
+                        if (f == f2) {
+                            continue;
+                        }
+                        T term = base * value_of(gg_stage, factors[f]);
+                        for (int32_t k = 0; k < order; k++) {
+                            if (k != f && k != f2) {
+                                term *= value_of(a_stage, factors[k]);
+                            }
+                        }
+                        total += term;
+                    }
+                    mine[target * R] += total;
+                }
+            }
+        }
+    }
+    partial[g * R + r] = sum;
+    __syncthreads();
+
+    if (want_O && tid < rows) {
+        T total = T(0);
+        for (int group = 0; group < G; group++) {
+            total += partial[group * R + tid];
+        }
+        grad_grad_output[row0 + tid] = total;
+    }
+    if (want_A) {
+        T* dst = grad_A_2 + static_cast<size_t>(row0) * nA;
+        for (int32_t i = tid; i < rows * nA; i += WAVE) {
+            const int32_t row = i / nA;
+            const int32_t feature = i - row * nA;
+            T total = T(0);
+            for (int group = 0; group < G; group++) {
+                total += accumulator[(static_cast<size_t>(group) * nA + feature) * R + row];
+            }
+            dst[i] = total;
+        }
+    }
+}
+
+// The same with everything in global memory, one thread per batch row, for
+// feature counts whose tiles do not fit in LDS.
+template <typename T>
+__global__ __launch_bounds__(256) void vjp_vjp_global_kernel(
+    T* grad_grad_output,
+    T* grad_A_2,
+    const T* __restrict__ grad_grad_A,
+    const T* __restrict__ grad_output,
+    const T* __restrict__ A,
+    const T* __restrict__ C,
+    const int32_t* __restrict__ P,
+    int32_t n_rows,
+    int32_t nA,
+    int32_t n_monomials,
+    int32_t order
+) {
+    const int32_t row = blockIdx.x * blockDim.x + threadIdx.x;
+    if (row >= n_rows) {
+        return;
+    }
+    const T* a_row = A + static_cast<size_t>(row) * nA;
+    const T* gg_row = grad_grad_A + static_cast<size_t>(row) * nA;
+    T* out_row = grad_A_2 != nullptr ? grad_A_2 + static_cast<size_t>(row) * nA : nullptr;
+    if (out_row != nullptr) {
+        for (int32_t feature = 0; feature < nA; feature++) {
+            out_row[feature] = T(0);
+        }
+    }
+    auto value_of = [&](const T* values, int32_t feature) {
+        return in_bounds(feature, nA) ? values[feature] : T(0);
+    };
+    const T upstream = grad_output[row];
+    T sum = T(0);
+    for (int32_t j = 0; j < n_monomials; j++) {
+        const int32_t* factors = P + static_cast<size_t>(j) * order;
+        for (int32_t f2 = 0; f2 < order; f2++) {
+            // f2 = the factor differentiated last; the f2-th term of the first
+            // sum is the product with gg in place of that factor
+            T first = C[j] * value_of(gg_row, factors[f2]);
+            T second = T(0);
+            for (int32_t k = 0; k < order; k++) {
+                if (k != f2) {
+                    first *= value_of(a_row, factors[k]);
+                }
+            }
+            sum += first;
+            if (out_row != nullptr && in_bounds(factors[f2], nA)) {
+                for (int32_t f = 0; f < order; f++) {
+                    if (f == f2) {
+                        continue;
+                    }
+                    T term = C[j] * upstream * value_of(gg_row, factors[f]);
+                    for (int32_t k = 0; k < order; k++) {
+                        if (k != f && k != f2) {
+                            term *= value_of(a_row, factors[k]);
+                        }
+                    }
+                    second += term;
+                }
+                out_row[factors[f2]] += second;
+            }
+        }
+    }
+    if (grad_grad_output != nullptr) {
+        grad_grad_output[row] = sum;
+    }
+}
+
 // Rows per workgroup: as many as possible (fewer table reads per row) while
 // the launch still has about a thousand workgroups and the tiles fit in LDS.
 // Returns 0 when even R = 1 does not fit.
@@ -585,10 +778,60 @@ void homogeneous_polynomial_evaluation_vjp(MOPS_HPE_VJP_PARAMS(MOPS_CXX_FIRST, M
     finish_call(operation);
 }
 
+// Second order. The reference has it on the host only
+// (mops/src/hpe/cpu.tpp:275-539; device: "Not implemented",
+// mops/src/hpe/hpe.cu:402-413) and reads through a null grad_grad_A
+// (cpu.tpp:367-388); here a cotangent that is not given counts as zero.
 template <typename scalar_t>
 void homogeneous_polynomial_evaluation_vjp_vjp(MOPS_HPE_VJP_VJP_PARAMS(MOPS_CXX_FIRST, MOPS_CXX_NEXT)) {
-    // same state as the reference's device path (mops/src/hpe/hpe.cu:402-413)
-    throw std::runtime_error("Not implemented");
+    using namespace mops::amd;
+    const char* operation = "cuda_homogeneous_polynomial_evaluation_vjp_vjp";
+    checks::Validator validator(operation);
+    checks::hpe_vjp_vjp(validator, grad_grad_output, grad_A_2, grad_grad_A, grad_output, A, C, indices_A);
+    if (grad_grad_output.data == nullptr && grad_A_2.data == nullptr) {
+        return;
+    }
+    validate_gather_index(indices_A, A.shape[1], "indices_A", operation);
+
+    const int32_t n_rows = narrow_i32(A.shape[0], "A.shape[0]");
+    const int32_t nA = narrow_i32(A.shape[1], "A.shape[1]");
+    const int32_t n_monomials = narrow_i32(indices_A.shape[0], "indices_A.shape[0]");
+    const int32_t order = narrow_i32(indices_A.shape[1], "indices_A.shape[1]");
+    if (n_rows == 0) {
+        return;
+    }
+    hipStream_t stream = current_stream();
+    if (grad_grad_A.data == nullptr || nA == 0) {
+        if (grad_grad_output.data != nullptr) {
+            fill_zero<scalar_t>(grad_grad_output.data, static_cast<size_t>(n_rows), stream);
+        }
+        if (grad_A_2.data != nullptr) {
+            fill_zero<scalar_t>(grad_A_2.data, static_cast<size_t>(n_rows) * nA, stream);
+        }
+        finish_call(operation);
+        return;
+    }
+    // LDS: 2 R rows (A and grad_grad_A), WAVE accumulator rows, WAVE partial sums
+    const size_t fixed_bytes = (static_cast<size_t>(nA) + 1) * WAVE * sizeof(scalar_t);
+    auto lds_for = [&](int rows) { return fixed_bytes + 2 * static_cast<size_t>(nA) * rows * sizeof(scalar_t); };
+    int R = 64;
+    while (R > 1 && (static_cast<size_t>(n_rows) / R < 1024 || lds_for(R) > LDS_BUDGET)) {
+        R >>= 1;
+    }
+    if (lds_for(R) <= LDS_BUDGET) {
+        const unsigned blocks = static_cast<unsigned>(ceil_div(static_cast<size_t>(n_rows), R));
+        vjp_vjp_kernel<scalar_t><<<blocks, WAVE, lds_for(R), stream>>>(
+            grad_grad_output.data, grad_A_2.data, grad_grad_A.data, grad_output.data, A.data, C.data,
+            indices_A.data, n_rows, nA, n_monomials, order, R
+        );
+    } else {
+        const unsigned blocks = static_cast<unsigned>(ceil_div(static_cast<size_t>(n_rows), 256));
+        vjp_vjp_global_kernel<scalar_t><<<blocks, 256, 0, stream>>>(
+            grad_grad_output.data, grad_A_2.data, grad_grad_A.data, grad_output.data, A.data, C.data,
+            indices_A.data, n_rows, nA, n_monomials, order
+        );
+    }
+    finish_call(operation);
 }
 
 MOPS_CXX_INSTANTIATE(homogeneous_polynomial_evaluation, MOPS_HPE_PARAMS)

@@ -39,6 +39,7 @@
 #include "first_occurrences.hpp"
 #include "index_validation.hpp"
 #include "mfma.hpp"
+#include "elementwise.hpp"
 #include "runtime.hpp"
 #include "segment_walk.hpp"
 #include "sender_buckets.hpp"
@@ -977,10 +978,61 @@ void outer_product_scatter_add_vjp(MOPS_OPSA_VJP_PARAMS(MOPS_CXX_FIRST, MOPS_CXX
     );
 }
 
+// Second order (semantics of mops/src/opsa/cpu.tpp:114-246; the reference's
+// device path has none, mops/src/opsa/opsa.cu:305-318). The operation is
+// bilinear, so every output is a first-order call with one operand replaced
+// by a cotangent:
+//   grad_grad_output = forward(grad_grad_A, B) + forward(A, grad_grad_B)
+//   grad_A_2         = vjp's grad_A with B := grad_grad_B
+//   grad_B_2         = vjp's grad_B with A := grad_grad_A
+// A cotangent that is not given counts as zero.
 template <typename scalar_t>
 void outer_product_scatter_add_vjp_vjp(MOPS_OPSA_VJP_VJP_PARAMS(MOPS_CXX_FIRST, MOPS_CXX_NEXT)) {
-    // same state as the reference's device path (mops/src/opsa/opsa.cu:305-318)
-    throw std::runtime_error("Not implemented");
+    using namespace mops::amd;
+    const char* operation = "cuda_outer_product_scatter_add_vjp_vjp";
+    checks::Validator validator(operation);
+    checks::opsa_vjp_vjp(
+        validator, grad_grad_output, grad_A_2, grad_B_2, grad_grad_A, grad_grad_B, grad_output, A, B,
+        indices_output
+    );
+    validate_scatter_index(indices_output, grad_output.shape[0], "indices_output", operation);
+    const bool have_A = grad_grad_A.data != nullptr, have_B = grad_grad_B.data != nullptr;
+    const Tensor<scalar_t, 2> nothing{nullptr, {0, 0}};
+    hipStream_t stream = current_stream();
+    const size_t output_count = grad_output.shape[0] * grad_output.shape[1] * grad_output.shape[2];
+
+    if (grad_grad_output.data != nullptr) {
+        if (have_A) {
+            ::mops::cuda::outer_product_scatter_add<scalar_t>(grad_grad_output, grad_grad_A, B, indices_output);
+        }
+        if (have_A && have_B) {
+            StreamTemporary<scalar_t> second(output_count, stream);
+            ::mops::cuda::outer_product_scatter_add<scalar_t>(
+                Tensor<scalar_t, 3>{second.data(), {grad_output.shape[0], grad_output.shape[1], grad_output.shape[2]}},
+                A, grad_grad_B, indices_output
+            );
+            add_in_place<scalar_t>(grad_grad_output.data, second.data(), output_count, stream);
+        } else if (have_B) {
+            ::mops::cuda::outer_product_scatter_add<scalar_t>(grad_grad_output, A, grad_grad_B, indices_output);
+        } else if (!have_A) {
+            fill_zero<scalar_t>(grad_grad_output.data, output_count, stream);
+        }
+    }
+    if (grad_A_2.data != nullptr) {
+        if (have_B) {
+            ::mops::cuda::outer_product_scatter_add_vjp<scalar_t>(grad_A_2, nothing, grad_output, A, grad_grad_B, indices_output);
+        } else {
+            fill_zero<scalar_t>(grad_A_2.data, A.shape[0] * A.shape[1], stream);
+        }
+    }
+    if (grad_B_2.data != nullptr) {
+        if (have_A) {
+            ::mops::cuda::outer_product_scatter_add_vjp<scalar_t>(nothing, grad_B_2, grad_output, grad_grad_A, B, indices_output);
+        } else {
+            fill_zero<scalar_t>(grad_B_2.data, B.shape[0] * B.shape[1], stream);
+        }
+    }
+    finish_call(operation);
 }
 
 template <typename scalar_t>

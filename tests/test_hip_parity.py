@@ -199,3 +199,61 @@ def test_baseline_configuration(oracle, device, op, config, dtype, build):
         scaled["A"] = on_device["A"] * 2.0
         order = case["indices_A"].shape[1]
         assert_close(hip_forward(op, scaled).cpu().numpy(), out * 2.0**order, dtype, "hpe homogeneity")
+
+
+# ---- second order: vjp_vjp of HPE, SAP, OPSA -------------------------------
+SECOND = [(op, name) for op in support.SECOND_ORDER for name in CASES[op]]
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=["f32", "f64"])
+@pytest.mark.parametrize("op,name", SECOND)
+def test_vjp_vjp(oracle, device, op, name, dtype):
+    case = support.add_cotangents(CASES[op][name](606, dtype), op)
+    expected = support.cpu_vjp_vjp(oracle, op, case)
+    actual = support.hip_vjp_vjp(op, to_device(case, device))
+    for key in ["grad_output"] + OPS[op].differentiable:
+        assert_close(actual[key].cpu().numpy(), expected[key], dtype, f"{op}/{name} second order {key}", 2.0)
+
+
+@pytest.mark.parametrize("op", support.SECOND_ORDER)
+def test_vjp_vjp_absent_cotangents_and_skipped_outputs(oracle, device, op):
+    case = support.add_cotangents(CASES[op]["ragged"](707, np.float64), op)
+    on_device = to_device(case, device)
+    names = OPS[op].differentiable
+    outputs = ["grad_output"] + names
+    full = {k: v.cpu().numpy() for k, v in support.hip_vjp_vjp(op, on_device).items()}
+    for r in range(len(names) + 1):
+        for have in itertools.combinations(names, r):
+            expected = support.cpu_vjp_vjp(oracle, op, case, have=list(have))
+            actual = support.hip_vjp_vjp(op, on_device, have=list(have))
+            for key in outputs:
+                assert_close(actual[key].cpu().numpy(), expected[key], np.float64, f"{op} have={have} {key}", 2.0)
+    for alone in outputs:
+        actual = support.hip_vjp_vjp(op, on_device, wanted=[alone])
+        assert np.array_equal(actual[alone].cpu().numpy(), full[alone]), (op, alone)
+        assert all(value is None for key, value in actual.items() if key != alone)
+
+
+@pytest.mark.parametrize("op,config,dtype,build", [b for b in BASELINE if b[0] in support.SECOND_ORDER],
+                         ids=[f"c{c}-{o}-{np.dtype(t).name}" for o, c, t, _ in BASELINE if o in support.SECOND_ORDER])
+def test_vjp_vjp_baseline_configuration(oracle, device, op, config, dtype, build):
+    case = support.add_cotangents(build(dtype), op)
+    on_device = to_device(case, device)
+    expected = support.cpu_vjp_vjp(oracle, op, case)
+    actual = support.hip_vjp_vjp(op, on_device)
+    for key in ["grad_output"] + OPS[op].differentiable:
+        assert_close(actual[key].cpu().numpy(), expected[key], dtype, f"c{config} {op} second order {key}", 2.0)
+    # size-independent property: the second-order function is the transpose of the
+    # derivative of the vjp, so <gg, vjp(g + dg) - vjp(g)> == <grad_grad_output, dg> exactly
+    # (the vjp is linear in grad_output)
+    rng = np.random.default_rng(17)
+    dg = rng.normal(size=case["grad_output"].shape).astype(dtype)
+    shifted = dict(on_device)
+    shifted["grad_output"] = to_device({"x": dg}, device)["x"]
+    moved = hip_vjp(op, shifted)
+    left = sum(
+        np.sum(case["grad_grad_" + key].astype(np.float64) * moved[key].cpu().numpy())
+        for key in OPS[op].differentiable
+    )
+    product = actual["grad_output"].cpu().numpy().astype(np.float64) * dg
+    assert abs(left - np.sum(product)) <= support.TOLERANCE[np.dtype(dtype)] * 100 * np.sum(np.abs(product)), op
