@@ -12,8 +12,11 @@ tensors (which PyTorch reports as ``cuda``) to the HIP library over its C ABI,
 on the current PyTorch stream. The backward of each operator is the
 library's ``*_vjp`` function; only the gradients autograd asks for are
 computed. As in the reference, tensors are made contiguous and there is no
-gradient with respect to ``C`` or the index tensors. Second derivatives are
-not available yet (the ``*_vjp`` operators carry no autograd formula).
+gradient with respect to ``C`` or the index tensors. Second derivatives: the
+``*_vjp`` operators of HPE, SAP and OPSA have a backward of their own, the
+library's ``*_vjp_vjp`` functions (the operations for which the reference
+has one, ``mops-torch/src/{hpe,sap,opsa}.cpp``); the two weighted operations
+have none, as in the reference.
 
 Host tensors are refused: this library is the device path only.
 """
@@ -69,6 +72,22 @@ _library.define(
     "Tensor W, Tensor indices_A, Tensor indices_W_1, Tensor indices_W_2, Tensor indices_output_1, "
     "Tensor indices_output_2, bool[3] wanted) -> (Tensor, Tensor, Tensor)"
 )
+# second order: cotangents of the vjp's outputs in, cotangents of its inputs out;
+# `have`: which cotangents are given (the others are empty tensors), `wanted`:
+# which of (grad_grad_output, grad_A_2[, grad_B_2]) are computed
+_library.define(
+    "homogeneous_polynomial_evaluation_vjp_vjp(Tensor grad_grad_A, Tensor grad_output, Tensor A, Tensor C, "
+    "Tensor indices_A, bool[2] wanted) -> (Tensor, Tensor)"
+)
+_library.define(
+    "outer_product_scatter_add_vjp_vjp(Tensor grad_grad_A, Tensor grad_grad_B, Tensor grad_output, Tensor A, "
+    "Tensor B, Tensor indices_output, bool[2] have, bool[3] wanted) -> (Tensor, Tensor, Tensor)"
+)
+_library.define(
+    "sparse_accumulation_of_products_vjp_vjp(Tensor grad_grad_A, Tensor grad_grad_B, Tensor grad_output, "
+    "Tensor A, Tensor B, Tensor C, Tensor indices_A, Tensor indices_B, Tensor indices_output, bool[2] have, "
+    "bool[3] wanted) -> (Tensor, Tensor, Tensor)"
+)
 
 
 def _or_empty(gradient, like):
@@ -83,6 +102,33 @@ def _hpe(A, C, indices_A):
 
 def _hpe_vjp(grad_output, A, C, indices_A):
     return _ops.homogeneous_polynomial_evaluation_vjp(grad_output, A, C, indices_A)
+
+
+def _hpe_vjp_vjp(grad_grad_A, grad_output, A, C, indices_A, wanted):
+    grad_grad_output, grad_A_2 = _ops.homogeneous_polynomial_evaluation_vjp_vjp(
+        grad_grad_A, grad_output, A, C, indices_A,
+        compute_grad_grad_output=wanted[0], compute_grad_A_2=wanted[1],
+    )  # fmt: skip
+    return _or_empty(grad_grad_output, A), _or_empty(grad_A_2, A)
+
+
+def _opsa_vjp_vjp(grad_grad_A, grad_grad_B, grad_output, A, B, indices_output, have, wanted):
+    grad_grad_output, grad_A_2, grad_B_2 = _ops.outer_product_scatter_add_vjp_vjp(
+        grad_grad_A if have[0] else None, grad_grad_B if have[1] else None, grad_output, A, B, indices_output,
+        compute_grad_grad_output=wanted[0], compute_grad_A_2=wanted[1], compute_grad_B_2=wanted[2],
+    )  # fmt: skip
+    return _or_empty(grad_grad_output, A), _or_empty(grad_A_2, A), _or_empty(grad_B_2, B)
+
+
+def _sap_vjp_vjp(
+    grad_grad_A, grad_grad_B, grad_output, A, B, C, indices_A, indices_B, indices_output, have, wanted
+):
+    grad_grad_output, grad_A_2, grad_B_2 = _ops.sparse_accumulation_of_products_vjp_vjp(
+        grad_grad_A if have[0] else None, grad_grad_B if have[1] else None, grad_output, A, B, C,
+        indices_A, indices_B, indices_output,
+        compute_grad_grad_output=wanted[0], compute_grad_A_2=wanted[1], compute_grad_B_2=wanted[2],
+    )  # fmt: skip
+    return _or_empty(grad_grad_output, A), _or_empty(grad_A_2, A), _or_empty(grad_B_2, B)
 
 
 def _opsa(A, B, indices_output, output_size):
@@ -147,6 +193,9 @@ for _name, _kernel in [
     ("outer_product_scatter_add_with_weights_vjp", _opsaw_vjp),
     ("sparse_accumulation_scatter_add_with_weights", _sasaw),
     ("sparse_accumulation_scatter_add_with_weights_vjp", _sasaw_vjp),
+    ("homogeneous_polynomial_evaluation_vjp_vjp", _hpe_vjp_vjp),
+    ("outer_product_scatter_add_vjp_vjp", _opsa_vjp_vjp),
+    ("sparse_accumulation_of_products_vjp_vjp", _sap_vjp_vjp),
 ]:
     # ROCm tensors carry the CUDA dispatch key
     _library.impl(_name, _kernel, "CUDA")
@@ -170,6 +219,12 @@ for _name in [
 ]:
     _library.impl(_name, _refuse_host(_name), "CPU")
     _library.impl(_name + "_vjp", _refuse_host(_name + "_vjp"), "CPU")
+for _name in [
+    "homogeneous_polynomial_evaluation_vjp_vjp",
+    "outer_product_scatter_add_vjp_vjp",
+    "sparse_accumulation_of_products_vjp_vjp",
+]:
+    _library.impl(_name, _refuse_host(_name), "CPU")
 
 
 # ------------------------------------------------------------------ shapes --
@@ -280,7 +335,74 @@ def _sasaw_backward(ctx, grad_output):
     )  # fmt: skip
 
 
+# ---- second order: backward of the *_vjp operators of HPE, OPSA and SAP ----
+def _given(cotangent, wanted):
+    """A cotangent counts when its output was computed and autograd passes one."""
+    return bool(wanted) and cotangent is not None
+
+
+def _hpe_vjp_setup(ctx, inputs, output):
+    ctx.save_for_backward(*inputs)
+
+
+def _hpe_vjp_backward(ctx, grad_grad_A):
+    grad_output, A, C, indices_A = ctx.saved_tensors
+    if ctx.needs_input_grad[2]:
+        raise RuntimeError("gradients with respect to C are not supported")
+    wanted = [ctx.needs_input_grad[0], ctx.needs_input_grad[1]]
+    grad_grad_output, grad_A_2 = torch.ops.mops.homogeneous_polynomial_evaluation_vjp_vjp(
+        grad_grad_A.contiguous(), grad_output, A, C, indices_A, wanted
+    )
+    return grad_grad_output if wanted[0] else None, grad_A_2 if wanted[1] else None, None, None
+
+
+def _opsa_vjp_setup(ctx, inputs, output):
+    grad_output, A, B, indices_output, wanted = inputs
+    ctx.save_for_backward(grad_output, A, B, indices_output)
+    ctx.computed = list(wanted)
+
+
+def _opsa_vjp_backward(ctx, grad_grad_A, grad_grad_B):
+    grad_output, A, B, indices_output = ctx.saved_tensors
+    have = [_given(grad_grad_A, ctx.computed[0]), _given(grad_grad_B, ctx.computed[1])]
+    wanted = [ctx.needs_input_grad[0], ctx.needs_input_grad[1], ctx.needs_input_grad[2]]
+    grad_grad_output, grad_A_2, grad_B_2 = torch.ops.mops.outer_product_scatter_add_vjp_vjp(
+        grad_grad_A.contiguous() if have[0] else A.new_empty((0,)),
+        grad_grad_B.contiguous() if have[1] else B.new_empty((0,)),
+        grad_output, A, B, indices_output, have, wanted,
+    )  # fmt: skip
+    return (
+        grad_grad_output if wanted[0] else None, grad_A_2 if wanted[1] else None,
+        grad_B_2 if wanted[2] else None, None, None,
+    )  # fmt: skip
+
+
+def _sap_vjp_setup(ctx, inputs, output):
+    ctx.save_for_backward(*inputs[:7])
+    ctx.computed = list(inputs[7])
+
+
+def _sap_vjp_backward(ctx, grad_grad_A, grad_grad_B):
+    grad_output, A, B, C, indices_A, indices_B, indices_output = ctx.saved_tensors
+    if ctx.needs_input_grad[3]:
+        raise RuntimeError("gradients with respect to C are not supported")
+    have = [_given(grad_grad_A, ctx.computed[0]), _given(grad_grad_B, ctx.computed[1])]
+    wanted = [ctx.needs_input_grad[0], ctx.needs_input_grad[1], ctx.needs_input_grad[2]]
+    grad_grad_output, grad_A_2, grad_B_2 = torch.ops.mops.sparse_accumulation_of_products_vjp_vjp(
+        grad_grad_A.contiguous() if have[0] else A.new_empty((0,)),
+        grad_grad_B.contiguous() if have[1] else B.new_empty((0,)),
+        grad_output, A, B, C, indices_A, indices_B, indices_output, have, wanted,
+    )  # fmt: skip
+    return (
+        grad_grad_output if wanted[0] else None, grad_A_2 if wanted[1] else None,
+        grad_B_2 if wanted[2] else None, None, None, None, None, None,
+    )  # fmt: skip
+
+
 for _name, _backward, _setup in [
+    ("homogeneous_polynomial_evaluation_vjp", _hpe_vjp_backward, _hpe_vjp_setup),
+    ("outer_product_scatter_add_vjp", _opsa_vjp_backward, _opsa_vjp_setup),
+    ("sparse_accumulation_of_products_vjp", _sap_vjp_backward, _sap_vjp_setup),
     ("homogeneous_polynomial_evaluation", _hpe_backward, _hpe_setup),
     ("outer_product_scatter_add", _opsa_backward, _opsa_setup),
     ("sparse_accumulation_of_products", _sap_backward, _sap_setup),

@@ -82,3 +82,25 @@ def test_only_requested_gradients_are_computed(device):
     output = torch.ops.mops.outer_product_scatter_add_with_weights(*arguments("opsaw", case))
     output.sum().backward()
     assert case["B"].grad is not None and case["A"].grad is None and case["W"].grad is None
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("op", support.SECOND_ORDER)
+def test_operator_second_derivatives(oracle, device, op):
+    """Double backward = the oracle's vjp_vjp; torch's gradgradcheck as the reference's own tests
+    (python/mops-torch/tests/{hpe,sap,opsa}.py)."""
+    case = support.add_cotangents(SMALL[op](np.float64), op)
+    expected = support.cpu_vjp_vjp(oracle, op, case)
+    on_device = support.to_device(case, device)
+    spec = support.OPS[op]
+    for name in spec.differentiable + ["grad_output"]:
+        on_device[name].requires_grad_(True)
+    operator = getattr(torch.ops.mops, spec.function)
+    output = operator(*arguments(op, on_device))
+    wanted = [on_device[name] for name in spec.differentiable]
+    gradients = torch.autograd.grad(output, wanted, on_device["grad_output"], create_graph=True)
+    contracted = sum((on_device["grad_grad_" + n] * g).sum() for n, g in zip(spec.differentiable, gradients))
+    second = torch.autograd.grad(contracted, [on_device["grad_output"]] + wanted)
+    for name, value in zip(["grad_output"] + spec.differentiable, second):
+        support.assert_close(value.cpu().numpy(), expected[name], np.float64, f"{op} second order {name}", 2.0)
+    assert torch.autograd.gradgradcheck(operator, arguments(op, on_device), fast_mode=True)
