@@ -27,6 +27,15 @@ struct ThreadState {
     int device = -1;
     hipStream_t block_stream = nullptr;
 
+    // side stream and its two events, per device
+    struct Side {
+        int device;
+        hipStream_t stream;
+        hipEvent_t forked;
+        hipEvent_t joined;
+    };
+    std::vector<Side> sides;
+
     // kernel timing
     bool timing = false;
     std::vector<std::pair<hipEvent_t, hipEvent_t>> recorded;
@@ -70,6 +79,36 @@ void finish_call(const char* operation) {
     auto& st = state();
     if (st.synchronous) {
         check_hip(hipStreamSynchronize(st.stream), operation);
+    }
+}
+
+SideStream::SideStream(hipStream_t main) : main_(main) {
+    auto& st = state();
+    int device = 0;
+    MOPS_HIP_CHECK(hipGetDevice(&device));
+    ThreadState::Side* side = nullptr;
+    for (auto& candidate : st.sides) {
+        if (candidate.device == device) {
+            side = &candidate;
+        }
+    }
+    if (side == nullptr) {
+        ThreadState::Side created{device, nullptr, nullptr, nullptr};
+        MOPS_HIP_CHECK(hipStreamCreateWithFlags(&created.stream, hipStreamNonBlocking));
+        MOPS_HIP_CHECK(hipEventCreateWithFlags(&created.forked, hipEventDisableTiming));
+        MOPS_HIP_CHECK(hipEventCreateWithFlags(&created.joined, hipEventDisableTiming));
+        st.sides.push_back(created);
+        side = &st.sides.back();
+    }
+    side_ = side->stream;
+    joined_ = side->joined;
+    MOPS_HIP_CHECK(hipEventRecord(side->forked, main_));
+    MOPS_HIP_CHECK(hipStreamWaitEvent(side_, side->forked, 0));
+}
+
+SideStream::~SideStream() {
+    if (hipEventRecord(joined_, side_) == hipSuccess) {
+        (void)hipStreamWaitEvent(main_, joined_, 0);
     }
 }
 

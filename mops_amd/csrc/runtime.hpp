@@ -42,6 +42,27 @@ void finish_call(const char* operation);
 /// block at the same time.
 void* scratch(size_t bytes);
 
+/// A second stream of the calling thread, for a kernel of a call that does not
+/// depend on the call's other kernels and leaves room on the device beside
+/// them. Construction makes the side stream wait for everything enqueued on
+/// `main` so far; destruction makes `main` wait for everything enqueued on the
+/// side stream, so that for the caller the call still happens on `main` alone
+/// (also when `main` is being captured into a graph: the side stream joins the
+/// capture and leaves it again). Default stream priority.
+class SideStream {
+public:
+    explicit SideStream(hipStream_t main);
+    ~SideStream();
+    SideStream(const SideStream&) = delete;
+    SideStream& operator=(const SideStream&) = delete;
+    hipStream_t get() const { return side_; }
+
+private:
+    hipStream_t main_;
+    hipStream_t side_ = nullptr;
+    hipEvent_t joined_ = nullptr;
+};
+
 /// Device time of an operation's main kernel, for benchmarks that want the
 /// duration of one kernel and not of the whole call. While a thread has
 /// kernel timing on (set_kernel_timing), every MainKernelTimer in scope of a

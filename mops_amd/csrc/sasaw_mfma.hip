@@ -1110,8 +1110,24 @@ void vjp(
     const DenseLayout layout = dense_layout(s);
     const DenseBuffers<T> dense = enqueue_dense<T>(workspace, layout, C, indices, s, stream);
     const int tiles = tiles_for(s.L);
+    const bool want_edges = grad_A != nullptr || grad_B != nullptr;
 
-    if (grad_A != nullptr || grad_B != nullptr) {
+    auto launch_weights = [&](hipStream_t on) {
+        const Contraction<T> c = contraction<T>(
+            A, B, grad_output, indices.output_1, dense.to_cells, layout, s, s.n2, s.n3, 1, s.n2
+        );
+        constexpr int SENDERS_PER_GROUP = senders_per_group<T>();
+        const int32_t grid = (s.n_nodes + SENDERS_PER_GROUP - 1) / SENDERS_PER_GROUP;
+        const size_t lds = weight_gradient_lds(s, sizeof(T));
+        const bool aligned = aligned_for_vectors(indices.W_1, sizeof(int32_t));
+        with_shape_constants(tiles, (s.n3 + 3) / 4, [&](auto tiles_constant, auto steps) {
+            weight_gradient_kernel<T, decltype(tiles_constant)::value, decltype(steps)::value>
+                <<<grid, SENDERS_PER_GROUP * WAVE, lds, on>>>(grad_W, indices.W_1, s.n_edges, aligned, c);
+        });
+        MOPS_HIP_CHECK(hipGetLastError());
+    };
+
+    auto launch_edges = [&]() {
         const bool vectors = s.L % 4 == 0 && aligned_for_vectors(W, sizeof(T));
         const int vec = vectors ? 4 : 1;
         EdgeGradArgs<T> args{};
@@ -1144,21 +1160,20 @@ void vjp(
                 <<<grid, WAVE, lds, stream>>>(args);
         });
         MOPS_HIP_CHECK(hipGetLastError());
-    }
+    };
 
-    if (grad_W != nullptr) {
-        const Contraction<T> c = contraction<T>(
-            A, B, grad_output, indices.output_1, dense.to_cells, layout, s, s.n2, s.n3, 1, s.n2
-        );
-        constexpr int SENDERS_PER_GROUP = senders_per_group<T>();
-        const int32_t grid = (s.n_nodes + SENDERS_PER_GROUP - 1) / SENDERS_PER_GROUP;
-        const size_t lds = weight_gradient_lds(s, sizeof(T));
-        const bool aligned = aligned_for_vectors(indices.W_1, sizeof(int32_t));
-        with_shape_constants(tiles, (s.n3 + 3) / 4, [&](auto tiles_constant, auto steps) {
-            weight_gradient_kernel<T, decltype(tiles_constant)::value, decltype(steps)::value>
-                <<<grid, SENDERS_PER_GROUP * WAVE, lds, stream>>>(grad_W, indices.W_1, s.n_edges, aligned, c);
-        });
-        MOPS_HIP_CHECK(hipGetLastError());
+    if (want_edges && grad_W != nullptr) {
+        // The two kernels are independent and both wait for memory most of
+        // the time: they share the device, the weight kernel on a side stream
+        // that forks from `stream` after the dense table and joins it again.
+        // (weights first: the other order is slower, 109 instead of 97 us in f32)
+        SideStream side(stream);
+        launch_weights(side.get());
+        launch_edges();
+    } else if (want_edges) {
+        launch_edges();
+    } else if (grad_W != nullptr) {
+        launch_weights(stream);
     }
 }
 
