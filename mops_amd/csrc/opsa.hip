@@ -780,6 +780,80 @@ __global__ __launch_bounds__(GATHER_SENDERS* WAVE) void sum_by_sender_kernel(
     }
 }
 
+// vjp for rows too wide for the LDS tile of vjp_kernel: one wavefront per
+// edge, lanes over l in chunks of 64, the receiver's grad_output row read
+// from global memory (L2). grad_A[e, k] is a fixed shuffle tree over the
+// lanes, accumulated chunk after chunk by one lane; grad_B / the per-edge row
+// of grad_W are sums over k inside a lane. Slow (every edge reads K * L
+// values) and general.
+constexpr int WIDE_WAVES = 4;
+
+template <typename T, bool WEIGHTED>
+__global__ __launch_bounds__(WIDE_WAVES* WAVE) void vjp_wide_kernel(
+    T* grad_A,
+    T* __restrict__ grad_B,
+    T* __restrict__ edge_W,
+    const T* __restrict__ grad_output,
+    const T* __restrict__ A,
+    const T* __restrict__ B,
+    const T* __restrict__ W,
+    const int32_t* __restrict__ indices_W,
+    const int32_t* __restrict__ indices_output,
+    int32_t n_edges,
+    int32_t n_output,
+    int32_t K,
+    int32_t L
+) {
+    const int lane = threadIdx.x & (WAVE - 1);
+    const int32_t e = blockIdx.x * WIDE_WAVES + (threadIdx.x >> 6);
+    if (e >= n_edges) {
+        return;
+    }
+    const int32_t receiver = indices_output[e];
+    const bool receiver_ok = in_bounds(receiver, n_output);
+    const T* g_row = grad_output + static_cast<size_t>(receiver_ok ? receiver : 0) * K * L;
+    const T* a_row = A + static_cast<size_t>(e) * K;
+    int32_t w_row = 0;
+    bool w_ok = true;
+    if constexpr (WEIGHTED) {
+        w_row = indices_W[e];
+        w_ok = in_bounds(w_row, n_output);
+        w_row = w_ok ? w_row : 0;
+    }
+    for (int32_t l0 = 0; l0 < L; l0 += WAVE) {
+        const int32_t l = l0 + lane;
+        const bool ok = l < L;
+        const T b = load_or_zero(B, static_cast<size_t>(e) * L + l, ok);
+        T w = T(1);
+        if constexpr (WEIGHTED) {
+            w = load_or_zero(W, static_cast<size_t>(w_row) * L + l, ok && w_ok);
+        }
+        const T bw = b * w;
+        T along_k = T(0);
+        for (int32_t k = 0; k < K; k++) {
+            const T g = load_or_zero(g_row, static_cast<size_t>(k) * L + l, ok && receiver_ok);
+            along_k += g * a_row[k];
+            T along_l = g * bw;
+#pragma unroll
+            for (int offset = WAVE / 2; offset > 0; offset >>= 1) {
+                along_l += __shfl_xor(along_l, offset);
+            }
+            if (grad_A != nullptr && lane == 0) {
+                T* target = grad_A + static_cast<size_t>(e) * K + k;
+                *target = (l0 == 0 ? T(0) : *target) + along_l;
+            }
+        }
+        if (ok) {
+            if (grad_B != nullptr) {
+                grad_B[static_cast<size_t>(e) * L + l] = along_k * w;
+            }
+            if (WEIGHTED && edge_W != nullptr) {
+                edge_W[static_cast<size_t>(e) * L + l] = along_k * b;
+            }
+        }
+    }
+}
+
 unsigned blocks_for(int32_t n_edges) {
     size_t waves = ceil_div(static_cast<size_t>(n_edges), CHUNK);
     return static_cast<unsigned>(ceil_div(waves, WAVES_PER_BLOCK));
@@ -887,12 +961,6 @@ void launch_vjp(
         const size_t Ks = odd_stride(K), Ls = odd_stride(L);
         const size_t lds =
             (K * Ls + STAGE_EDGES * Ks + (WEIGHTED ? 2 : 1) * STAGE_EDGES * Ls) * sizeof(T);
-        if (lds > 64 * 1024) {
-            throw std::runtime_error(
-                std::string(operation) + ": size_A * size_B = " + std::to_string(K) + " * " +
-                std::to_string(L) + " is too large for the LDS tile of the device kernel"
-            );
-        }
         auto log2_ceil = [](int32_t n) {
             int32_t shift = 0;
             while ((1 << shift) < n) {
@@ -901,7 +969,13 @@ void launch_vjp(
             return shift;
         };
         const unsigned waves = static_cast<unsigned>(ceil_div(static_cast<size_t>(n_edges), CHUNK));
-        if (K <= 32 && L <= 64) {
+        if (lds > 64 * 1024) {
+            const unsigned blocks = static_cast<unsigned>(ceil_div(static_cast<size_t>(n_edges), WIDE_WAVES));
+            vjp_wide_kernel<T, WEIGHTED><<<blocks, WIDE_WAVES * WAVE, 0, stream>>>(
+                grad_A.data, grad_B.data, edge_W, grad_output.data, A.data, B.data, W, indices_W,
+                indices_output.data, n_edges, n_output, K, L
+            );
+        } else if (K <= 32 && L <= 64) {
             const unsigned groups = static_cast<unsigned>(ceil_div(static_cast<size_t>(n_edges), 16));
             MainKernelTimer timer(stream);
 #define MOPS_LAUNCH_ROWS(KT, NT)                                                                   \

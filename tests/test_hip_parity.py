@@ -65,6 +65,52 @@ CASES = {
 }  # fmt: skip
 
 
+# Large and lopsided inputs: many times the BASELINE sizes, one receiver that
+# owns almost every edge, senders named by tens of thousands of edges, feature
+# counts beyond the matrix-core paths (the general kernels).
+LARGE = {
+    "hpe": {
+        "many_rows": lambda s, d: support.hpe_case(s, d, I=300000, nA=40, J=300, K=4),
+        "many_monomials": lambda s, d: support.hpe_case(s, d, I=500, nA=60, J=40000, K=5),
+    },
+    "sap": {
+        "many_rows": lambda s, d: support.sap_case(s, d, I=1000003, nA=13, nB=7, K=900, nO=20),
+        "long_table": lambda s, d: support.sap_case(s, d, I=20000, nA=16, nB=16, K=6000, nO=30),
+        "big_table_dimensions": lambda s, d: support.sap_case(s, d, I=5000, nA=40, nB=30, K=3000, nO=50),
+    },
+    "opsa": {
+        "many_edges": lambda s, d: support.opsa_case(s, d, J=1000003, K=13, L=20, n_out=30000, allow_empty=True),
+        "one_receiver": lambda s, d: _one_receiver(support.opsa_case(s, d, J=120000, K=13, L=20, n_out=50), "indices_output"),
+        "wide_rows": lambda s, d: support.opsa_case(s, d, J=20000, K=50, L=200, n_out=300, allow_empty=True),
+    },
+    "opsaw": {
+        "many_edges": lambda s, d: support.opsaw_case(s, d, E=500001, K=16, L=64, n_nodes=20000, allow_empty=True),
+        "one_receiver_one_sender": lambda s, d: _hub(
+            _one_receiver(support.opsaw_case(s, d, E=120000, K=13, L=32, n_nodes=50), "indices_output"), "indices_W"
+        ),
+        "wide_rows": lambda s, d: support.opsaw_case(s, d, E=20000, K=40, L=300, n_nodes=300, allow_empty=True),
+    },
+    "sasaw": {
+        "many_edges": lambda s, d: support.sasaw_case(s, d, E=300001, nA=9, L=32, n_nodes=10000, allow_empty=True),
+        "one_receiver_one_sender": lambda s, d: _hub(
+            _one_receiver(support.sasaw_case(s, d, E=60000, nA=9, L=32, n_nodes=40), "indices_output_1"), "indices_W_1"
+        ),
+        "sixteen": lambda s, d: support.sasaw_case(s, d, E=30000, nA=16, L=64, n_nodes=900, n2=16, n3=16, N=700),
+        "beyond_the_matrix_path": lambda s, d: support.sasaw_case(
+            s, d, E=8000, nA=20, L=100, n_nodes=300, n2=18, n3=25, N=900, allow_empty=True
+        ),
+    },
+}  # fmt: skip
+
+
+def _one_receiver(case, key):
+    """Nine edges in ten go to output row 3 (the index stays sorted)."""
+    index = case[key]
+    index[len(index) // 20 : len(index) * 19 // 20] = 3
+    case[key] = np.sort(index)
+    return case
+
+
 def _hub(case, key):
     """Most edges name the same sender: one gather list longer than the LDS sort buffer."""
     case[key][: len(case[key]) * 3 // 4] = 2
@@ -152,6 +198,30 @@ def test_bit_reproducible(device, op):
     g2 = hip_vjp(op, case)
     for key in OPS[op].differentiable:
         assert np.array_equal(g1[key].cpu().numpy(), g2[key].cpu().numpy()), (op, key)
+
+
+ALL_LARGE = [(op, name) for op, cases in LARGE.items() for name in cases]
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=["f32", "f64"])
+@pytest.mark.parametrize("op,name", ALL_LARGE)
+def test_large_inputs(oracle, device, op, name, dtype):
+    case = LARGE[op][name](808, dtype)
+    on_device = to_device(case, device)
+    # Expected values from the oracle in float64 on the same (already rounded) inputs: with
+    # tens of thousands of terms per sum a float32 oracle is itself only good to ~1e-4, and
+    # the bar is closeness to the exact result. Sums of ~1e5 float32 terms get 8x the bound.
+    exact = {
+        key: value.astype(np.float64) if isinstance(value, np.ndarray) and value.dtype == dtype else value
+        for key, value in case.items()
+    }
+    factor = 8.0 if dtype == np.float32 and "one_receiver" in name else 2.0
+    actual = hip_forward(op, on_device).cpu().numpy()
+    assert_close(actual, cpu_forward(oracle, op, exact), dtype, f"{op}/{name} forward", factor)
+    expected = cpu_vjp(oracle, op, exact)
+    gradients = hip_vjp(op, on_device)
+    for key in OPS[op].differentiable:
+        assert_close(gradients[key].cpu().numpy(), expected[key], dtype, f"{op}/{name} grad_{key}", factor)
 
 
 # ---- BASELINE configurations at full size ---------------------------------
