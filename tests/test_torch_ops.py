@@ -104,3 +104,26 @@ def test_operator_second_derivatives(oracle, device, op):
     for name, value in zip(["grad_output"] + spec.differentiable, second):
         support.assert_close(value.cpu().numpy(), expected[name], np.float64, f"{op} second order {name}", 2.0)
     assert torch.autograd.gradgradcheck(operator, arguments(op, on_device), fast_mode=True)
+
+
+@pytest.mark.gpu
+def test_torchscript_save_and_load(oracle, device, tmp_path):
+    """A scripted module that calls the operators survives save / load, as in the reference's
+    python/mops-torch/tests/torchscript.py."""
+
+    class Model(torch.nn.Module):
+        def forward(self, A, B, indices_output, output_size: int):
+            return torch.ops.mops.outer_product_scatter_add(A, B, indices_output, output_size)
+
+    case = SMALL["opsa"](np.float64)
+    on_device = support.to_device(case, device)
+    scripted = torch.jit.script(Model())
+    path = str(tmp_path / "model.pt")
+    scripted.save(path)
+    loaded = torch.jit.load(path)
+    actual = loaded(*arguments("opsa", on_device))
+    support.assert_close(actual.cpu().numpy(), support.cpu_forward(oracle, "opsa", case), np.float64, "scripted opsa")
+    on_device["A"].requires_grad_(True)
+    loaded(*arguments("opsa", on_device)).backward(on_device["grad_output"])
+    expected = support.cpu_vjp(oracle, "opsa", case, wanted=["A"])["A"]
+    support.assert_close(on_device["A"].grad.cpu().numpy(), expected, np.float64, "scripted opsa grad_A")
