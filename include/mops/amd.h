@@ -60,6 +60,22 @@ MOPS_EXPORT int mops_amd_first_occurrences(
 MOPS_EXPORT int mops_amd_kernel_timing(int enable);
 MOPS_EXPORT int mops_amd_kernel_time(double* total_milliseconds, int64_t* launches);
 
+/* Scatter indices that are not sorted.
+ *
+ * The device kernels of outer_product_scatter_add[_with_weights] and
+ * sparse_accumulation_scatter_add_with_weights need their scatter index
+ * (indices_output, indices_output_1) non-decreasing, as the device path of the
+ * reference does (python/mops/tests/opsa.py:96); the reference's HOST path
+ * accepts any order (mops/src/opsa/cpu.tpp:29). accept != 0 gives the calling
+ * thread the host semantics on the device: each of these calls (forward, vjp,
+ * vjp_vjp) first tests the index on the device and, when it is not sorted,
+ * re-orders the edges by a stable sort, so that the result is the one the host
+ * loops give. The test makes the call wait for the device once, so such calls
+ * cannot be captured into a HIP graph. Default: off (or on when the
+ * environment variable MOPS_AMD_ACCEPT_UNSORTED is set to something other
+ * than 0). Returns the previous setting. */
+MOPS_EXPORT int mops_amd_accept_unsorted_indices(int accept);
+
 #ifdef __cplusplus
 }
 #endif

@@ -6,6 +6,7 @@ The public names are those of the reference's Python package
 (``python/mops/src/mops/__init__.py`` of lab-cosmo/mops).
 """
 from .ops import (  # noqa: F401
+    accept_unsorted_indices,
     first_occurrences,
     homogeneous_polynomial_evaluation,
     homogeneous_polynomial_evaluation_vjp,

@@ -48,6 +48,8 @@ def device_library():
             ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64, ctypes.c_void_p,
         ]  # fmt: skip
         cdll.mops_amd_first_occurrences.restype = ctypes.c_int
+        cdll.mops_amd_accept_unsorted_indices.argtypes = [ctypes.c_int]
+        cdll.mops_amd_accept_unsorted_indices.restype = ctypes.c_int
         cdll.mops_amd_kernel_timing.argtypes = [ctypes.c_int]
         cdll.mops_amd_kernel_timing.restype = ctypes.c_int
         cdll.mops_amd_kernel_time.argtypes = [

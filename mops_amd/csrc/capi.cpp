@@ -13,6 +13,7 @@
 #include "mops.hpp"
 
 #include "first_occurrences.hpp"
+#include "edge_order.hpp"
 #include "runtime.hpp"
 
 namespace {
@@ -127,6 +128,10 @@ extern "C" int mops_amd_first_occurrences(
     );
     mops::amd::finish_call("first_occurrences");
     MOPS_CATCH_EXCEPTIONS_END
+}
+
+extern "C" int mops_amd_accept_unsorted_indices(int accept) {
+    return mops::amd::set_accept_unsorted(accept != 0) ? 1 : 0;
 }
 
 extern "C" int mops_amd_kernel_timing(int enable) {

@@ -1,6 +1,7 @@
 #include "elementwise.hpp"
 
 #include <algorithm>
+#include <cstdint>
 
 #include "runtime.hpp"
 
@@ -68,5 +69,7 @@ template void add_in_place<float>(float*, const float*, size_t, hipStream_t);
 template void add_in_place<double>(double*, const double*, size_t, hipStream_t);
 template class StreamTemporary<float>;
 template class StreamTemporary<double>;
+template class StreamTemporary<int32_t>;
+template class StreamTemporary<unsigned char>;
 
 } // namespace mops::amd

@@ -39,6 +39,7 @@
 #include "first_occurrences.hpp"
 #include "index_validation.hpp"
 #include "mfma.hpp"
+#include "edge_order.hpp"
 #include "elementwise.hpp"
 #include "runtime.hpp"
 #include "segment_walk.hpp"
@@ -1025,6 +1026,51 @@ void launch_vjp(
     finish_call(operation);
 }
 
+/// The per-edge tensors of one OPSA / OPSAW call re-ordered by a stable sort
+/// of the scatter index, with room for the per-edge gradients in that order.
+template <typename T> class SortedEdges {
+public:
+    SortedEdges(
+        Tensor<T, 2> A, Tensor<T, 2> B, const int32_t* second_index, Tensor<int32_t, 1> indices_output,
+        bool want_A, bool want_B
+    )
+        : stream_(current_stream()), n_(A.shape[0]), K_(A.shape[1]), L_(B.shape[1]),
+          order_(indices_output.data, narrow_i32(A.shape[0], "A.shape[0]"), stream_), A_(n_ * K_, stream_),
+          B_(n_ * L_, stream_), second_(second_index != nullptr ? n_ : 0, stream_),
+          grad_A_(want_A ? n_ * K_ : 0, stream_), grad_B_(want_B ? n_ * L_ : 0, stream_), want_A_(want_A),
+          want_B_(want_B) {
+        order_.gather_rows(A_.data(), A.data, narrow_i32(K_, "A.shape[1]"));
+        order_.gather_rows(B_.data(), B.data, narrow_i32(L_, "B.shape[1]"));
+        if (second_index != nullptr) {
+            order_.gather_rows(second_.data(), second_index, 1);
+        }
+    }
+    Tensor<T, 2> A() const { return {A_.data(), {n_, K_}}; }
+    Tensor<T, 2> B() const { return {B_.data(), {n_, L_}}; }
+    Tensor<int32_t, 1> index() const { return {const_cast<int32_t*>(order_.sorted_index()), {n_}}; }
+    Tensor<int32_t, 1> second_index() const { return {second_.data(), {n_}}; }
+    Tensor<T, 2> grad_A() const { return {grad_A_.data(), {want_A_ ? n_ : 0, want_A_ ? K_ : 0}}; }
+    Tensor<T, 2> grad_B() const { return {grad_B_.data(), {want_B_ ? n_ : 0, want_B_ ? L_ : 0}}; }
+    /// per-edge gradients back to the callers' rows
+    void put_back(Tensor<T, 2> grad_A, Tensor<T, 2> grad_B) const {
+        if (want_A_) {
+            order_.scatter_rows(grad_A.data, grad_A_.data(), static_cast<int32_t>(K_));
+        }
+        if (want_B_) {
+            order_.scatter_rows(grad_B.data, grad_B_.data(), static_cast<int32_t>(L_));
+        }
+    }
+
+private:
+    hipStream_t stream_;
+    size_t n_, K_, L_;
+    EdgeOrder order_;
+    StreamTemporary<T> A_, B_;
+    StreamTemporary<int32_t> second_;
+    StreamTemporary<T> grad_A_, grad_B_;
+    bool want_A_, want_B_;
+};
+
 } // namespace
 } // namespace mops::amd
 
@@ -1036,6 +1082,13 @@ void outer_product_scatter_add(MOPS_OPSA_PARAMS(MOPS_CXX_FIRST, MOPS_CXX_NEXT)) 
     const char* operation = "cuda_outer_product_scatter_add";
     checks::Validator validator(operation);
     checks::opsa(validator, output, A, B, indices_output);
+    if (amd::accept_unsorted() &&
+        !amd::is_sorted_on_device(indices_output.data, amd::narrow_i32(A.shape[0], "A.shape[0]"), amd::current_stream())) {
+        // the same call on the edges in the order of a stable sort by destination
+        const amd::SortedEdges<scalar_t> sorted(A, B, nullptr, indices_output, false, false);
+        ::mops::cuda::outer_product_scatter_add<scalar_t>(output, sorted.A(), sorted.B(), sorted.index());
+        return;
+    }
     amd::validate_scatter_index(indices_output, output.shape[0], "indices_output", operation);
     amd::launch_forward<scalar_t, false>(output, A, B, nullptr, nullptr, indices_output, operation);
 }
@@ -1045,6 +1098,18 @@ void outer_product_scatter_add_vjp(MOPS_OPSA_VJP_PARAMS(MOPS_CXX_FIRST, MOPS_CXX
     const char* operation = "cuda_outer_product_scatter_add_vjp";
     checks::Validator validator(operation);
     checks::opsa_vjp(validator, grad_A, grad_B, grad_output, A, B, indices_output);
+    if (amd::accept_unsorted() &&
+        !amd::is_sorted_on_device(indices_output.data, amd::narrow_i32(A.shape[0], "A.shape[0]"), amd::current_stream())) {
+        const amd::SortedEdges<scalar_t> sorted(
+            A, B, nullptr, indices_output, grad_A.data != nullptr, grad_B.data != nullptr
+        );
+        ::mops::cuda::outer_product_scatter_add_vjp<scalar_t>(
+            sorted.grad_A(), sorted.grad_B(), grad_output, sorted.A(), sorted.B(), sorted.index()
+        );
+        sorted.put_back(grad_A, grad_B);
+        amd::finish_call(operation);
+        return;
+    }
     amd::validate_scatter_index(indices_output, grad_output.shape[0], "indices_output", operation);
     amd::launch_vjp<scalar_t, false>(
         grad_A, grad_B, Tensor<scalar_t, 2>{nullptr, {0, 0}}, grad_output, A, B, nullptr, nullptr,
@@ -1114,6 +1179,14 @@ void outer_product_scatter_add_with_weights(MOPS_OPSAW_PARAMS(MOPS_CXX_FIRST, MO
     const char* operation = "cuda_outer_product_scatter_add_with_weights";
     checks::Validator validator(operation);
     checks::opsaw(validator, output, A, B, W, indices_W, indices_output);
+    if (amd::accept_unsorted() &&
+        !amd::is_sorted_on_device(indices_output.data, amd::narrow_i32(A.shape[0], "A.shape[0]"), amd::current_stream())) {
+        const amd::SortedEdges<scalar_t> sorted(A, B, indices_W.data, indices_output, false, false);
+        ::mops::cuda::outer_product_scatter_add_with_weights<scalar_t>(
+            output, sorted.A(), sorted.B(), W, sorted.second_index(), sorted.index()
+        );
+        return;
+    }
     amd::validate_scatter_index(indices_output, output.shape[0], "indices_output", operation);
     amd::validate_gather_index(indices_W, output.shape[0], "indices_W", operation);
     amd::launch_forward<scalar_t, true>(output, A, B, W.data, indices_W.data, indices_output, operation);
@@ -1124,6 +1197,19 @@ void outer_product_scatter_add_with_weights_vjp(MOPS_OPSAW_VJP_PARAMS(MOPS_CXX_F
     const char* operation = "cuda_outer_product_scatter_add_with_weights_vjp";
     checks::Validator validator(operation);
     checks::opsaw_vjp(validator, grad_A, grad_B, grad_W, grad_output, A, B, W, indices_W, indices_output);
+    if (amd::accept_unsorted() &&
+        !amd::is_sorted_on_device(indices_output.data, amd::narrow_i32(A.shape[0], "A.shape[0]"), amd::current_stream())) {
+        const amd::SortedEdges<scalar_t> sorted(
+            A, B, indices_W.data, indices_output, grad_A.data != nullptr, grad_B.data != nullptr
+        );
+        ::mops::cuda::outer_product_scatter_add_with_weights_vjp<scalar_t>(
+            sorted.grad_A(), sorted.grad_B(), grad_W, grad_output, sorted.A(), sorted.B(), W,
+            sorted.second_index(), sorted.index()
+        );
+        sorted.put_back(grad_A, grad_B);
+        amd::finish_call(operation);
+        return;
+    }
     amd::validate_scatter_index(indices_output, grad_output.shape[0], "indices_output", operation);
     amd::validate_gather_index(indices_W, grad_output.shape[0], "indices_W", operation);
     amd::launch_vjp<scalar_t, true>(

@@ -44,6 +44,7 @@
 #include "device_common.hpp"
 #include "first_occurrences.hpp"
 #include "index_validation.hpp"
+#include "edge_order.hpp"
 #include "runtime.hpp"
 #include "sasaw_mfma.hpp"
 #include "sender_buckets.hpp"
@@ -587,6 +588,27 @@ void sparse_accumulation_scatter_add_with_weights(MOPS_SASAW_PARAMS(MOPS_CXX_FIR
     checks::sasaw(
         validator, output, A, B, C, W, indices_A, indices_W_1, indices_W_2, indices_output_1, indices_output_2
     );
+    if (accept_unsorted() && !is_sorted_on_device(
+                                 indices_output_1.data, narrow_i32(A.shape[0], "A.shape[0]"), current_stream()
+                             )) {
+        // the same call on the edges in the order of a stable sort by receiver
+        hipStream_t stream = current_stream();
+        const int32_t n_edges = narrow_i32(A.shape[0], "A.shape[0]");
+        const int32_t nA = narrow_i32(A.shape[1], "A.shape[1]"), L = narrow_i32(B.shape[1], "B.shape[1]");
+        EdgeOrder order(indices_output_1.data, n_edges, stream);
+        StreamTemporary<scalar_t> sorted_A(A.shape[0] * A.shape[1], stream);
+        StreamTemporary<scalar_t> sorted_B(B.shape[0] * B.shape[1], stream);
+        StreamTemporary<int32_t> sorted_W_1(A.shape[0], stream);
+        order.gather_rows(sorted_A.data(), A.data, nA);
+        order.gather_rows(sorted_B.data(), B.data, L);
+        order.gather_rows(sorted_W_1.data(), indices_W_1.data, 1);
+        ::mops::cuda::sparse_accumulation_scatter_add_with_weights<scalar_t>(
+            output, {sorted_A.data(), {A.shape[0], A.shape[1]}}, {sorted_B.data(), {B.shape[0], B.shape[1]}}, C, W,
+            indices_A, {sorted_W_1.data(), {A.shape[0]}}, indices_W_2,
+            {const_cast<int32_t*>(order.sorted_index()), {A.shape[0]}}, indices_output_2
+        );
+        return;
+    }
     validate_gather_index(indices_A, A.shape[1], "indices_A", operation);
     validate_gather_index(indices_W_1, output.shape[0], "indices_W_1", operation);
     validate_gather_index(indices_W_2, W.shape[1], "indices_W_2", operation);
@@ -650,6 +672,39 @@ void sparse_accumulation_scatter_add_with_weights_vjp(MOPS_SASAW_VJP_PARAMS(MOPS
     const bool want_B = grad_B.data != nullptr;
     const bool want_W = grad_W.data != nullptr;
     if (!want_A && !want_B && !want_W) {
+        return;
+    }
+    if (accept_unsorted() && !is_sorted_on_device(
+                                 indices_output_1.data, narrow_i32(A.shape[0], "A.shape[0]"), current_stream()
+                             )) {
+        // the same call on the edges in the order of a stable sort by receiver;
+        // the per-edge gradients go back to their own rows afterwards
+        hipStream_t stream = current_stream();
+        const int32_t n_edges = narrow_i32(A.shape[0], "A.shape[0]");
+        const int32_t nA = narrow_i32(A.shape[1], "A.shape[1]"), L = narrow_i32(B.shape[1], "B.shape[1]");
+        EdgeOrder order(indices_output_1.data, n_edges, stream);
+        StreamTemporary<scalar_t> sorted_A(A.shape[0] * A.shape[1], stream);
+        StreamTemporary<scalar_t> sorted_B(B.shape[0] * B.shape[1], stream);
+        StreamTemporary<int32_t> sorted_W_1(A.shape[0], stream);
+        StreamTemporary<scalar_t> sorted_grad_A(want_A ? A.shape[0] * A.shape[1] : 0, stream);
+        StreamTemporary<scalar_t> sorted_grad_B(want_B ? B.shape[0] * B.shape[1] : 0, stream);
+        order.gather_rows(sorted_A.data(), A.data, nA);
+        order.gather_rows(sorted_B.data(), B.data, L);
+        order.gather_rows(sorted_W_1.data(), indices_W_1.data, 1);
+        ::mops::cuda::sparse_accumulation_scatter_add_with_weights_vjp<scalar_t>(
+            {sorted_grad_A.data(), {want_A ? A.shape[0] : 0, want_A ? A.shape[1] : 0}},
+            {sorted_grad_B.data(), {want_B ? B.shape[0] : 0, want_B ? B.shape[1] : 0}}, grad_W, grad_output,
+            {sorted_A.data(), {A.shape[0], A.shape[1]}}, {sorted_B.data(), {B.shape[0], B.shape[1]}}, C, W,
+            indices_A, {sorted_W_1.data(), {A.shape[0]}}, indices_W_2,
+            {const_cast<int32_t*>(order.sorted_index()), {A.shape[0]}}, indices_output_2
+        );
+        if (want_A) {
+            order.scatter_rows(grad_A.data, sorted_grad_A.data(), nA);
+        }
+        if (want_B) {
+            order.scatter_rows(grad_B.data, sorted_grad_B.data(), L);
+        }
+        finish_call(operation);
         return;
     }
     // the reference repeats the gradient shape tests here under the operation

@@ -448,3 +448,17 @@ def first_occurrences(sorted_indices, output_size):
 
         raise MopsError(library.last_error(), status)
     return result
+
+
+# ----------------------------------------------------- unsorted indices ----
+def accept_unsorted_indices(accept=True):
+    """Let the scatter operations take a scatter index in any order (this thread).
+
+    The device kernels need ``indices_output`` / ``indices_output_1`` sorted,
+    like the reference's device path; with this switch on, every call tests
+    the index on the device and re-orders the edges by a stable sort when it
+    has to, which gives the results of the reference's host path
+    (``mops/src/opsa/cpu.tpp:29``). Costs one wait for the device per call.
+    Returns the previous setting.
+    """
+    return bool(device_library().cdll.mops_amd_accept_unsorted_indices(1 if accept else 0))

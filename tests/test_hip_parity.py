@@ -327,3 +327,67 @@ def test_vjp_vjp_baseline_configuration(oracle, device, op, config, dtype, build
     )
     product = actual["grad_output"].cpu().numpy().astype(np.float64) * dg
     assert abs(left - np.sum(product)) <= support.TOLERANCE[np.dtype(dtype)] * 100 * np.sum(np.abs(product)), op
+
+
+# ---- scatter index in any order (host semantics on the device) -------------
+@pytest.fixture
+def unsorted_accepted(device):
+    import mops_amd
+
+    previous = mops_amd.accept_unsorted_indices(True)
+    yield
+    mops_amd.accept_unsorted_indices(previous)
+
+
+def _shuffled(case, op, seed):
+    """The same edges in a random order (so the scatter index is no longer sorted)."""
+    rng = np.random.default_rng(seed)
+    per_edge = {
+        "opsa": ["A", "B", "indices_output"],
+        "opsaw": ["A", "B", "indices_W", "indices_output"],
+        "sasaw": ["A", "B", "indices_W_1", "indices_output_1"],
+    }[op]
+    order = rng.permutation(case["A"].shape[0])
+    for key in per_edge:
+        case[key] = np.ascontiguousarray(case[key][order])
+    return case
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=["f32", "f64"])
+@pytest.mark.parametrize("op", ["opsa", "opsaw", "sasaw"])
+@pytest.mark.parametrize("name", ["ragged", "long_segments", "mostly_empty"])
+def test_unsorted_scatter_index(oracle, device, unsorted_accepted, op, name, dtype):
+    if name not in CASES[op]:
+        pytest.skip("no such case for this operation")
+    case = _shuffled(CASES[op][name](909, dtype), op, 5)
+    key = "indices_output_1" if op == "sasaw" else "indices_output"
+    assert np.any(np.diff(case[key]) < 0)
+    on_device = to_device(case, device)
+    actual = hip_forward(op, on_device).cpu().numpy()
+    assert_close(actual, cpu_forward(oracle, op, case), dtype, f"{op}/{name} unsorted forward")
+    expected = cpu_vjp(oracle, op, case)
+    gradients = hip_vjp(op, on_device)
+    for name_ in OPS[op].differentiable:
+        assert_close(gradients[name_].cpu().numpy(), expected[name_], dtype, f"{op}/{name} unsorted grad_{name_}")
+    # only some of the gradients
+    partial = hip_vjp(op, on_device, wanted=["B"])
+    assert np.array_equal(partial["B"].cpu().numpy(), gradients["B"].cpu().numpy())
+    if op in support.SECOND_ORDER:
+        support.add_cotangents(case, op)
+        on_device = to_device(case, device)
+        second = support.hip_vjp_vjp(op, on_device)
+        expected = support.cpu_vjp_vjp(oracle, op, case)
+        for name_ in ["grad_output"] + OPS[op].differentiable:
+            assert_close(second[name_].cpu().numpy(), expected[name_], dtype, f"{op}/{name} unsorted second {name_}", 2.0)
+
+
+def test_sorted_index_takes_the_usual_path_when_unsorted_is_accepted(device, unsorted_accepted):
+    """With the switch on, a sorted index gives the same bits as with the switch off."""
+    import mops_amd
+
+    case = to_device(CASES["opsaw"]["ragged"](111, np.float32), device)
+    with_switch = hip_forward("opsaw", case).cpu().numpy()
+    mops_amd.accept_unsorted_indices(False)
+    without = hip_forward("opsaw", case).cpu().numpy()
+    mops_amd.accept_unsorted_indices(True)
+    assert np.array_equal(with_switch, without)
