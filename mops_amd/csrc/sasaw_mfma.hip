@@ -460,7 +460,7 @@ __device__ __forceinline__ void clear_zero_row(T* __restrict__ t_area, const Den
 /// Wavefronts per workgroup (their T areas share 64 KB of LDS) ...
 template <typename T> constexpr int forward_waves() { return 2; }
 /// ... and positions of the sorted index per workgroup, 16 per wavefront.
-template <typename T> constexpr int forward_chunk() { return STAGE * forward_waves<T>(); }
+template <typename T> constexpr int forward_chunk() { return 2 * STAGE * forward_waves<T>(); }
 
 /// Segments whose partial sums wait in LDS before the wavefronts meet.
 template <typename T> constexpr int round_segments() { return sizeof(T) == 4 ? 2 : 1; }
