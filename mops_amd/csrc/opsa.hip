@@ -713,7 +713,7 @@ __global__ __launch_bounds__(WAVE) void edge_rows_vjp_kernel(
 // wavefronts find the edges of their eight senders by one pass over the
 // sender index (sender_gather.hpp) and add the rows up, sixteen loads in
 // flight. Used when a row of W fits one value per lane and register.
-constexpr int GATHER_SENDERS = 16;
+constexpr int GATHER_SENDERS = 8;
 constexpr int GATHER_COLUMNS = 4; // values of a row per lane
 
 template <typename T>
