@@ -41,7 +41,7 @@ __device__ __forceinline__ void wave_sync() {
 
 template <int NW> struct SenderGather {
     static constexpr int CAPACITY = 256; // >= 64 * 4: one load of a wavefront always fits
-    static constexpr int RING = 128;
+    static constexpr int RING = 128; // a power of two
     static constexpr int STAGE = 16;
 
     struct Storage {
@@ -57,6 +57,10 @@ template <int NW> struct SenderGather {
     /// batch of n <= 16 edges of node node0 + s; lane k (and k + 16, k + 32,
     /// k + 48) holds edge k of the batch in `my_edge`, -1 beyond n.
     /// VEC = 4 needs `senders` aligned to 16 bytes.
+    /// `keep_waiting`: batches are handed on while more edges than this wait
+    /// (at most RING - 64, so that the matches of one more look fit): STAGE - 1
+    /// hands every full batch on at once, RING - 64 collects as many edges as
+    /// possible first, for consumers that only start loads per batch.
     template <int VEC, typename StageFn>
     static __device__ __forceinline__ void run(
         Storage& lds,
@@ -64,7 +68,8 @@ template <int NW> struct SenderGather {
         int32_t n_edges,
         int32_t node0,
         int32_t n_nodes,
-        StageFn&& on_stage
+        StageFn&& on_stage,
+        int32_t keep_waiting = STAGE - 1
     ) {
         const int lane = threadIdx.x & (WAVE - 1);
         const int wave = threadIdx.x >> 6;
@@ -76,23 +81,18 @@ template <int NW> struct SenderGather {
         int32_t unit = min(wave * units_per_wave, total_units);
         const unsigned long long below = (1ull << lane) - 1ull;
 
+        // the waiting edges of my node: a circular buffer of RING positions
+        int32_t ring_head = 0;
         int32_t ring_count = 0;
         auto drain = [&](int32_t keep_below) {
-            // hands on full batches while more than `keep_below` edges wait
+            // hands on batches while more than `keep_below` edges wait
             while (ring_count > keep_below) {
                 const int32_t n = min(STAGE, ring_count);
                 const int k = lane & (STAGE - 1);
-                const int32_t my_edge = k < n ? lds.ring[wave][k] : -1;
-                const int32_t moved = STAGE + lane < ring_count ? lds.ring[wave][STAGE + lane] : 0;
-                wave_sync();
+                const int32_t my_edge = k < n ? lds.ring[wave][(ring_head + k) & (RING - 1)] : -1;
                 on_stage(my_edge, n);
-                if (STAGE + lane < ring_count) {
-                    lds.ring[wave][lane] = moved;
-                }
-                // RING - STAGE > 64 would need a second move; RING is 128 and at
-                // most STAGE - 1 + 64 edges wait, so one move of 64 covers it
+                ring_head = (ring_head + n) & (RING - 1);
                 ring_count -= n;
-                wave_sync();
             }
         };
 
@@ -195,11 +195,12 @@ template <int NW> struct SenderGather {
                     const unsigned long long mask = __ballot(mine);
                     if (mask != 0) {
                         if (mine) {
-                            lds.ring[wave][ring_count + __popcll(mask & below)] = lds.edges[v][at];
+                            lds.ring[wave][(ring_head + ring_count + __popcll(mask & below)) & (RING - 1)] =
+                                lds.edges[v][at];
                         }
                         ring_count += __popcll(mask);
                         wave_sync();
-                        drain(STAGE - 1);
+                        drain(keep_waiting);
                     }
                 }
             }
