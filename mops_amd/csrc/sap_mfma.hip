@@ -180,55 +180,81 @@ __device__ __forceinline__ void build_operands(
         if (first_of_list[e]) {
             const int32_t head = areas.heads[dense[e]];
             T sum = T(0);
-            // short lists (all of them, in practice) are read once, sorted in
-            // registers and summed; NOBODY is larger than any entry number
-            constexpr int SHORT = 8;
-            int32_t member[SHORT];
-            int32_t cursor = head;
+            // Short lists (all of them, in practice) are read once, sorted in
+            // registers and added up in ascending entry order; NOBODY is larger
+            // than any entry number. The wavefront reads until all its lists
+            // have ended: at most four members each is the usual case and has
+            // its own, shorter code; up to eight are sorted likewise; longer
+            // lists are walked once per member.
+            int32_t member[8];
 #pragma unroll
-            for (int j = 0; j < SHORT; j++) {
-                member[j] = cursor;
-                if (cursor != NOBODY) {
-                    cursor = areas.next[cursor];
-                }
+            for (int j = 0; j < 8; j++) {
+                member[j] = NOBODY;
             }
-            if (cursor == NOBODY) {
+            int32_t cursor = head;
+            auto walk = [&](int from, int to) {
 #pragma unroll
-                for (int pass = 0; pass < SHORT; pass++) {
-#pragma unroll
-                    for (int j = pass & 1; j + 1 < SHORT; j += 2) { // odd-even transposition sort
-                        const int32_t low = min(member[j], member[j + 1]);
-                        const int32_t high = max(member[j], member[j + 1]);
-                        member[j] = low;
-                        member[j + 1] = high;
+                for (int j = from; j < to; j++) {
+                    if (__ballot(cursor != NOBODY) == 0) {
+                        break;
+                    }
+                    member[j] = cursor;
+                    if (cursor != NOBODY) {
+                        cursor = areas.next[cursor];
                     }
                 }
-                T value[SHORT];
+            };
+            auto order = [&](int j, int k) {
+                const int32_t low = min(member[j], member[k]);
+                const int32_t high = max(member[j], member[k]);
+                member[j] = low;
+                member[k] = high;
+            };
+            auto add_members = [&](auto count) {
+                constexpr int COUNT = decltype(count)::value;
+                T value[COUNT];
 #pragma unroll
-                for (int j = 0; j < SHORT; j++) {
+                for (int j = 0; j < COUNT; j++) {
                     value[j] = load_or_zero(areas.coefficients, member[j], member[j] != NOBODY);
                 }
 #pragma unroll
-                for (int j = 0; j < SHORT; j++) {
+                for (int j = 0; j < COUNT; j++) {
                     if (member[j] != NOBODY) {
                         sum += value[j];
                     }
                 }
+            };
+            walk(0, 4);
+            if (__ballot(cursor != NOBODY) == 0) {
+                order(0, 1), order(2, 3), order(0, 2), order(1, 3), order(1, 2);
+                add_members(std::integral_constant<int, 4>{});
             } else {
-                int32_t last = -1;
-                for (;;) {
-                    // the smallest member above `last`
-                    int32_t smallest = NOBODY;
-                    for (int32_t k = head; k != NOBODY; k = areas.next[k]) {
-                        if (k > last && k < smallest) {
-                            smallest = k;
+                walk(4, 8);
+                if (cursor == NOBODY) {
+#pragma unroll
+                    for (int pass = 0; pass < 8; pass++) {
+#pragma unroll
+                        for (int j = pass & 1; j + 1 < 8; j += 2) { // odd-even transposition sort
+                            order(j, j + 1);
                         }
                     }
-                    if (smallest == NOBODY) {
-                        break;
+                    add_members(std::integral_constant<int, 8>{});
+                } else {
+                    int32_t last = -1;
+                    for (;;) {
+                        // the smallest member above `last`
+                        int32_t smallest = NOBODY;
+                        for (int32_t k = head; k != NOBODY; k = areas.next[k]) {
+                            if (k > last && k < smallest) {
+                                smallest = k;
+                            }
+                        }
+                        if (smallest == NOBODY) {
+                            break;
+                        }
+                        sum += areas.coefficients[smallest];
+                        last = smallest;
                     }
-                    sum += areas.coefficients[smallest];
-                    last = smallest;
                 }
             }
             // (selects, not an array indexed by role: that would live in scratch memory)
@@ -284,6 +310,16 @@ __device__ __forceinline__ void pair_products(
             }
         }
     };
+    // Two sets of accumulators, used in turn and added at the end: a matrix
+    // instruction that continues the sum of the one before it waits for it.
+    typename M::Acc other[ROW_TILES][NT];
+#pragma unroll
+    for (int r = 0; r < ROW_TILES; r++) {
+#pragma unroll
+        for (int t = 0; t < NT; t++) {
+            other[r][t] = M::zero();
+        }
+    }
     auto multiply = [&](const Step& from) {
 #pragma unroll
         for (int g = 0; g < GROUPS; g++) {
@@ -292,7 +328,11 @@ __device__ __forceinline__ void pair_products(
                 const T product = from.outer[r] * inner[r][g];
 #pragma unroll
                 for (int t = 0; t < NT; t++) {
-                    acc[r][t] = M::mma(product, from.right[g][t], acc[r][t]);
+                    if (g % 2 == 0) {
+                        acc[r][t] = M::mma(product, from.right[g][t], acc[r][t]);
+                    } else {
+                        other[r][t] = M::mma(product, from.right[g][t], other[r][t]);
+                    }
                 }
             }
         }
@@ -309,6 +349,16 @@ __device__ __forceinline__ void pair_products(
     }
     if (x < n_outer) {
         multiply(even);
+    }
+#pragma unroll
+    for (int r = 0; r < ROW_TILES; r++) {
+#pragma unroll
+        for (int t = 0; t < NT; t++) {
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                acc[r][t][e] += other[r][t][e];
+            }
+        }
     }
 }
 
