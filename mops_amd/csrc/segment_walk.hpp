@@ -48,6 +48,11 @@ __device__ __forceinline__ void walk_owned_segments(
     const bool inside = lane < CHUNK && position < n_input;
     const int32_t mine = inside ? sorted_index[position] : 0;
     const int32_t before = (inside && position > 0) ? sorted_index[position - 1] : -1;
+    // the 64 positions after the chunk, asked for now: the last segment of the
+    // chunk almost always ends there, and its end is then known without
+    // another round trip to memory
+    const int32_t ahead_position = chunk_begin + CHUNK + lane;
+    const int32_t ahead = load_or_zero(sorted_index, static_cast<size_t>(ahead_position), ahead_position < n_input);
     const bool starts_here = inside && (position == 0 || mine != before);
 
     unsigned long long starts = __ballot(starts_here);
@@ -66,7 +71,9 @@ __device__ __forceinline__ void walk_owned_segments(
             last = n_input;
             for (int32_t probe = chunk_begin + CHUNK; probe < n_input; probe += WAVE) {
                 const int32_t at = probe + lane;
-                const bool differs = at >= n_input || sorted_index[at] != row;
+                const bool first_look = probe == chunk_begin + CHUNK; // uniform
+                const int32_t value = first_look ? ahead : load_or_zero(sorted_index, static_cast<size_t>(at), at < n_input);
+                const bool differs = at >= n_input || value != row;
                 const unsigned long long mask = __ballot(differs);
                 if (mask != 0) {
                     last = min(probe + __ffsll(static_cast<long long>(mask)) - 1, n_input);
