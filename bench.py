@@ -217,8 +217,8 @@ def capture_steps(workload, steps, device):
 def main_kernel_time(library, function, calls):
     """Average duration (seconds) of the main kernel of ``function`` over ``calls`` eager calls.
 
-    The library records a pair of HIP events around that kernel on the stream
-    it launches it on (mops_amd_kernel_timing in include/mops/amd.h).
+    The library attaches a pair of HIP events to that kernel's launch on the
+    stream it launches it on (mops_amd_kernel_timing in include/mops/amd.h).
     """
     import ctypes
 
@@ -366,10 +366,11 @@ def main():
 
     # ---------------- roofline of the dominant kernel -----------------------
     # At this shape each call is one kernel (mops_amd/csrc/sap_mfma.hip), timed
-    # with a pair of HIP events that the library records around every launch on
-    # the stream the kernel runs on (the pair itself costs about 1 us, which is
-    # inside the figure; consecutive eager calls from Python cannot be used, the
-    # interpreter needs longer per call than the kernel runs).
+    # with a pair of HIP events that the library hands to the launch itself
+    # (hipExtLaunchKernelGGL stamps them with the begin and the end of that
+    # kernel on the stream it runs on). Consecutive eager calls from Python
+    # cannot be used instead: the interpreter needs longer per call than the
+    # kernel runs.
     library = bind_library_to_torch_stream(device)
     kernels = {}
     for kind, function, name in (
@@ -397,7 +398,8 @@ def main():
         "algorithmic_bytes_per_launch": kernel_bytes,
         "avg_launch_us": round(kernel_seconds * 1e6, 3),
         "launches_timed": kernel_launches,
-        "timed": "HIP events around the kernel on its launch stream, eager launches, rotating inputs",
+        "timed": "HIP events attached to the kernel launch (start/stop of that kernel on its launch stream), "
+        "eager launches, rotating inputs",
         "other_kernel_us": {
             kind: None if kernels[kind][0] is None else round(kernels[kind][0] * 1e6, 3) for kind in kernels
         },

@@ -51,9 +51,11 @@ MOPS_EXPORT int mops_amd_first_occurrences(
 /* Device time of the main kernel of each operation (for benchmarks).
  *
  * mops_amd_kernel_timing(1) makes every following mops_cuda_* call of this
- * thread record a pair of HIP events around its main kernel (the one that
- * does the arithmetic; not the small set-up kernels in front of it) on the
- * stream it is launched on. mops_amd_kernel_time waits for the recorded
+ * thread time its main kernel (the one that does the arithmetic; not the
+ * small set-up kernels in front of it) with a pair of HIP events on the
+ * stream it is launched on: attached to the launch itself where the kernel is
+ * launched that way (sparse_accumulation_of_products), recorded just before
+ * and after it otherwise. mops_amd_kernel_time waits for the recorded
  * events, stores the sum of the intervals in milliseconds and their number,
  * and forgets them. Calls captured into a HIP graph are not timed. The first
  * function returns the previous setting, the second 0 / 1 / 2. */

@@ -134,6 +134,23 @@ MainKernelTimer::~MainKernelTimer() {
     }
 }
 
+LaunchEvents launch_events(hipStream_t stream) {
+    auto& st = state();
+    LaunchEvents events;
+    if (!st.timing) {
+        return events;
+    }
+    hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+    MOPS_HIP_CHECK(hipStreamIsCapturing(stream, &capture));
+    if (capture != hipStreamCaptureStatusNone) {
+        return events;
+    }
+    events.start = take_event(st);
+    events.stop = take_event(st);
+    st.recorded.emplace_back(events.start, events.stop);
+    return events;
+}
+
 bool set_kernel_timing(bool value) {
     bool previous = state().timing;
     state().timing = value;

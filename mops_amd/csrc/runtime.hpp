@@ -80,6 +80,16 @@ private:
     hipStream_t stream_;
     hipEvent_t stop_ = nullptr;
 };
+/// The same for a launch through hipExtLaunchKernelGGL, which takes the two
+/// events itself and has them stamped with the begin and the end of that
+/// kernel: no event packets of their own in the stream, so the interval is the
+/// kernel's duration as a profiler reports it. Both are null when timing is off
+/// or the stream is being captured.
+struct LaunchEvents {
+    hipEvent_t start = nullptr;
+    hipEvent_t stop = nullptr;
+};
+LaunchEvents launch_events(hipStream_t stream);
 bool set_kernel_timing(bool value);
 /// Sum (milliseconds) and number of the intervals recorded since the last
 /// call on this thread.

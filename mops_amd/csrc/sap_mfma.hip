@@ -30,6 +30,8 @@
 #include <stdexcept>
 #include <type_traits>
 
+#include <hip/hip_ext.h>
+
 #include "device_common.hpp"
 #include "mfma.hpp"
 #include "runtime.hpp"
@@ -666,11 +668,11 @@ void forward(T* output, const T* A, const T* B, const Table& table, const Shape&
     p.first = operand_shape(s.nA, s.nB, s.nO);
     const unsigned grid = static_cast<unsigned>((s.n_rows + ROWS_PER_GROUP - 1) / ROWS_PER_GROUP);
     const size_t lds = forward_lds(s, sizeof(T));
-    MainKernelTimer timer(stream);
+    const LaunchEvents events = launch_events(stream);
     with_constants<4, 4>(p.first.n_tiles, p.first.n_groups, [&](auto tiles, auto groups) {
         auto kernel = forward_kernel<T, decltype(tiles)::value, decltype(groups)::value>;
         allow_lds(kernel, lds);
-        kernel<<<grid, THREADS, lds, stream>>>(p);
+        hipExtLaunchKernelGGL(kernel, dim3(grid), dim3(THREADS), lds, stream, events.start, events.stop, 0, p);
     });
     MOPS_HIP_CHECK(hipGetLastError());
 }
@@ -688,11 +690,11 @@ void vjp(
     p.second = operand_shape(s.nA, s.nO, s.nB);
     const unsigned grid = static_cast<unsigned>((s.n_rows + ROWS_PER_GROUP - 1) / ROWS_PER_GROUP);
     const size_t lds = vjp_lds(s, sizeof(T), grad_A != nullptr, grad_B != nullptr);
-    MainKernelTimer timer(stream);
+    const LaunchEvents events = launch_events(stream);
     with_constants<1, 16>(1, p.first.n_groups, [&](auto, auto groups) {
         auto kernel = vjp_kernel<T, decltype(groups)::value>;
         allow_lds(kernel, lds);
-        kernel<<<grid, THREADS, lds, stream>>>(p);
+        hipExtLaunchKernelGGL(kernel, dim3(grid), dim3(THREADS), lds, stream, events.start, events.stop, 0, p);
     });
     MOPS_HIP_CHECK(hipGetLastError());
 }
