@@ -724,15 +724,26 @@ void homogeneous_polynomial_evaluation_vjp(MOPS_HPE_VJP_PARAMS(MOPS_CXX_FIRST, M
     hipStream_t stream = current_stream();
     // LDS holds R rows of A and WAVE private accumulator rows, whatever R is
     const size_t accumulator_bytes = static_cast<size_t>(nA) * WAVE * sizeof(scalar_t);
+    // Rows per workgroup: the fewest for which all workgroups are on the
+    // device at once (256 CUs, as many workgroups per CU as the 160 KB of LDS
+    // hold): a second round of workgroups costs more than rows twice as long
+    // (c0: 37 us with 1000 workgroups of one row, 31 us with 500 of two).
     int R = 0;
-    if (accumulator_bytes < LDS_BUDGET) {
-        R = 64;
-        while (R > 1 && (static_cast<size_t>(n_rows) / R < 1024 ||
-                         accumulator_bytes + static_cast<size_t>(nA) * R * sizeof(scalar_t) > LDS_BUDGET)) {
-            R >>= 1;
+    for (int rows = 1; rows <= 64 && R == 0; rows <<= 1) {
+        const size_t lds = accumulator_bytes + static_cast<size_t>(nA) * rows * sizeof(scalar_t);
+        if (lds > LDS_BUDGET) {
+            break;
         }
-        if (accumulator_bytes + static_cast<size_t>(nA) * R * sizeof(scalar_t) > LDS_BUDGET) {
-            R = 0;
+        const size_t resident = 256 * std::max<size_t>(1, (160 * 1024) / lds);
+        if (ceil_div(static_cast<size_t>(n_rows), rows) <= resident || rows == 64) {
+            R = rows;
+        }
+    }
+    if (R == 0 && accumulator_bytes + static_cast<size_t>(nA) * sizeof(scalar_t) <= LDS_BUDGET) {
+        // the tiles of 64 rows do not fit: as many rows as do
+        R = 1;
+        while (accumulator_bytes + static_cast<size_t>(nA) * (2 * R) * sizeof(scalar_t) <= LDS_BUDGET && R < 64) {
+            R <<= 1;
         }
     }
     if (R > 0) {
