@@ -92,6 +92,17 @@ template <typename T> struct MyEntries {
     int32_t index_O[ENTRIES_PER_THREAD];
     T coefficient[ENTRIES_PER_THREAD];
 
+    /// No entries (threads that take part in the build's barriers only).
+    __device__ __forceinline__ void clear() {
+#pragma unroll
+        for (int e = 0; e < ENTRIES_PER_THREAD; e++) {
+            index_A[e] = -1;
+            index_B[e] = 0;
+            index_O[e] = 0;
+            coefficient[e] = T(0);
+        }
+    }
+
     __device__ __forceinline__ void load(
         const T* __restrict__ C, const int32_t* __restrict__ PA, const int32_t* __restrict__ PB,
         const int32_t* __restrict__ PO, int32_t K
@@ -282,7 +293,9 @@ __device__ __forceinline__ void build_operands(
 /// lane's row of the outer values in LDS, row tile r is `outer_tile_stride`
 /// elements further. The LDS reads of step x + 1 are issued before the matrix
 /// instructions of step x; nothing inside the loop is conditional.
-template <typename T, int NT, int GROUPS>
+/// The operand has NT_TOTAL column tiles per (x, g), of which this call uses
+/// the NT from `first_tile` on.
+template <typename T, int NT, int GROUPS, int NT_TOTAL = NT>
 __device__ __forceinline__ void pair_products(
     typename Mfma<T>::Acc (&acc)[ROW_TILES][NT],
     const T* __restrict__ outer_rows,
@@ -290,16 +303,17 @@ __device__ __forceinline__ void pair_products(
     int32_t n_outer,
     const T (&inner)[ROW_TILES][GROUPS],
     const T* __restrict__ operand,
-    int lane
+    int lane,
+    int first_tile = 0
 ) {
     using M = Mfma<T>;
     struct Step {
         T outer[ROW_TILES];
         T right[GROUPS][NT];
     };
-    constexpr int STEP_ELEMENTS = GROUPS * NT * WAVE;
+    constexpr int STEP_ELEMENTS = GROUPS * NT_TOTAL * WAVE;
     auto fetch = [&](Step& to, int32_t x) {
-        const T* right = operand + lane + x * STEP_ELEMENTS;
+        const T* right = operand + lane + x * STEP_ELEMENTS + first_tile * WAVE;
 #pragma unroll
         for (int r = 0; r < ROW_TILES; r++) {
             to.outer[r] = outer_rows[r * outer_tile_stride + x];
@@ -308,7 +322,7 @@ __device__ __forceinline__ void pair_products(
         for (int g = 0; g < GROUPS; g++) {
 #pragma unroll
             for (int t = 0; t < NT; t++) {
-                to.right[g][t] = right[(g * NT + t) * WAVE];
+                to.right[g][t] = right[(g * NT_TOTAL + t) * WAVE];
             }
         }
     };
@@ -390,6 +404,29 @@ __device__ __forceinline__ void stage_rows(
     }
 }
 
+/// Writes NT column tiles of accumulators, from tile `first_tile` on, to LDS
+/// [16][width].
+template <typename T, int NT>
+__device__ __forceinline__ void stage_tiles(
+    T* __restrict__ lds, const typename Mfma<T>::Acc (&acc)[ROW_TILES][NT], int first_tile, int32_t width, int lane
+) {
+    using M = Mfma<T>;
+    const int j = lane & 15;
+#pragma unroll
+    for (int r = 0; r < ROW_TILES; r++) {
+#pragma unroll
+        for (int t = 0; t < NT; t++) {
+            const int32_t column = 16 * (first_tile + t) + j;
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                if (column < width) {
+                    lds[(16 * r + M::row(lane, e)) * width + column] = acc[r][t][e];
+                }
+            }
+        }
+    }
+}
+
 /// Writes a wavefront's accumulators (rows x columns tile by tile) to LDS
 /// [32][width] and from there, contiguously, to global memory.
 template <typename T, int NT>
@@ -454,9 +491,14 @@ size_t build_areas_bytes(const Shape& s, size_t element_size) {
            align16(static_cast<size_t>(s.K) * element_size);
 }
 
+/// Two wavefronts per tile of 16 rows, as in vjp_kernel below: with an even
+/// number of column tiles each takes half of them (otherwise the second one
+/// only helps with loading and storing).
 template <typename T, int NT, int GROUPS>
-__global__ __launch_bounds__(THREADS) void forward_kernel(const Arguments<T> p) {
+__global__ __launch_bounds__(2 * THREADS) void forward_kernel(const Arguments<T> p) {
     using M = Mfma<T>;
+    constexpr bool SPLIT = NT % 2 == 0;
+    constexpr int MY_TILES = SPLIT ? NT / 2 : NT;
     extern __shared__ __align__(16) char lds_raw[];
     char* cursor = lds_raw;
     T* operand = reinterpret_cast<T*>(cursor);
@@ -464,21 +506,29 @@ __global__ __launch_bounds__(THREADS) void forward_kernel(const Arguments<T> p) 
     const BuildAreas<T> areas = carve_build_areas<T>(cursor, p.nA * p.nB * p.nO, p.K);
     const int lane = threadIdx.x & (WAVE - 1);
     const int wave = threadIdx.x >> 6;
+    const int tile = wave & (WAVES - 1);
+    const bool second_half = wave >= WAVES; // uniform per wavefront
     const int32_t row_width = p.nA + p.nB;
     MyEntries<T> entries;
-    entries.load(p.C, p.PA, p.PB, p.PO, p.K);
-    T* mine = reinterpret_cast<T*>(cursor) + wave * ROWS_PER_WAVE * max(row_width, p.nO);
-    T* a_tile = mine;                          // [32][nA]
-    T* b_tile = mine + ROWS_PER_WAVE * p.nA;   // [32][nB]
+    if (second_half) {
+        entries.clear();
+    } else {
+        entries.load(p.C, p.PA, p.PB, p.PO, p.K);
+    }
+    T* mine = reinterpret_cast<T*>(cursor) + tile * ROWS_PER_WAVE * max(row_width, p.nO);
+    T* a_tile = mine;                          // [16][nA]
+    T* b_tile = mine + ROWS_PER_WAVE * p.nA;   // [16][nB]
 
-    const int32_t first_row = (blockIdx.x * WAVES + wave) * ROWS_PER_WAVE;
+    const int32_t first_row = (blockIdx.x * WAVES + tile) * ROWS_PER_WAVE;
     const int32_t valid_rows = p.n_rows - first_row;
     const int32_t safe_first = valid_rows > 0 ? first_row : 0; // wavefronts beyond the end read row 0
-    // this wavefront's rows of A and B
-    stage_rows<T>(a_tile, p.A + static_cast<size_t>(safe_first) * p.nA, p.nA, valid_rows, ROWS_PER_WAVE, lane);
-    stage_rows<T>(b_tile, p.B + static_cast<size_t>(safe_first) * p.nB, p.nB, valid_rows, ROWS_PER_WAVE, lane);
+    if (second_half) {
+        stage_rows<T>(b_tile, p.B + static_cast<size_t>(safe_first) * p.nB, p.nB, valid_rows, ROWS_PER_WAVE, lane);
+    } else {
+        stage_rows<T>(a_tile, p.A + static_cast<size_t>(safe_first) * p.nA, p.nA, valid_rows, ROWS_PER_WAVE, lane);
+    }
     const OperandTarget<T> targets[1] = {{operand, p.first, {0, 1, 2}}};
-    build_operands<T, 1>(targets, areas, p.nA, p.nB, p.nO, entries);
+    build_operands<T, 1>(targets, areas, p.nA, p.nB, p.nO, entries); // ends with a barrier: the tiles are there
 
     const int i = lane & 15;
     const int q = lane >> 4;
@@ -491,24 +541,40 @@ __global__ __launch_bounds__(THREADS) void forward_kernel(const Arguments<T> p) 
             inner[r][g] = load_or_zero(b_tile, (16 * r + i) * p.nB + b, b < p.nB);
         }
     }
-    typename M::Acc acc[ROW_TILES][NT];
+    typename M::Acc acc[ROW_TILES][MY_TILES];
 #pragma unroll
     for (int r = 0; r < ROW_TILES; r++) {
 #pragma unroll
-        for (int t = 0; t < NT; t++) {
+        for (int t = 0; t < MY_TILES; t++) {
             acc[r][t] = M::zero();
         }
     }
-    pair_products<T, NT, GROUPS>(acc, a_tile + i * p.nA, 16 * p.nA, p.nA, inner, operand, lane);
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
+    const int first_tile = SPLIT && second_half ? MY_TILES : 0;
+    const bool computes = SPLIT || !second_half;
+    if (computes) {
+        pair_products<T, MY_TILES, GROUPS, NT>(acc, a_tile + i * p.nA, 16 * p.nA, p.nA, inner, operand, lane, first_tile);
+    }
+    __syncthreads(); // nobody reads the tiles any more: they become the staging area of the store
+    if (computes) {
+        stage_tiles<T, MY_TILES>(mine, acc, first_tile, p.nO, lane);
+    }
+    __syncthreads();
     if (valid_rows > 0) {
-        store_rows<T, NT>(p.output + static_cast<size_t>(first_row) * p.nO, mine, acc, p.nO, valid_rows, lane);
+        // the 16 output rows are contiguous in memory: both wavefronts copy
+        T* target = p.output + static_cast<size_t>(first_row) * p.nO;
+        const int32_t total = min(valid_rows, ROWS_PER_WAVE) * p.nO;
+        for (int32_t at = lane + (second_half ? WAVE : 0); at < total; at += 2 * WAVE) {
+            target[at] = mine[at];
+        }
     }
 }
 
+/// Two wavefronts per tile of 16 rows: wavefront t computes grad_A of tile t,
+/// wavefront t + 8 grad_B, from the same rows in LDS; four wavefronts per SIMD
+/// keep the matrix cores busier than two. The table is built by the first
+/// eight wavefronts' threads (the others only take part in the barriers).
 template <typename T, int GROUPS>
-__global__ __launch_bounds__(THREADS) void vjp_kernel(const Arguments<T> p) {
+__global__ __launch_bounds__(2 * THREADS) void vjp_kernel(const Arguments<T> p) {
     using M = Mfma<T>;
     extern __shared__ __align__(16) char lds_raw[];
     char* cursor = lds_raw;
@@ -521,25 +587,34 @@ __global__ __launch_bounds__(THREADS) void vjp_kernel(const Arguments<T> p) {
     const BuildAreas<T> areas = carve_build_areas<T>(cursor, p.nA * p.nB * p.nO, p.K);
     const int lane = threadIdx.x & (WAVE - 1);
     const int wave = threadIdx.x >> 6;
+    const int tile = wave & (WAVES - 1);
+    const bool second_half = wave >= WAVES; // uniform per wavefront
     const int32_t row_width = p.nA + p.nB + p.nO;
     MyEntries<T> entries;
-    entries.load(p.C, p.PA, p.PB, p.PO, p.K);
-    T* mine = reinterpret_cast<T*>(cursor) + wave * ROWS_PER_WAVE * row_width;
-    T* a_tile = mine;                                  // [32][nA], later grad_A
-    T* b_tile = a_tile + ROWS_PER_WAVE * p.nA;         // [32][nB], later grad_B
-    T* g_tile = b_tile + ROWS_PER_WAVE * p.nB;         // [32][nO]
+    if (second_half) {
+        entries.clear();
+    } else {
+        entries.load(p.C, p.PA, p.PB, p.PO, p.K);
+    }
+    T* mine = reinterpret_cast<T*>(cursor) + tile * ROWS_PER_WAVE * row_width;
+    T* a_tile = mine;                                  // [16][nA]
+    T* b_tile = a_tile + ROWS_PER_WAVE * p.nA;         // [16][nB]
+    T* g_tile = b_tile + ROWS_PER_WAVE * p.nB;         // [16][nO]
 
-    const int32_t first_row = (blockIdx.x * WAVES + wave) * ROWS_PER_WAVE;
+    const int32_t first_row = (blockIdx.x * WAVES + tile) * ROWS_PER_WAVE;
     const int32_t valid_rows = p.n_rows - first_row;
     const int32_t safe_first = valid_rows > 0 ? first_row : 0; // wavefronts beyond the end read row 0
-    stage_rows<T>(a_tile, p.A + static_cast<size_t>(safe_first) * p.nA, p.nA, valid_rows, ROWS_PER_WAVE, lane);
-    stage_rows<T>(b_tile, p.B + static_cast<size_t>(safe_first) * p.nB, p.nB, valid_rows, ROWS_PER_WAVE, lane);
-    stage_rows<T>(g_tile, p.G + static_cast<size_t>(safe_first) * p.nO, p.nO, valid_rows, ROWS_PER_WAVE, lane);
+    if (second_half) {
+        stage_rows<T>(g_tile, p.G + static_cast<size_t>(safe_first) * p.nO, p.nO, valid_rows, ROWS_PER_WAVE, lane);
+    } else {
+        stage_rows<T>(a_tile, p.A + static_cast<size_t>(safe_first) * p.nA, p.nA, valid_rows, ROWS_PER_WAVE, lane);
+        stage_rows<T>(b_tile, p.B + static_cast<size_t>(safe_first) * p.nB, p.nB, valid_rows, ROWS_PER_WAVE, lane);
+    }
     const OperandTarget<T> targets[2] = {
         {want_A ? operand_A : nullptr, p.first, {1, 2, 0}},
         {want_B ? operand_B : nullptr, p.second, {0, 2, 1}},
     };
-    build_operands<T, 2>(targets, areas, p.nA, p.nB, p.nO, entries);
+    build_operands<T, 2>(targets, areas, p.nA, p.nB, p.nO, entries); // ends with a barrier: the tiles are there
 
     const int i = lane & 15;
     const int q = lane >> 4;
@@ -552,27 +627,26 @@ __global__ __launch_bounds__(THREADS) void vjp_kernel(const Arguments<T> p) {
             inner[r][g] = load_or_zero(g_tile, (16 * r + i) * p.nO + o, o < p.nO);
         }
     }
-    typename M::Acc acc_A[ROW_TILES][1];
-    typename M::Acc acc_B[ROW_TILES][1];
+    typename M::Acc acc[ROW_TILES][1];
 #pragma unroll
     for (int r = 0; r < ROW_TILES; r++) {
-        acc_A[r][0] = M::zero();
-        acc_B[r][0] = M::zero();
+        acc[r][0] = M::zero();
     }
-    if (want_A) {
-        pair_products<T, 1, GROUPS>(acc_A, b_tile + i * p.nB, 16 * p.nB, p.nB, inner, operand_A, lane);
-    }
-    if (want_B) {
-        pair_products<T, 1, GROUPS>(acc_B, a_tile + i * p.nA, 16 * p.nA, p.nA, inner, operand_B, lane);
-    }
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    if (valid_rows > 0) {
-        if (want_A) {
-            store_rows<T, 1>(p.grad_A + static_cast<size_t>(first_row) * p.nA, a_tile, acc_A, p.nA, valid_rows, lane);
-        }
+    if (second_half) {
         if (want_B) {
-            store_rows<T, 1>(p.grad_B + static_cast<size_t>(first_row) * p.nB, b_tile, acc_B, p.nB, valid_rows, lane);
+            pair_products<T, 1, GROUPS>(acc, a_tile + i * p.nA, 16 * p.nA, p.nA, inner, operand_B, lane);
+        }
+    } else if (want_A) {
+        pair_products<T, 1, GROUPS>(acc, b_tile + i * p.nB, 16 * p.nB, p.nB, inner, operand_A, lane);
+    }
+    __syncthreads(); // nobody reads the tiles any more: they become the staging areas of the stores
+    if (valid_rows > 0) {
+        if (second_half) {
+            if (want_B) {
+                store_rows<T, 1>(p.grad_B + static_cast<size_t>(first_row) * p.nB, b_tile, acc, p.nB, valid_rows, lane);
+            }
+        } else if (want_A) {
+            store_rows<T, 1>(p.grad_A + static_cast<size_t>(first_row) * p.nA, a_tile, acc, p.nA, valid_rows, lane);
         }
     }
 }
@@ -672,7 +746,7 @@ void forward(T* output, const T* A, const T* B, const Table& table, const Shape&
     with_constants<4, 4>(p.first.n_tiles, p.first.n_groups, [&](auto tiles, auto groups) {
         auto kernel = forward_kernel<T, decltype(tiles)::value, decltype(groups)::value>;
         allow_lds(kernel, lds);
-        hipExtLaunchKernelGGL(kernel, dim3(grid), dim3(THREADS), lds, stream, events.start, events.stop, 0, p);
+        hipExtLaunchKernelGGL(kernel, dim3(grid), dim3(2 * THREADS), lds, stream, events.start, events.stop, 0, p);
     });
     MOPS_HIP_CHECK(hipGetLastError());
 }
@@ -694,7 +768,7 @@ void vjp(
     with_constants<1, 16>(1, p.first.n_groups, [&](auto, auto groups) {
         auto kernel = vjp_kernel<T, decltype(groups)::value>;
         allow_lds(kernel, lds);
-        hipExtLaunchKernelGGL(kernel, dim3(grid), dim3(THREADS), lds, stream, events.start, events.stop, 0, p);
+        hipExtLaunchKernelGGL(kernel, dim3(grid), dim3(2 * THREADS), lds, stream, events.start, events.stop, 0, p);
     });
     MOPS_HIP_CHECK(hipGetLastError());
 }
