@@ -43,7 +43,7 @@ constexpr int WAVES = 8;          // wavefronts per workgroup
 constexpr int ROW_TILES = 1;      // tiles of 16 rows per wavefront
 constexpr int ROWS_PER_WAVE = 16 * ROW_TILES;
 constexpr int ROWS_PER_GROUP = WAVES * ROWS_PER_WAVE;
-constexpr int THREADS = WAVES * WAVE;
+constexpr int THREADS = 2 * WAVES * WAVE; // two wavefronts per tile of 16 rows
 constexpr int MAX_INNER_GROUPS_FORWARD = 4; // nB <= 16
 constexpr int MAX_INNER_GROUPS_VJP = 16;    // nO <= 64
 constexpr int MAX_OUTER = 16;
@@ -91,17 +91,6 @@ template <typename T> struct MyEntries {
     int32_t index_B[ENTRIES_PER_THREAD];
     int32_t index_O[ENTRIES_PER_THREAD];
     T coefficient[ENTRIES_PER_THREAD];
-
-    /// No entries (threads that take part in the build's barriers only).
-    __device__ __forceinline__ void clear() {
-#pragma unroll
-        for (int e = 0; e < ENTRIES_PER_THREAD; e++) {
-            index_A[e] = -1;
-            index_B[e] = 0;
-            index_O[e] = 0;
-            coefficient[e] = T(0);
-        }
-    }
 
     __device__ __forceinline__ void load(
         const T* __restrict__ C, const int32_t* __restrict__ PA, const int32_t* __restrict__ PB,
@@ -495,7 +484,7 @@ size_t build_areas_bytes(const Shape& s, size_t element_size) {
 /// number of column tiles each takes half of them (otherwise the second one
 /// only helps with loading and storing).
 template <typename T, int NT, int GROUPS>
-__global__ __launch_bounds__(2 * THREADS) void forward_kernel(const Arguments<T> p) {
+__global__ __launch_bounds__(THREADS) void forward_kernel(const Arguments<T> p) {
     using M = Mfma<T>;
     constexpr bool SPLIT = NT % 2 == 0;
     constexpr int MY_TILES = SPLIT ? NT / 2 : NT;
@@ -510,11 +499,7 @@ __global__ __launch_bounds__(2 * THREADS) void forward_kernel(const Arguments<T>
     const bool second_half = wave >= WAVES; // uniform per wavefront
     const int32_t row_width = p.nA + p.nB;
     MyEntries<T> entries;
-    if (second_half) {
-        entries.clear();
-    } else {
-        entries.load(p.C, p.PA, p.PB, p.PO, p.K);
-    }
+    entries.load(p.C, p.PA, p.PB, p.PO, p.K);
     T* mine = reinterpret_cast<T*>(cursor) + tile * ROWS_PER_WAVE * max(row_width, p.nO);
     T* a_tile = mine;                          // [16][nA]
     T* b_tile = mine + ROWS_PER_WAVE * p.nA;   // [16][nB]
@@ -571,10 +556,9 @@ __global__ __launch_bounds__(2 * THREADS) void forward_kernel(const Arguments<T>
 
 /// Two wavefronts per tile of 16 rows: wavefront t computes grad_A of tile t,
 /// wavefront t + 8 grad_B, from the same rows in LDS; four wavefronts per SIMD
-/// keep the matrix cores busier than two. The table is built by the first
-/// eight wavefronts' threads (the others only take part in the barriers).
+/// keep the matrix cores busier than two.
 template <typename T, int GROUPS>
-__global__ __launch_bounds__(2 * THREADS) void vjp_kernel(const Arguments<T> p) {
+__global__ __launch_bounds__(THREADS) void vjp_kernel(const Arguments<T> p) {
     using M = Mfma<T>;
     extern __shared__ __align__(16) char lds_raw[];
     char* cursor = lds_raw;
@@ -591,11 +575,7 @@ __global__ __launch_bounds__(2 * THREADS) void vjp_kernel(const Arguments<T> p) 
     const bool second_half = wave >= WAVES; // uniform per wavefront
     const int32_t row_width = p.nA + p.nB + p.nO;
     MyEntries<T> entries;
-    if (second_half) {
-        entries.clear();
-    } else {
-        entries.load(p.C, p.PA, p.PB, p.PO, p.K);
-    }
+    entries.load(p.C, p.PA, p.PB, p.PO, p.K);
     T* mine = reinterpret_cast<T*>(cursor) + tile * ROWS_PER_WAVE * row_width;
     T* a_tile = mine;                                  // [16][nA]
     T* b_tile = a_tile + ROWS_PER_WAVE * p.nA;         // [16][nB]
@@ -746,7 +726,7 @@ void forward(T* output, const T* A, const T* B, const Table& table, const Shape&
     with_constants<4, 4>(p.first.n_tiles, p.first.n_groups, [&](auto tiles, auto groups) {
         auto kernel = forward_kernel<T, decltype(tiles)::value, decltype(groups)::value>;
         allow_lds(kernel, lds);
-        hipExtLaunchKernelGGL(kernel, dim3(grid), dim3(2 * THREADS), lds, stream, events.start, events.stop, 0, p);
+        hipExtLaunchKernelGGL(kernel, dim3(grid), dim3(THREADS), lds, stream, events.start, events.stop, 0, p);
     });
     MOPS_HIP_CHECK(hipGetLastError());
 }
@@ -768,7 +748,7 @@ void vjp(
     with_constants<1, 16>(1, p.first.n_groups, [&](auto, auto groups) {
         auto kernel = vjp_kernel<T, decltype(groups)::value>;
         allow_lds(kernel, lds);
-        hipExtLaunchKernelGGL(kernel, dim3(grid), dim3(2 * THREADS), lds, stream, events.start, events.stop, 0, p);
+        hipExtLaunchKernelGGL(kernel, dim3(grid), dim3(THREADS), lds, stream, events.start, events.stop, 0, p);
     });
     MOPS_HIP_CHECK(hipGetLastError());
 }
