@@ -271,7 +271,8 @@ def main():
     if args.gpus != 1:
         sys.stderr.write(
             "bench.py measures one GPU: every box of this build has a single MI355X and the five "
-            "operations have no multi-GPU path (how they would shard is described in DESIGN.md). "
+            "operations have no multi-GPU path (they would shard over rows / receivers, one gather and one "
+            "reduce-scatter of the weights per call). "
             "Run with --gpus 1.\n"
         )
         sys.exit(2)
