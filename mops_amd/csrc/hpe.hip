@@ -336,7 +336,7 @@ __global__ __launch_bounds__(WAVE) void vjp_ordered_kernel(
                 const T term = prefix[f] * suffix;
                 suffix *= value[f];
                 if (valid[f]) {
-                    mine[now.factor[f] * R] += term;
+                    unsafeAtomicAdd(&mine[now.factor[f] * R], term); // a slot of my own: an add without the round trip of read, add, write
                 }
             }
         }
