@@ -664,7 +664,8 @@ template <typename T> struct EdgeGradArgs {
     FastDivisor by_items, by_lvec, by_L; // n2 * L / vec, L / vec, L
 };
 
-constexpr int EDGE_BATCH = 4; // edges whose W blocks are in LDS together
+constexpr int EDGE_BATCH = 2; // edges whose W blocks are in LDS together (4: more LDS and registers
+                              // per wavefront, 98 instead of 89 us for the whole vjp; 1: 112 us)
 
 template <typename T, int NT, int M2S>
 __global__ __launch_bounds__(WAVE) void edge_gradients_kernel(const EdgeGradArgs<T> p) {
