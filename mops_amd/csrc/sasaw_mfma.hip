@@ -461,17 +461,20 @@ __device__ __forceinline__ void clear_zero_row(T* __restrict__ t_area, const Den
 /// Wavefronts per workgroup (their T areas share 64 KB of LDS) ...
 template <typename T> constexpr int forward_waves() { return 2; }
 /// ... and positions of the sorted index per workgroup, 16 per wavefront.
-template <typename T> constexpr int forward_chunk() { return 2 * STAGE * forward_waves<T>(); }
+/// (32 or 64: 64 when 32 would need more workgroups than the device holds at once)
+constexpr int SHORT_CHUNK = 32;
+constexpr int LONG_CHUNK = 64;
+/// Workgroups of the forward kernel that are on the device together: 256 CUs, 3 wavefronts per SIMD.
+constexpr int32_t FORWARD_RESIDENT_GROUPS = 256 * 6;
 
 /// Segments whose partial sums wait in LDS before the wavefronts meet.
 template <typename T> constexpr int round_segments() { return sizeof(T) == 4 ? 2 : 1; }
 
-template <typename T, int NT, int RS>
+template <typename T, int NT, int RS, int FORWARD_CHUNK>
 __global__ __launch_bounds__(forward_waves<T>() * WAVE) void forward_kernel(
     T* __restrict__ output, const int32_t* __restrict__ receivers, int32_t n_edges, const Contraction<T> p
 ) {
     constexpr int FORWARD_WAVES = forward_waves<T>();
-    constexpr int FORWARD_CHUNK = forward_chunk<T>();
     constexpr int ROUND_SEGMENTS = round_segments<T>();
     constexpr int TILE = NT * 4 * WAVE; // elements of one wavefront's partial sums
     extern __shared__ __align__(16) char lds_raw[];
@@ -1095,11 +1098,20 @@ void forward(
     const DenseBuffers<T> dense = enqueue_dense<T>(workspace, layout, C, indices, s, stream);
     const Contraction<T> c =
         contraction<T>(A, B, W, indices.W_1, dense.to_cells, layout, s, s.n3, s.n2, s.n2, 1);
-    const int32_t grid = (s.n_edges + forward_chunk<T>() - 1) / forward_chunk<T>();
+    // positions of the sorted index per workgroup: one stage per wavefront while all
+    // workgroups still fit on the device together, else two
+    const bool short_chunks = (s.n_edges + SHORT_CHUNK - 1) / SHORT_CHUNK <= FORWARD_RESIDENT_GROUPS;
+    const int32_t chunk = short_chunks ? SHORT_CHUNK : LONG_CHUNK;
+    const int32_t grid = (s.n_edges + chunk - 1) / chunk;
     const size_t lds = forward_lds(s, sizeof(T));
     with_shape_constants(tiles_for(s.L), (s.n2 + 3) / 4, [&](auto tiles, auto steps) {
-        forward_kernel<T, decltype(tiles)::value, decltype(steps)::value>
-            <<<grid, forward_waves<T>() * WAVE, lds, stream>>>(output, indices.output_1, s.n_edges, c);
+        if (short_chunks) {
+            forward_kernel<T, decltype(tiles)::value, decltype(steps)::value, SHORT_CHUNK>
+                <<<grid, forward_waves<T>() * WAVE, lds, stream>>>(output, indices.output_1, s.n_edges, c);
+        } else {
+            forward_kernel<T, decltype(tiles)::value, decltype(steps)::value, LONG_CHUNK>
+                <<<grid, forward_waves<T>() * WAVE, lds, stream>>>(output, indices.output_1, s.n_edges, c);
+        }
     });
     MOPS_HIP_CHECK(hipGetLastError());
 }
