@@ -526,7 +526,16 @@ __global__ __launch_bounds__(256) void gather_weights_kernel(
 // receivers add up in the same accumulators. Two dependent round trips to
 // memory (index, then grad_output), every wavefront the same amount of work.
 // ---------------------------------------------------------------------------
-template <typename T, int KT, int NT, bool WEIGHTED>
+//
+// VECTORS: the rows of B, W and grad_output are read 16 bytes at a time (L a
+// multiple of the vector length, pointers aligned). A lane's vector then holds
+// VL consecutive l, so the reduction over l is taken in a different ORDER than
+// l = 4 s + q: vector v, component c is step s = VL v + c and stands for
+// l = 4 VL v + VL q + c, in the left and in the right operand alike. One
+// 16-byte load per lane replaces VL loads that each touch 16 cache lines,
+// which is what these kernels otherwise spend their time on (address
+// processing, not bandwidth).
+template <typename T, int KT, int NT, bool WEIGHTED, bool VECTORS>
 __global__ __launch_bounds__(WAVE) void edge_rows_vjp_kernel(
     T* __restrict__ grad_A,
     T* __restrict__ grad_B,
@@ -562,16 +571,44 @@ __global__ __launch_bounds__(WAVE) void edge_rows_vjp_kernel(
     }
     const bool sender_ok = !WEIGHTED || in_bounds(my_sender, n_output);
 
-    // left operands: lane (row = edge i, reduction index 4 s + q)
+    constexpr int VL = 16 / sizeof(T); // elements of a 16-byte vector
+    typedef T Wide __attribute__((ext_vector_type(VL)));
+    constexpr int L_VECTORS = L_STEPS / VL;
+    auto wide_or_zero = [](const T* pointer, size_t index, bool ok) {
+        const Wide value = *reinterpret_cast<const Wide*>(pointer + (ok ? index : 0));
+        Wide zero;
+#pragma unroll
+        for (int c = 0; c < VL; c++) {
+            zero[c] = T(0);
+        }
+        return ok ? value : zero;
+    };
+    // left operands: lane (row = edge i, reduction index 4 s + q; with VECTORS see above)
     T b_left[L_STEPS]; // (B * W)[e, l]
     T a_left[K_STEPS]; // A[e, k]
+    if constexpr (VECTORS) {
 #pragma unroll
-    for (int s = 0; s < L_STEPS; s++) {
-        const int32_t l = 4 * s + q;
-        const bool ok = my_edge >= 0 && l < L;
-        b_left[s] = load_or_zero(B, static_cast<size_t>(my_edge) * L + l, ok && want_A);
-        if constexpr (WEIGHTED) {
-            b_left[s] *= load_or_zero(W, static_cast<size_t>(my_sender) * L + l, ok && want_A && sender_ok);
+        for (int v = 0; v < L_VECTORS; v++) {
+            const int32_t l = 4 * VL * v + VL * q;
+            const bool ok = my_edge >= 0 && l < L;
+            Wide b = wide_or_zero(B, static_cast<size_t>(my_edge) * L + l, ok && want_A);
+            if constexpr (WEIGHTED) {
+                b *= wide_or_zero(W, static_cast<size_t>(my_sender) * L + l, ok && want_A && sender_ok);
+            }
+#pragma unroll
+            for (int c = 0; c < VL; c++) {
+                b_left[VL * v + c] = b[c];
+            }
+        }
+    } else {
+#pragma unroll
+        for (int s = 0; s < L_STEPS; s++) {
+            const int32_t l = 4 * s + q;
+            const bool ok = my_edge >= 0 && l < L;
+            b_left[s] = load_or_zero(B, static_cast<size_t>(my_edge) * L + l, ok && want_A);
+            if constexpr (WEIGHTED) {
+                b_left[s] *= load_or_zero(W, static_cast<size_t>(my_sender) * L + l, ok && want_A && sender_ok);
+            }
         }
     }
 #pragma unroll
@@ -621,20 +658,38 @@ __global__ __launch_bounds__(WAVE) void edge_rows_vjp_kernel(
             const bool mine = my_node == node;
             const T* block = grad_output + static_cast<size_t>(node) * K * L;
             if (want_A) {
-                // right operand: lane (column k = 16 t + i, reduction index l = 4 s + q)
+                // right operand: lane (column k = 16 t + i, reduction index l = 4 s + q,
+                // or the order of the vectors)
                 T right[L_STEPS][KT];
+                if constexpr (VECTORS) {
 #pragma unroll
-                for (int s = 0; s < L_STEPS; s++) {
-                    const int32_t l = 4 * s + q;
+                    for (int v = 0; v < L_VECTORS; v++) {
+                        const int32_t l = 4 * VL * v + VL * q;
 #pragma unroll
-                    for (int t = 0; t < KT; t++) {
-                        const int32_t k = 16 * t + i;
-                        right[s][t] = load_or_zero(block, k * L + l, k < K && l < L);
+                        for (int t = 0; t < KT; t++) {
+                            const int32_t k = 16 * t + i;
+                            const Wide values = wide_or_zero(block, static_cast<size_t>(k) * L + l, k < K && l < L);
+#pragma unroll
+                            for (int c = 0; c < VL; c++) {
+                                right[VL * v + c][t] = values[c];
+                            }
+                        }
+                    }
+                } else {
+#pragma unroll
+                    for (int s = 0; s < L_STEPS; s++) {
+                        const int32_t l = 4 * s + q;
+#pragma unroll
+                        for (int t = 0; t < KT; t++) {
+                            const int32_t k = 16 * t + i;
+                            right[s][t] = load_or_zero(block, k * L + l, k < K && l < L);
+                        }
                     }
                 }
 #pragma unroll
                 for (int s = 0; s < L_STEPS; s++) {
-                    if (s < l_steps) {
+                    // steps whose l are all beyond L are left out (with VECTORS: whole vectors)
+                    if (VECTORS ? 4 * VL * (s / VL) < L : s < l_steps) {
                         const T left = mine ? b_left[s] : T(0);
 #pragma unroll
                         for (int t = 0; t < KT; t++) {
@@ -979,11 +1034,22 @@ void launch_vjp(
         } else if (K <= 32 && L <= 64) {
             const unsigned groups = static_cast<unsigned>(ceil_div(static_cast<size_t>(n_edges), 16));
             MainKernelTimer timer(stream);
+            const bool vectors = L % (16 / static_cast<int32_t>(sizeof(T))) == 0 &&
+                                 reinterpret_cast<uintptr_t>(B.data) % 16 == 0 &&
+                                 reinterpret_cast<uintptr_t>(grad_output.data) % 16 == 0 &&
+                                 (!WEIGHTED || reinterpret_cast<uintptr_t>(W) % 16 == 0);
 #define MOPS_LAUNCH_ROWS(KT, NT)                                                                   \
-    edge_rows_vjp_kernel<T, KT, NT, WEIGHTED><<<groups, WAVE, 0, stream>>>(                        \
-        grad_A.data, grad_B.data, edge_W, grad_output.data, A.data, B.data, W, indices_W,          \
-        indices_output.data, n_edges, n_output, K, L                                               \
-    )
+    if (vectors) {                                                                                 \
+        edge_rows_vjp_kernel<T, KT, NT, WEIGHTED, true><<<groups, WAVE, 0, stream>>>(              \
+            grad_A.data, grad_B.data, edge_W, grad_output.data, A.data, B.data, W, indices_W,      \
+            indices_output.data, n_edges, n_output, K, L                                           \
+        );                                                                                         \
+    } else {                                                                                       \
+        edge_rows_vjp_kernel<T, KT, NT, WEIGHTED, false><<<groups, WAVE, 0, stream>>>(             \
+            grad_A.data, grad_B.data, edge_W, grad_output.data, A.data, B.data, W, indices_W,      \
+            indices_output.data, n_edges, n_output, K, L                                           \
+        );                                                                                         \
+    }
             if (K <= 16) {
                 if (L <= 16) {
                     MOPS_LAUNCH_ROWS(1, 1);
