@@ -611,10 +611,33 @@ __global__ __launch_bounds__(WAVE) void edge_rows_vjp_kernel(
             }
         }
     }
+    // The 16 rows of A are one contiguous piece of memory: read as such (a few
+    // cache lines per load instead of 16) and handed to the operand layout
+    // through LDS.
+    __shared__ T a_tile[16 * 16 * KT];
+    {
+        constexpr int LOADS = (16 * 16 * KT + WAVE - 1) / WAVE;
+        const int32_t tile_elements = n * K;
+        T piece[LOADS];
+#pragma unroll
+        for (int u = 0; u < LOADS; u++) {
+            const int32_t at = u * WAVE + lane;
+            piece[u] = load_or_zero(A, static_cast<size_t>(first_edge) * K + at, at < tile_elements && (want_B || want_W));
+        }
+#pragma unroll
+        for (int u = 0; u < LOADS; u++) {
+            a_tile[u * WAVE + lane] = piece[u];
+        }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 #pragma unroll
     for (int s = 0; s < K_STEPS; s++) {
         const int32_t k = 4 * s + q;
-        a_left[s] = load_or_zero(A, static_cast<size_t>(my_edge) * K + k, my_edge >= 0 && k < K && (want_B || want_W));
+        const bool ok = my_edge >= 0 && k < K;
+        const T value = a_tile[ok ? i * K + k : 0];
+        a_left[s] = ok ? value : T(0);
     }
 
     // factors of the results, per accumulator element (row = edge, column l = 16 t + i):
