@@ -126,9 +126,11 @@ template <int NW> struct SenderGather {
                         values[u][0] = ok ? values[u][0] : -1;
                     }
                 }
-                // Matches are rare (one lane in a few hundred), so they are
-                // handled one at a time by the whole wavefront: a uniform loop
-                // over the lanes that found something, in lane (= edge) order.
+                // The matches of one load go to the list together: every lane
+                // counts its own, the lanes before it give its place (sums of
+                // ballots over the bits of the counts: no loop over matches, no
+                // scalar branches), and it writes them itself. Lane order, then
+                // component order, is ascending edge order.
                 int consumed = 0;
 #pragma unroll
                 for (int u = 0; u < BATCH; u++) {
@@ -140,25 +142,27 @@ template <int NW> struct SenderGather {
                     for (int c = 0; c < VEC; c++) {
                         found |= in_bounds(values[u][c] - node0, served) ? (1u << c) : 0u;
                     }
-                    unsigned long long finders = __ballot(found != 0);
-                    if (count + VEC * __popcll(finders) > CAPACITY) {
-                        full = true;
-                        continue;
-                    }
-                    while (finders != 0) {
-                        const int finder = __ffsll(static_cast<long long>(finders)) - 1;
-                        finders &= finders - 1;
-                        const uint32_t bits = __builtin_amdgcn_readlane(found, finder);
+                    if (__ballot(found != 0) != 0) {
+                        const uint32_t mine = __popc(found); // 0..VEC, VEC <= 4
+                        const unsigned long long ones = __ballot((mine & 1u) != 0);
+                        const unsigned long long twos = __ballot((mine & 2u) != 0);
+                        const unsigned long long fours = __ballot((mine & 4u) != 0);
+                        const int32_t total = __popcll(ones) + 2 * __popcll(twos) + 4 * __popcll(fours);
+                        if (count + total > CAPACITY) {
+                            full = true;
+                            continue;
+                        }
+                        const int32_t before =
+                            __popcll(ones & below) + 2 * __popcll(twos & below) + 4 * __popcll(fours & below);
 #pragma unroll
                         for (int c = 0; c < VEC; c++) {
-                            if (bits & (1u << c)) {
-                                const int32_t value = __builtin_amdgcn_readlane(values[u][c], finder);
-                                // every lane writes the same value to the same place
-                                lds.edges[wave][count] = (unit + u) * UNIT + finder * VEC + c;
-                                lds.which[wave][count] = static_cast<uint8_t>(value - node0);
-                                count++;
+                            if (found & (1u << c)) {
+                                const int32_t slot = count + before + __popc(found & ((1u << c) - 1u));
+                                lds.edges[wave][slot] = (unit + u) * UNIT + lane * VEC + c;
+                                lds.which[wave][slot] = static_cast<uint8_t>(values[u][c] - node0);
                             }
                         }
+                        count += total;
                     }
                     consumed = u + 1;
                 }
