@@ -733,6 +733,53 @@ __global__ __launch_bounds__(WAVE) void edge_gradients_kernel(const EdgeGradArgs
     // left operand of grad_A = U * D: lane (edge = i, cell = 4 step + q), step as immediate
     const uint32_t u_by_edge = (q * T_ROW + i) * ELEMENT;
 
+    // W blocks on their way to LDS: 16-byte vectors in registers, asked for one
+    // batch ahead so that a batch does not start with a round trip to memory
+    typedef T Vec __attribute__((ext_vector_type(4)));
+    constexpr int ROUND = 3;
+    struct RowsOnTheWay {
+        Vec loaded[ROUND];
+        uint32_t where[ROUND];
+        bool ok[ROUND];
+    };
+    const uint32_t items_per_edge = p.by_items.divisor;
+    const uint32_t lvecs = p.by_lvec.divisor;
+    const int32_t block_elements = p.n2 * p.L;
+    auto ask_for_rows = [&](RowsOnTheWay& to, int32_t k0, int32_t n_batch, uint32_t base) {
+        const uint32_t total = static_cast<uint32_t>(n_batch) * items_per_edge;
+#pragma unroll
+        for (int u = 0; u < ROUND; u++) {
+            const uint32_t item = base + u * WAVE + lane;
+            to.ok[u] = item < total;
+            const uint32_t safe = to.ok[u] ? item : 0;
+            const uint32_t kw = p.by_items.divide(safe);
+            const uint32_t rest = safe - kw * items_per_edge;
+            const uint32_t row = p.by_lvec.divide(rest);
+            const uint32_t lv = rest - row * lvecs;
+            const int32_t source = __shfl(my_source, k0 + static_cast<int>(kw));
+            const bool valid = to.ok[u] && in_bounds(source, p.n_nodes);
+            const size_t from = valid ? static_cast<size_t>(source) * block_elements + rest * 4 : 0;
+            const Vec value = *reinterpret_cast<const Vec*>(p.W + from);
+            to.loaded[u] = valid ? value : Vec(T(0));
+            to.where[u] = (kw * p.n2 + row) * p.Ls + lv * 4;
+        }
+    };
+    auto commit_rows = [&](const RowsOnTheWay& from) {
+#pragma unroll
+        for (int u = 0; u < ROUND; u++) {
+            if (from.ok[u]) {
+#pragma unroll
+                for (int v = 0; v < 4; v++) {
+                    w_lds[from.where[u] + v] = from.loaded[u][v];
+                }
+            }
+        }
+    };
+    RowsOnTheWay ahead;
+    if (p.vector_loads) {
+        ask_for_rows(ahead, 0, min(EDGE_BATCH, n), 0);
+    }
+
     __syncthreads();
     if (want_B) {
         T a_rows[MAX_A_STEPS];
@@ -756,47 +803,22 @@ __global__ __launch_bounds__(WAVE) void edge_gradients_kernel(const EdgeGradArgs
         g_left[s] = T(0);
     }
 
-    const uint32_t items_per_edge = p.by_items.divisor;
-    const uint32_t lvecs = p.by_lvec.divisor;
-    const int32_t block_elements = p.n2 * p.L;
-
     for (int32_t k0 = 0; k0 < n; k0 += EDGE_BATCH) {
         const int32_t n_batch = min(EDGE_BATCH, n - k0);
         __syncthreads(); // the previous batch is no longer read
         // ---- W blocks and B rows of the batch into LDS
         if (p.vector_loads) {
-            typedef T Vec __attribute__((ext_vector_type(4)));
-            constexpr int ROUND = 5;
+            // the first ROUND x 64 vectors of the batch were asked for one batch
+            // ago; what a large block has beyond them is read now
+            commit_rows(ahead);
             const uint32_t total = static_cast<uint32_t>(n_batch) * items_per_edge;
-            for (uint32_t base = 0; base < total; base += ROUND * WAVE) {
-                Vec loaded[ROUND];
-                uint32_t where[ROUND];
-                bool ok[ROUND];
-#pragma unroll
-                for (int u = 0; u < ROUND; u++) {
-                    const uint32_t item = base + u * WAVE + lane;
-                    ok[u] = item < total;
-                    const uint32_t safe = ok[u] ? item : 0;
-                    const uint32_t kw = p.by_items.divide(safe);
-                    const uint32_t rest = safe - kw * items_per_edge;
-                    const uint32_t row = p.by_lvec.divide(rest);
-                    const uint32_t lv = rest - row * lvecs;
-                    const int32_t source = __shfl(my_source, k0 + static_cast<int>(kw));
-                    const bool valid = ok[u] && in_bounds(source, p.n_nodes);
-                    const size_t from = valid ? static_cast<size_t>(source) * block_elements + rest * 4 : 0;
-                    const Vec value = *reinterpret_cast<const Vec*>(p.W + from);
-                    loaded[u] = valid ? value : Vec(T(0));
-                    where[u] = (kw * p.n2 + row) * p.Ls + lv * 4;
-                }
-#pragma unroll
-                for (int u = 0; u < ROUND; u++) {
-                    if (ok[u]) {
-#pragma unroll
-                        for (int v = 0; v < 4; v++) {
-                            w_lds[where[u] + v] = loaded[u][v];
-                        }
-                    }
-                }
+            for (uint32_t base = ROUND * WAVE; base < total; base += ROUND * WAVE) {
+                RowsOnTheWay more;
+                ask_for_rows(more, k0, n_batch, base);
+                commit_rows(more);
+            }
+            if (k0 + EDGE_BATCH < n) {
+                ask_for_rows(ahead, k0 + EDGE_BATCH, min(EDGE_BATCH, n - k0 - EDGE_BATCH), 0);
             }
         } else {
             const uint32_t total = static_cast<uint32_t>(n_batch) * items_per_edge;
