@@ -73,6 +73,9 @@ def build_configs():
         ("c3", "opsaw", np.float32, support.opsaw_case(3, np.float32)),
         ("c4", "sasaw", np.float32, support.sasaw_case(4, np.float32)),
         ("c4", "sasaw", np.float64, support.sasaw_case(4, np.float64)),
+        # beyond the BASELINE shapes: feature counts that fill whole 16-wide matrix tiles
+        ("wide", "opsa", np.float32, support.opsa_case(5, np.float32, K=32, L=64)),
+        ("wide", "opsaw", np.float32, support.opsaw_case(6, np.float32, K=32, L=64)),
     ]
 
 
@@ -101,8 +104,11 @@ class DeviceWorkload:
                 tensors["grad_" + name] = torch.empty_like(tensors[name])
             self.sets.append(tensors)
         self.cursor = 0
+        self.rotate = True
 
     def _next(self):
+        if not self.rotate:
+            return self.sets[0]  # the same buffers every call: whatever the caches keep stays
         tensors = self.sets[self.cursor]
         self.cursor = (self.cursor + 1) % self.n_sets
         return tensors
@@ -290,8 +296,8 @@ def main():
     configs = build_configs()
 
     if args.profile:
-        for _, op_name, _, op_case in configs:
-            if args.profile in (op_name, "all"):
+        for config, op_name, _, op_case in configs:
+            if config != "wide" and args.profile in (op_name, "all"):
                 w = DeviceWorkload(op_name, op_case, device)
                 for _ in range(50):
                     w.step()
@@ -351,6 +357,10 @@ def main():
                 "hbm_frac": round(abytes / seconds / 1e9 / HBM_PEAK_GBS, 4),
                 "timed": "hip-graph replay, HIP events" if captured else "eager launches, HIP events",
             }
+            w.rotate = False
+            warm_seconds, _ = device_time_per_call(function, calls, 20, device)
+            w.rotate = True
+            entry["device_us_same_buffers"] = round(warm_seconds * 1e6, 3)
             if not args.no_per_op:
                 cpu_function = (
                     (lambda c=op_case, o=op_name: support.cpu_forward(oracle, o, c))

@@ -89,28 +89,53 @@ __device__ __forceinline__ void forward_segment(
             for (int32_t e0 = first; e0 < last; e0 += 4 * UNROLL) {
                 T a[UNROLL];
                 T b[UNROLL][NT];
+                T w[WEIGHTED ? UNROLL : 1][NT];
+                int32_t w_row[UNROLL];
+                if (WEIGHTED) {
+#pragma unroll
+                    for (int u = 0; u < UNROLL; u++) {
+                        const int32_t e = e0 + 4 * u + quarter;
+                        const int32_t loaded = indices_W[e < last ? e : first];
+                        w_row[u] = e < last ? loaded : -1;
+                    }
+                }
 #pragma unroll
                 for (int u = 0; u < UNROLL; u++) {
                     const int32_t e = e0 + 4 * u + quarter;
                     const bool e_ok = e < last;
                     a[u] = load_or_zero(A, static_cast<size_t>(e) * K + k, e_ok && k_ok);
-                    int32_t w_row = -1;
-                    if (WEIGHTED) {
-                        const int32_t loaded = indices_W[e_ok ? e : first];
-                        w_row = e_ok ? loaded : -1;
-                    }
 #pragma unroll
                     for (int t = 0; t < NT; t++) {
                         const int32_t col = l0 + 16 * t + sub;
-                        T value = load_or_zero(B, static_cast<size_t>(e) * L + col, e_ok && col < L);
-                        if (WEIGHTED) {
-                            value *= load_or_zero(
+                        b[u][t] = load_or_zero(B, static_cast<size_t>(e) * L + col, e_ok && col < L);
+                    }
+                }
+                if (WEIGHTED) {
+#pragma unroll
+                    for (int u = 0; u < UNROLL; u++) {
+#pragma unroll
+                        for (int t = 0; t < NT; t++) {
+                            const int32_t col = l0 + 16 * t + sub;
+                            w[u][t] = load_or_zero(
                                 W,
-                                static_cast<size_t>(w_row) * L + col,
-                                in_bounds(w_row, n_weights) && col < L
+                                static_cast<size_t>(w_row[u]) * L + col,
+                                in_bounds(w_row[u], n_weights) && col < L
                             );
                         }
-                        b[u][t] = value;
+                    }
+                    // every load is asked for before the first product needs one:
+                    // left to itself the compiler chains them in the widest variant,
+                    // each waiting for the one before (its own order is kept for the
+                    // narrower ones, where it measured a little faster)
+                    if (NT >= 4) {
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+#pragma unroll
+                    for (int u = 0; u < UNROLL; u++) {
+#pragma unroll
+                        for (int t = 0; t < NT; t++) {
+                            b[u][t] *= w[u][t];
+                        }
                     }
                 }
                 // keep every load above ahead of the first matrix instruction:
@@ -511,8 +536,8 @@ __global__ __launch_bounds__(256) void gather_weights_kernel(
 }
 
 // ---------------------------------------------------------------------------
-// vjp for moderate feature counts (K <= 32, L <= 64), the shapes of the
-// reference's benchmarks: the gradients are per EDGE, so nothing has to follow
+// vjp for K <= 32 (any L; beyond 64 columns in passes of 64, see BLOCKS), which
+// includes the shapes of the reference's benchmarks: the gradients are per EDGE, so nothing has to follow
 // the segments. A wavefront takes 16 consecutive edges, whatever receivers
 // they have: it knows which rows of A, B (and W) it needs before it has seen
 // any index, all its loads go straight from global memory into matrix
@@ -535,7 +560,7 @@ __global__ __launch_bounds__(256) void gather_weights_kernel(
 // 16-byte load per lane replaces VL loads that each touch 16 cache lines,
 // which is what these kernels otherwise spend their time on (address
 // processing, not bandwidth).
-template <typename T, int KT, int NT, bool WEIGHTED, bool VECTORS>
+template <typename T, int KT, int NT, bool WEIGHTED, bool VECTORS, bool BLOCKS>
 __global__ __launch_bounds__(WAVE) void edge_rows_vjp_kernel(
     T* __restrict__ grad_A,
     T* __restrict__ grad_B,
@@ -584,12 +609,15 @@ __global__ __launch_bounds__(WAVE) void edge_rows_vjp_kernel(
         return ok ? value : zero;
     };
     // left operands: lane (row = edge i, reduction index 4 s + q; with VECTORS see above)
+    // BLOCKS: L is wider than the 16 NT columns of one pass; the passes follow each
+    // other, grad_A collects over all of them, the columns of grad_B are per pass
     T b_left[L_STEPS]; // (B * W)[e, l]
     T a_left[K_STEPS]; // A[e, k]
+    auto load_b_left = [&](int32_t l_base) {
     if constexpr (VECTORS) {
 #pragma unroll
         for (int v = 0; v < L_VECTORS; v++) {
-            const int32_t l = 4 * VL * v + VL * q;
+            const int32_t l = l_base + 4 * VL * v + VL * q;
             const bool ok = my_edge >= 0 && l < L;
             Wide b = wide_or_zero(B, static_cast<size_t>(my_edge) * L + l, ok && want_A);
             if constexpr (WEIGHTED) {
@@ -603,7 +631,7 @@ __global__ __launch_bounds__(WAVE) void edge_rows_vjp_kernel(
     } else {
 #pragma unroll
         for (int s = 0; s < L_STEPS; s++) {
-            const int32_t l = 4 * s + q;
+            const int32_t l = l_base + 4 * s + q;
             const bool ok = my_edge >= 0 && l < L;
             b_left[s] = load_or_zero(B, static_cast<size_t>(my_edge) * L + l, ok && want_A);
             if constexpr (WEIGHTED) {
@@ -611,6 +639,8 @@ __global__ __launch_bounds__(WAVE) void edge_rows_vjp_kernel(
             }
         }
     }
+    };
+    load_b_left(0);
     // The 16 rows of A are one contiguous piece of memory: read as such (a few
     // cache lines per load instead of 16) and handed to the operand layout
     // through LDS.
@@ -640,6 +670,15 @@ __global__ __launch_bounds__(WAVE) void edge_rows_vjp_kernel(
         a_left[s] = ok ? value : T(0);
     }
 
+    typename M::Acc acc_A[KT];
+#pragma unroll
+    for (int t = 0; t < KT; t++) {
+        acc_A[t] = M::zero();
+    }
+    const int32_t k_steps = (K + 3) >> 2;
+
+    for (int32_t next_base = 0;;) {
+    const int32_t l_base = BLOCKS ? next_base : 0;
     // factors of the results, per accumulator element (row = edge, column l = 16 t + i):
     // asked for now, needed after the matrix products
     T weight_out[NT][4];
@@ -650,7 +689,7 @@ __global__ __launch_bounds__(WAVE) void edge_rows_vjp_kernel(
 #pragma unroll
             for (int r = 0; r < 4; r++) {
                 const int32_t row = M::row(lane, r);
-                const int32_t l = 16 * t + i;
+                const int32_t l = l_base + 16 * t + i;
                 const bool ok = row < n && l < L;
                 const int32_t sender = __shfl(my_sender, row);
                 weight_out[t][r] = load_or_zero(
@@ -661,19 +700,13 @@ __global__ __launch_bounds__(WAVE) void edge_rows_vjp_kernel(
         }
     }
 
-    typename M::Acc acc_A[KT];
     typename M::Acc acc_B[NT];
-#pragma unroll
-    for (int t = 0; t < KT; t++) {
-        acc_A[t] = M::zero();
-    }
 #pragma unroll
     for (int t = 0; t < NT; t++) {
         acc_B[t] = M::zero();
     }
 
-    const int32_t l_steps = (L + 3) >> 2;
-    const int32_t k_steps = (K + 3) >> 2;
+    const int32_t l_steps = (L - l_base + 3) >> 2;
     // the receivers among my edges, in ascending order (the index is sorted)
     int32_t node = __builtin_amdgcn_readfirstlane(my_node);
     while (node >= 0) {
@@ -687,7 +720,7 @@ __global__ __launch_bounds__(WAVE) void edge_rows_vjp_kernel(
                 if constexpr (VECTORS) {
 #pragma unroll
                     for (int v = 0; v < L_VECTORS; v++) {
-                        const int32_t l = 4 * VL * v + VL * q;
+                        const int32_t l = l_base + 4 * VL * v + VL * q;
 #pragma unroll
                         for (int t = 0; t < KT; t++) {
                             const int32_t k = 16 * t + i;
@@ -701,7 +734,7 @@ __global__ __launch_bounds__(WAVE) void edge_rows_vjp_kernel(
                 } else {
 #pragma unroll
                     for (int s = 0; s < L_STEPS; s++) {
-                        const int32_t l = 4 * s + q;
+                        const int32_t l = l_base + 4 * s + q;
 #pragma unroll
                         for (int t = 0; t < KT; t++) {
                             const int32_t k = 16 * t + i;
@@ -712,7 +745,7 @@ __global__ __launch_bounds__(WAVE) void edge_rows_vjp_kernel(
 #pragma unroll
                 for (int s = 0; s < L_STEPS; s++) {
                     // steps whose l are all beyond L are left out (with VECTORS: whole vectors)
-                    if (VECTORS ? 4 * VL * (s / VL) < L : s < l_steps) {
+                    if (VECTORS ? l_base + 4 * VL * (s / VL) < L : s < l_steps) {
                         const T left = mine ? b_left[s] : T(0);
 #pragma unroll
                         for (int t = 0; t < KT; t++) {
@@ -729,7 +762,7 @@ __global__ __launch_bounds__(WAVE) void edge_rows_vjp_kernel(
                     const int32_t k = 4 * s + q;
 #pragma unroll
                     for (int t = 0; t < NT; t++) {
-                        const int32_t l = 16 * t + i;
+                        const int32_t l = l_base + 16 * t + i;
                         right[s][t] = load_or_zero(block, k * L + l, k < K && l < L);
                     }
                 }
@@ -750,26 +783,13 @@ __global__ __launch_bounds__(WAVE) void edge_rows_vjp_kernel(
     }
 
     // accumulators: lane (column = 16 t + i, rows = edges M::row(lane, r))
-    if (want_A) {
-#pragma unroll
-        for (int t = 0; t < KT; t++) {
-#pragma unroll
-            for (int r = 0; r < 4; r++) {
-                const int32_t row = M::row(lane, r);
-                const int32_t k = 16 * t + i;
-                if (row < n && k < K) {
-                    grad_A[static_cast<size_t>(first_edge + row) * K + k] = acc_A[t][r];
-                }
-            }
-        }
-    }
     if (want_B || want_W) {
 #pragma unroll
         for (int t = 0; t < NT; t++) {
 #pragma unroll
             for (int r = 0; r < 4; r++) {
                 const int32_t row = M::row(lane, r);
-                const int32_t l = 16 * t + i;
+                const int32_t l = l_base + 16 * t + i;
                 const bool ok = row < n && l < L;
                 const size_t at = static_cast<size_t>(first_edge + row) * L + l;
                 if constexpr (WEIGHTED) {
@@ -781,6 +801,28 @@ __global__ __launch_bounds__(WAVE) void edge_rows_vjp_kernel(
                     }
                 } else if (ok) {
                     grad_B[at] = acc_B[t][r];
+                }
+            }
+        }
+    }
+    if (!BLOCKS) {
+        break;
+    }
+    next_base += 16 * NT;
+    if (next_base >= L) {
+        break;
+    }
+    load_b_left(next_base);
+    }
+    if (want_A) {
+#pragma unroll
+        for (int t = 0; t < KT; t++) {
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                const int32_t row = M::row(lane, r);
+                const int32_t k = 16 * t + i;
+                if (row < n && k < K) {
+                    grad_A[static_cast<size_t>(first_edge + row) * K + k] = acc_A[t][r];
                 }
             }
         }
@@ -1048,49 +1090,60 @@ void launch_vjp(
             return shift;
         };
         const unsigned waves = static_cast<unsigned>(ceil_div(static_cast<size_t>(n_edges), CHUNK));
-        if (lds > 64 * 1024) {
+        if (lds > 64 * 1024 && K > 32) {
             const unsigned blocks = static_cast<unsigned>(ceil_div(static_cast<size_t>(n_edges), WIDE_WAVES));
             vjp_wide_kernel<T, WEIGHTED><<<blocks, WIDE_WAVES * WAVE, 0, stream>>>(
                 grad_A.data, grad_B.data, edge_W, grad_output.data, A.data, B.data, W, indices_W,
                 indices_output.data, n_edges, n_output, K, L
             );
-        } else if (K <= 32 && L <= 64) {
+        } else if (K <= 32) {
             const unsigned groups = static_cast<unsigned>(ceil_div(static_cast<size_t>(n_edges), 16));
             MainKernelTimer timer(stream);
             const bool vectors = L % (16 / static_cast<int32_t>(sizeof(T))) == 0 &&
                                  reinterpret_cast<uintptr_t>(B.data) % 16 == 0 &&
                                  reinterpret_cast<uintptr_t>(grad_output.data) % 16 == 0 &&
                                  (!WEIGHTED || reinterpret_cast<uintptr_t>(W) % 16 == 0);
+#define MOPS_LAUNCH_ROWS_AS(KT, NT, VECTORS, BLOCKS)                                                \
+    edge_rows_vjp_kernel<T, KT, NT, WEIGHTED, VECTORS, BLOCKS><<<groups, WAVE, 0, stream>>>(       \
+        grad_A.data, grad_B.data, edge_W, grad_output.data, A.data, B.data, W, indices_W,          \
+        indices_output.data, n_edges, n_output, K, L                                               \
+    )
 #define MOPS_LAUNCH_ROWS(KT, NT)                                                                   \
     if (vectors) {                                                                                 \
-        edge_rows_vjp_kernel<T, KT, NT, WEIGHTED, true><<<groups, WAVE, 0, stream>>>(              \
-            grad_A.data, grad_B.data, edge_W, grad_output.data, A.data, B.data, W, indices_W,      \
-            indices_output.data, n_edges, n_output, K, L                                           \
-        );                                                                                         \
+        MOPS_LAUNCH_ROWS_AS(KT, NT, true, false);                                                  \
     } else {                                                                                       \
-        edge_rows_vjp_kernel<T, KT, NT, WEIGHTED, false><<<groups, WAVE, 0, stream>>>(             \
-            grad_A.data, grad_B.data, edge_W, grad_output.data, A.data, B.data, W, indices_W,      \
-            indices_output.data, n_edges, n_output, K, L                                           \
-        );                                                                                         \
+        MOPS_LAUNCH_ROWS_AS(KT, NT, false, false);                                                 \
+    }
+#define MOPS_LAUNCH_ROW_PASSES(KT)                                                                 \
+    if (vectors) {                                                                                 \
+        MOPS_LAUNCH_ROWS_AS(KT, 4, true, true);                                                    \
+    } else {                                                                                       \
+        MOPS_LAUNCH_ROWS_AS(KT, 4, false, true);                                                   \
     }
             if (K <= 16) {
                 if (L <= 16) {
                     MOPS_LAUNCH_ROWS(1, 1);
                 } else if (L <= 32) {
                     MOPS_LAUNCH_ROWS(1, 2);
-                } else {
+                } else if (L <= 64) {
                     MOPS_LAUNCH_ROWS(1, 4);
+                } else {
+                    MOPS_LAUNCH_ROW_PASSES(1);
                 }
             } else {
                 if (L <= 16) {
                     MOPS_LAUNCH_ROWS(2, 1);
                 } else if (L <= 32) {
                     MOPS_LAUNCH_ROWS(2, 2);
-                } else {
+                } else if (L <= 64) {
                     MOPS_LAUNCH_ROWS(2, 4);
+                } else {
+                    MOPS_LAUNCH_ROW_PASSES(2);
                 }
             }
+#undef MOPS_LAUNCH_ROW_PASSES
 #undef MOPS_LAUNCH_ROWS
+#undef MOPS_LAUNCH_ROWS_AS
         } else {
             MainKernelTimer timer(stream);
             vjp_kernel<T, WEIGHTED><<<waves, WAVE, lds, stream>>>(

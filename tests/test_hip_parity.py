@@ -45,6 +45,8 @@ CASES = {
         "long_segments": lambda s, d: support.opsa_case(s, d, J=3000, K=5, L=7, n_out=6),
         "wide": lambda s, d: support.opsa_case(s, d, J=400, K=40, L=33, n_out=21, allow_empty=True),
         "mostly_empty": lambda s, d: support.opsa_case(s, d, J=20, K=4, L=4, n_out=300, allow_empty=True),
+        "many_columns": lambda s, d: support.opsa_case(s, d, J=700, K=16, L=128, n_out=31, allow_empty=True),
+        "ragged_columns": lambda s, d: support.opsa_case(s, d, J=500, K=20, L=70, n_out=23, allow_empty=True),
     },
     "opsaw": {
         "tiny": lambda s, d: support.opsaw_case(s, d, E=6, K=2, L=3, n_nodes=4, allow_empty=True),
@@ -52,6 +54,8 @@ CASES = {
         "long_segments": lambda s, d: support.opsaw_case(s, d, E=3000, K=5, L=7, n_nodes=6),
         "hub_sender": lambda s, d: _hub(support.opsaw_case(s, d, E=2600, K=3, L=5, n_nodes=9), "indices_W"),
         "mostly_empty": lambda s, d: support.opsaw_case(s, d, E=20, K=4, L=4, n_nodes=300, allow_empty=True),
+        "many_columns": lambda s, d: support.opsaw_case(s, d, E=700, K=32, L=192, n_nodes=31, allow_empty=True),
+        "ragged_columns": lambda s, d: support.opsaw_case(s, d, E=500, K=9, L=131, n_nodes=23, allow_empty=True),
     },
     "sasaw": {
         "tiny": lambda s, d: support.sasaw_case(s, d, E=6, nA=2, L=3, n_nodes=4, n2=2, n3=2, N=5, allow_empty=True),
