@@ -36,6 +36,11 @@
 //    segments they belong to;
 //  - grad_W: one wavefront per sender, senders found by sender_gather.hpp.
 // Sums never depend on the launch or on timing: no atomics anywhere.
+//
+// More than 64 feature channels are taken 64 at a time, one launch per block
+// of columns (rows keep their distance in memory, `ld`): outputs, grad_B and
+// grad_W are per column, and grad_A, a sum over the columns, is added to by
+// the launches one after the other on the stream.
 #include "sasaw_mfma.hpp"
 
 #include <algorithm>
@@ -254,12 +259,13 @@ __device__ __forceinline__ void coupling_times_A(
 //  grad_W:  o = m2, c = m3, rows = grad_output, source = receiver).
 template <typename T> struct Contraction {
     const T* A;    // [n_edges][nA]
-    const T* B;    // [n_edges][L]
-    const T* rows; // [n_blocks][n_red][L]
+    const T* B;    // [n_edges][ld], L columns of it
+    const T* rows; // [n_blocks][n_red][ld], L columns of it
     const int32_t* gather_index; // block of `rows` of every edge
     const T* to_cells;
     DenseLayout layout;
     int32_t n_blocks, nA, L, n_out, n_red;
+    int32_t ld; // distance between rows of B, of `rows` and of the result (>= L: L may be a block of columns)
     int32_t out_cell_stride, red_cell_stride; // cell = o * out_cell_stride + c * red_cell_stride
     bool vector_rows; // NT neighbouring elements of `rows` and of B may be loaded at once
 };
@@ -283,7 +289,7 @@ template <typename T, int NT, int RS> struct ContractionLane {
             a_offset[s] = cell * T_ROW * sizeof(T);
 #pragma unroll
             for (int t = 0; t < NT; t++) {
-                w_offset[s][t] = ((red_ok ? c : 0) * p.L + column(p, i, t)) * sizeof(T);
+                w_offset[s][t] = ((red_ok ? c : 0) * p.ld + column(p, i, t)) * sizeof(T);
             }
         }
 #pragma unroll
@@ -337,7 +343,7 @@ __device__ __forceinline__ void contract_batch(
     // costs about as much as the arithmetic of all 16 edges, so as many as
     // the registers hold (RS * NT + NT values per edge).
     constexpr int EB = 4 / (NT >= 4 ? 2 : 1);
-    const uint32_t block_elements = static_cast<uint32_t>(p.n_red) * p.L;
+    const uint32_t block_elements = static_cast<uint32_t>(p.n_red) * p.ld;
     // Nothing below is conditional: lanes 0..15 without an edge (or with a
     // source out of range) get a zero column of T, and their operand loads are
     // redirected to an edge that exists, so their products vanish.
@@ -356,7 +362,7 @@ __device__ __forceinline__ void contract_batch(
         const int32_t edge = __builtin_amdgcn_readlane(load_edge, k);
         const int32_t source = __builtin_amdgcn_readlane(load_source, k);
         const T* block = p.rows + static_cast<size_t>(source) * block_elements;
-        const T* b_row = p.B + static_cast<size_t>(edge) * p.L;
+        const T* b_row = p.B + static_cast<size_t>(edge) * p.ld;
         if constexpr (decltype(vectors)::value) {
 #pragma unroll
             for (int s = 0; s < RS; s++) {
@@ -427,10 +433,10 @@ __device__ __forceinline__ void contract_batch(
     }
 }
 
-/// Writes tile element (row, column i of tile t) to target[row * L + NT * i + t].
+/// Writes tile element (row, column i of tile t) to target[row * ld + NT * i + t].
 template <typename T, int NT, typename Value>
 __device__ __forceinline__ void store_block(
-    T* __restrict__ target, Value&& value, int32_t n_out, int32_t L, int lane
+    T* __restrict__ target, Value&& value, int32_t n_out, int32_t L, int32_t ld, int lane
 ) {
     using M = Mfma<T>;
     const int i = lane & 15;
@@ -441,7 +447,7 @@ __device__ __forceinline__ void store_block(
         for (int t = 0; t < NT; t++) {
             const int32_t col = NT * i + t;
             if (row < n_out && col < L) {
-                target[row * L + col] = value(t, r);
+                target[row * ld + col] = value(t, r);
             }
         }
     }
@@ -484,7 +490,7 @@ __global__ __launch_bounds__(forward_waves<T>() * WAVE) void forward_kernel(
     T* t_area = reinterpret_cast<T*>(lds_raw) + wave * p.layout.t_elements();
     // partial sums: [segment of the round][rank][NT][4][64]
     T* meeting = reinterpret_cast<T*>(lds_raw) + FORWARD_WAVES * p.layout.t_elements();
-    const size_t row_elements = static_cast<size_t>(p.n_out) * p.L;
+    const size_t row_elements = static_cast<size_t>(p.n_out) * p.ld;
 
     // the senders of this workgroup's positions, asked for before anything
     // is known about the segments
@@ -529,7 +535,7 @@ __global__ __launch_bounds__(forward_waves<T>() * WAVE) void forward_kernel(
                 }
                 store_block<T, NT>(
                     output + waiting_node[segment] * row_elements, [&](int t, int r) { return sum[t][r]; },
-                    p.n_out, p.L, lane
+                    p.n_out, p.L, p.ld, lane
                 );
             }
         }
@@ -562,7 +568,7 @@ __global__ __launch_bounds__(forward_waves<T>() * WAVE) void forward_kernel(
                 if (rank == 0) {
                     store_block<T, NT>(
                         output + node * row_elements, [&](int t, int r) { return acc.total(t, r); }, p.n_out,
-                        p.L, lane
+                        p.L, p.ld, lane
                     );
                 }
             } else {
@@ -592,9 +598,19 @@ __global__ __launch_bounds__(forward_waves<T>() * WAVE) void forward_kernel(
         },
         [&](int32_t begin, int32_t end) {
             T* target = output + begin * row_elements;
-            const size_t count = (end - begin) * row_elements;
-            for (size_t at = threadIdx.x; at < count; at += FORWARD_WAVES * WAVE) {
-                target[at] = T(0);
+            if (p.ld == p.L) {
+                const size_t count = (end - begin) * row_elements;
+                for (size_t at = threadIdx.x; at < count; at += FORWARD_WAVES * WAVE) {
+                    target[at] = T(0);
+                }
+            } else {
+                // a block of columns: row by row
+                const int32_t rows = (end - begin) * p.n_out;
+                for (int32_t row = 0; row < rows; row++) {
+                    for (int32_t col = threadIdx.x; col < p.L; col += FORWARD_WAVES * WAVE) {
+                        target[static_cast<size_t>(row) * p.ld + col] = T(0);
+                    }
+                }
             }
         }
     );
@@ -641,8 +657,8 @@ __global__ __launch_bounds__(senders_per_group<T>() * WAVE) void weight_gradient
     }
     if (node < p.n_blocks) {
         store_block<T, NT>(
-            grad_W + static_cast<size_t>(node) * p.n_out * p.L, [&](int t, int r) { return acc.total(t, r); },
-            p.n_out, p.L, lane
+            grad_W + static_cast<size_t>(node) * p.n_out * p.ld, [&](int t, int r) { return acc.total(t, r); },
+            p.n_out, p.L, p.ld, lane
         );
     }
 }
@@ -653,7 +669,7 @@ __global__ __launch_bounds__(senders_per_group<T>() * WAVE) void weight_gradient
 template <typename T> struct EdgeGradArgs {
     T* grad_A; // may be null
     T* grad_B; // may be null
-    const T* G; // grad_output [n_nodes][n3][L]
+    const T* G; // grad_output [n_nodes][n3][ld]
     const T* A;
     const T* B;
     const T* W;
@@ -663,6 +679,8 @@ template <typename T> struct EdgeGradArgs {
     const T* to_A;
     DenseLayout layout;
     int32_t n_edges, n_nodes, nA, L, n2, n3;
+    int32_t ld;        // distance between rows of B, W, grad_output, grad_B (>= L: L may be a block of columns)
+    bool add_to_A;     // grad_A += (a later block of columns) instead of grad_A =
     int32_t Ls;        // LDS stride of one row of W and of B
     bool vector_loads; // W may be read 128 bits at a time
     FastDivisor by_items, by_lvec, by_L; // n2 * L / vec, L / vec, L
@@ -744,7 +762,7 @@ __global__ __launch_bounds__(WAVE) void edge_gradients_kernel(const EdgeGradArgs
     };
     const uint32_t items_per_edge = p.by_items.divisor;
     const uint32_t lvecs = p.by_lvec.divisor;
-    const int32_t block_elements = p.n2 * p.L;
+    const int32_t block_elements = p.n2 * p.ld;
     auto ask_for_rows = [&](RowsOnTheWay& to, int32_t k0, int32_t n_batch, uint32_t base) {
         const uint32_t total = static_cast<uint32_t>(n_batch) * items_per_edge;
 #pragma unroll
@@ -758,7 +776,7 @@ __global__ __launch_bounds__(WAVE) void edge_gradients_kernel(const EdgeGradArgs
             const uint32_t lv = rest - row * lvecs;
             const int32_t source = __shfl(my_source, k0 + static_cast<int>(kw));
             const bool valid = to.ok[u] && in_bounds(source, p.n_nodes);
-            const size_t from = valid ? static_cast<size_t>(source) * block_elements + rest * 4 : 0;
+            const size_t from = valid ? static_cast<size_t>(source) * block_elements + row * p.ld + lv * 4 : 0;
             const Vec value = *reinterpret_cast<const Vec*>(p.W + from);
             to.loaded[u] = valid ? value : Vec(T(0));
             to.where[u] = (kw * p.n2 + row) * p.Ls + lv * 4;
@@ -835,18 +853,18 @@ __global__ __launch_bounds__(WAVE) void edge_gradients_kernel(const EdgeGradArgs
                 const int32_t source = __shfl(my_source, k0 + static_cast<int>(kw));
                 const bool valid = ok && in_bounds(source, p.n_nodes);
                 const T value =
-                    load_or_zero(p.W, static_cast<size_t>(source) * block_elements + rest, valid);
+                    load_or_zero(p.W, static_cast<size_t>(source) * block_elements + row * p.ld + l, valid);
                 if (ok) {
                     w_lds[(kw * p.n2 + row) * p.Ls + l] = value;
                 }
             }
         }
         {
-            const T* from = p.B + static_cast<size_t>(chunk_begin + k0) * p.L;
+            const T* from = p.B + static_cast<size_t>(chunk_begin + k0) * p.ld;
             const uint32_t count = static_cast<uint32_t>(n_batch) * p.L;
             for (uint32_t at = lane; at < count; at += WAVE) {
                 const uint32_t kw = p.by_L.divide(at);
-                b_lds[kw * p.Ls + (at - kw * p.L)] = from[at];
+                b_lds[kw * p.Ls + (at - kw * p.L)] = from[kw * p.ld + (at - kw * p.L)];
             }
         }
         __syncthreads();
@@ -861,20 +879,20 @@ __global__ __launch_bounds__(WAVE) void edge_gradients_kernel(const EdgeGradArgs
             if (node != current_node) {
                 current_node = node;
                 const bool valid = in_bounds(node, p.n_nodes);
-                const T* g_block = p.G + static_cast<size_t>(valid ? node : 0) * p.n3 * p.L;
+                const T* g_block = p.G + static_cast<size_t>(valid ? node : 0) * p.n3 * p.ld;
 #pragma unroll
                 for (int t = 0; t < NT; t++) {
 #pragma unroll
                     for (int r = 0; r < 4; r++) {
                         const int32_t m3 = M::row(lane, r);
                         const int32_t col = 16 * t + i;
-                        g_rows[t][r] = load_or_zero(g_block, m3 * p.L + col, valid && m3 < p.n3 && col < p.L);
+                        g_rows[t][r] = load_or_zero(g_block, m3 * p.ld + col, valid && m3 < p.n3 && col < p.L);
                     }
                 }
 #pragma unroll
                 for (int s = 0; s < L_STEPS; s++) {
                     const int32_t l = 4 * s + q;
-                    g_left[s] = load_or_zero(g_block, i * p.L + l, valid && i < p.n3 && l < p.L);
+                    g_left[s] = load_or_zero(g_block, i * p.ld + l, valid && i < p.n3 && l < p.L);
                 }
             }
             const uint32_t column = first_column + kw * ELEMENT;
@@ -936,7 +954,7 @@ __global__ __launch_bounds__(WAVE) void edge_gradients_kernel(const EdgeGradArgs
                 }
                 const int32_t col = 16 * t + i;
                 if (q < n_batch && col < p.L) {
-                    p.grad_B[static_cast<size_t>(chunk_begin + k0 + q) * p.L + col] = sum;
+                    p.grad_B[static_cast<size_t>(chunk_begin + k0 + q) * p.ld + col] = sum;
                 }
             }
         }
@@ -967,7 +985,9 @@ __global__ __launch_bounds__(WAVE) void edge_gradients_kernel(const EdgeGradArgs
         for (int r = 0; r < 4; r++) {
             const int32_t k = M::row(lane, r);
             if (k < n && i < p.nA) {
-                p.grad_A[static_cast<size_t>(chunk_begin + k) * p.nA + i] = even[r] + odd[r];
+                T* target = p.grad_A + static_cast<size_t>(chunk_begin + k) * p.nA + i;
+                const T before = p.add_to_A ? *target : T(0);
+                *target = before + (even[r] + odd[r]);
             }
         }
     }
@@ -1044,8 +1064,8 @@ bool aligned_for_vectors(const void* pointer, size_t element_size) {
 template <typename T>
 Contraction<T> contraction(
     const T* A, const T* B, const T* rows, const int32_t* gather_index, const T* to_cells,
-    const DenseLayout& layout, const Shape& s, int32_t n_out, int32_t n_red, int32_t out_cell_stride,
-    int32_t red_cell_stride
+    const DenseLayout& layout, const Shape& s, int32_t ld, int32_t n_out, int32_t n_red,
+    int32_t out_cell_stride, int32_t red_cell_stride
 ) {
     Contraction<T> c{};
     c.A = A;
@@ -1057,12 +1077,14 @@ Contraction<T> contraction(
     c.n_blocks = s.n_nodes;
     c.nA = s.nA;
     c.L = s.L;
+    c.ld = ld;
     c.n_out = n_out;
     c.n_red = n_red;
     c.out_cell_stride = out_cell_stride;
     c.red_cell_stride = red_cell_stride;
     const size_t vector_bytes = tiles_for(s.L) * sizeof(T);
-    c.vector_rows = s.L % tiles_for(s.L) == 0 && reinterpret_cast<uintptr_t>(rows) % vector_bytes == 0 &&
+    c.vector_rows = s.L % tiles_for(s.L) == 0 && ld % tiles_for(s.L) == 0 &&
+                    reinterpret_cast<uintptr_t>(rows) % vector_bytes == 0 &&
                     reinterpret_cast<uintptr_t>(B) % vector_bytes == 0;
     return c;
 }
@@ -1093,14 +1115,31 @@ template <typename Launch> void with_shape_constants(int tiles, int steps, Launc
     }
 }
 
+/// Feature channels beyond MAX_L are taken MAX_L at a time: `pass(first_column, shape)`
+/// is called with the shape narrowed to one such block of columns.
+template <typename Pass> void for_each_column_block(const Shape& s, Pass&& pass) {
+    for (int32_t first = 0; first < s.L; first += MAX_L) {
+        Shape block = s;
+        block.L = std::min<int32_t>(MAX_L, s.L - first);
+        pass(first, block);
+    }
+}
+
+Shape widest_block(const Shape& s) {
+    Shape block = s;
+    block.L = std::min<int32_t>(MAX_L, s.L);
+    return block;
+}
+
 } // namespace
 
-bool supports(const Shape& s, size_t element_size) {
+bool supports(const Shape& full, size_t element_size) {
+    const Shape s = widest_block(full);
     if (s.n_nodes < 1 || s.n_edges < 1 || s.N < 1) {
         return false;
     }
     if (s.nA < 1 || s.nA > 4 * MAX_A_STEPS || s.n2 < 1 || s.n2 > MAX_INDEX || s.n3 < 1 ||
-        s.n3 > MAX_INDEX || s.L < 1 || s.L > MAX_L) {
+        s.n3 > MAX_INDEX || s.L < 1) {
         return false;
     }
     return forward_lds(s, element_size) <= LDS_BUDGET && weight_gradient_lds(s, element_size) <= WEIGHT_LDS_BUDGET &&
@@ -1118,24 +1157,28 @@ void forward(
 ) {
     const DenseLayout layout = dense_layout(s);
     const DenseBuffers<T> dense = enqueue_dense<T>(workspace, layout, C, indices, s, stream);
-    const Contraction<T> c =
-        contraction<T>(A, B, W, indices.W_1, dense.to_cells, layout, s, s.n3, s.n2, s.n2, 1);
     // positions of the sorted index per workgroup: one stage per wavefront while all
     // workgroups still fit on the device together, else two
     const bool short_chunks = (s.n_edges + SHORT_CHUNK - 1) / SHORT_CHUNK <= FORWARD_RESIDENT_GROUPS;
     const int32_t chunk = short_chunks ? SHORT_CHUNK : LONG_CHUNK;
     const int32_t grid = (s.n_edges + chunk - 1) / chunk;
-    const size_t lds = forward_lds(s, sizeof(T));
-    with_shape_constants(tiles_for(s.L), (s.n2 + 3) / 4, [&](auto tiles, auto steps) {
-        if (short_chunks) {
-            forward_kernel<T, decltype(tiles)::value, decltype(steps)::value, SHORT_CHUNK>
-                <<<grid, forward_waves<T>() * WAVE, lds, stream>>>(output, indices.output_1, s.n_edges, c);
-        } else {
-            forward_kernel<T, decltype(tiles)::value, decltype(steps)::value, LONG_CHUNK>
-                <<<grid, forward_waves<T>() * WAVE, lds, stream>>>(output, indices.output_1, s.n_edges, c);
-        }
+    for_each_column_block(s, [&](int32_t first, const Shape& block) {
+        const Contraction<T> c = contraction<T>(
+            A, B + first, W + first, indices.W_1, dense.to_cells, layout, block, s.L, s.n3, s.n2, s.n2, 1
+        );
+        const size_t lds = forward_lds(block, sizeof(T));
+        T* target = output + first;
+        with_shape_constants(tiles_for(block.L), (s.n2 + 3) / 4, [&](auto tiles, auto steps) {
+            if (short_chunks) {
+                forward_kernel<T, decltype(tiles)::value, decltype(steps)::value, SHORT_CHUNK>
+                    <<<grid, forward_waves<T>() * WAVE, lds, stream>>>(target, indices.output_1, s.n_edges, c);
+            } else {
+                forward_kernel<T, decltype(tiles)::value, decltype(steps)::value, LONG_CHUNK>
+                    <<<grid, forward_waves<T>() * WAVE, lds, stream>>>(target, indices.output_1, s.n_edges, c);
+            }
+        });
+        MOPS_HIP_CHECK(hipGetLastError());
     });
-    MOPS_HIP_CHECK(hipGetLastError());
 }
 
 template <typename T>
@@ -1145,18 +1188,18 @@ void vjp(
 ) {
     const DenseLayout layout = dense_layout(s);
     const DenseBuffers<T> dense = enqueue_dense<T>(workspace, layout, C, indices, s, stream);
-    const int tiles = tiles_for(s.L);
     const bool want_edges = grad_A != nullptr || grad_B != nullptr;
 
-    auto launch_weights = [&](hipStream_t on) {
+    auto launch_weights = [&](hipStream_t on, int32_t first, const Shape& block) {
         const Contraction<T> c = contraction<T>(
-            A, B, grad_output, indices.output_1, dense.to_cells, layout, s, s.n2, s.n3, 1, s.n2
+            A, B + first, grad_output + first, indices.output_1, dense.to_cells, layout, block, s.L, s.n2,
+            s.n3, 1, s.n2
         );
         constexpr int SENDERS_PER_GROUP = senders_per_group<T>();
         const int32_t grid = (s.n_nodes + SENDERS_PER_GROUP - 1) / SENDERS_PER_GROUP;
-        const size_t lds = weight_gradient_lds(s, sizeof(T));
+        const size_t lds = weight_gradient_lds(block, sizeof(T));
         const bool aligned = aligned_for_vectors(indices.W_1, sizeof(int32_t));
-        with_shape_constants(tiles, (s.n3 + 3) / 4, [&](auto tiles_constant, auto steps) {
+        with_shape_constants(tiles_for(block.L), (s.n3 + 3) / 4, [&](auto tiles_constant, auto steps) {
             auto kernel = weight_gradient_kernel<T, decltype(tiles_constant)::value, decltype(steps)::value>;
             if (lds > 64 * 1024) {
                 MOPS_HIP_CHECK(hipFuncSetAttribute(
@@ -1164,21 +1207,24 @@ void vjp(
                     static_cast<int>(lds)
                 ));
             }
-            kernel<<<grid, SENDERS_PER_GROUP * WAVE, lds, on>>>(grad_W, indices.W_1, s.n_edges, aligned, c);
+            kernel<<<grid, SENDERS_PER_GROUP * WAVE, lds, on>>>(
+                grad_W + first, indices.W_1, s.n_edges, aligned, c
+            );
         });
         MOPS_HIP_CHECK(hipGetLastError());
     };
 
-    auto launch_edges = [&]() {
-        const bool vectors = s.L % 4 == 0 && aligned_for_vectors(W, sizeof(T));
+    auto launch_edges = [&](int32_t first, const Shape& block) {
+        const bool vectors = block.L % 4 == 0 && s.L % 4 == 0 && aligned_for_vectors(W + first, sizeof(T));
         const int vec = vectors ? 4 : 1;
         EdgeGradArgs<T> args{};
         args.grad_A = grad_A;
-        args.grad_B = grad_B;
-        args.G = grad_output;
+        args.add_to_A = first > 0; // the sums over the columns of the blocks follow each other on the stream
+        args.grad_B = grad_B != nullptr ? grad_B + first : nullptr;
+        args.G = grad_output + first;
         args.A = A;
-        args.B = B;
-        args.W = W;
+        args.B = B + first;
+        args.W = W + first;
         args.receivers = indices.output_1;
         args.senders = indices.W_1;
         args.to_cells = dense.to_cells;
@@ -1187,17 +1233,18 @@ void vjp(
         args.n_edges = s.n_edges;
         args.n_nodes = s.n_nodes;
         args.nA = s.nA;
-        args.L = s.L;
+        args.L = block.L;
+        args.ld = s.L;
         args.n2 = s.n2;
         args.n3 = s.n3;
-        args.Ls = weight_row_stride(s);
+        args.Ls = weight_row_stride(block);
         args.vector_loads = vectors;
-        args.by_items = FastDivisor::make(s.n2 * s.L / vec);
-        args.by_lvec = FastDivisor::make(s.L / vec);
-        args.by_L = FastDivisor::make(s.L);
+        args.by_items = FastDivisor::make(s.n2 * block.L / vec);
+        args.by_lvec = FastDivisor::make(block.L / vec);
+        args.by_L = FastDivisor::make(block.L);
         const int32_t grid = (s.n_edges + STAGE - 1) / STAGE;
-        const size_t lds = edge_gradients_lds(s, sizeof(T));
-        with_shape_constants(tiles, (s.n2 + 3) / 4, [&](auto tiles_constant, auto steps) {
+        const size_t lds = edge_gradients_lds(block, sizeof(T));
+        with_shape_constants(tiles_for(block.L), (s.n2 + 3) / 4, [&](auto tiles_constant, auto steps) {
             edge_gradients_kernel<T, decltype(tiles_constant)::value, decltype(steps)::value>
                 <<<grid, WAVE, lds, stream>>>(args);
         });
@@ -1210,12 +1257,14 @@ void vjp(
         // that forks from `stream` after the dense table and joins it again.
         // (weights first: the other order is slower, 109 instead of 97 us in f32)
         SideStream side(stream);
-        launch_weights(side.get());
-        launch_edges();
+        for_each_column_block(s, [&](int32_t first, const Shape& block) {
+            launch_weights(side.get(), first, block);
+            launch_edges(first, block);
+        });
     } else if (want_edges) {
-        launch_edges();
+        for_each_column_block(s, launch_edges);
     } else if (grad_W != nullptr) {
-        launch_weights(stream);
+        for_each_column_block(s, [&](int32_t first, const Shape& block) { launch_weights(stream, first, block); });
     }
 }
 

@@ -1,7 +1,7 @@
 // Matrix-core path of SASAW for the table shapes of equivariant message
-// passing (at most 16 values of every component index, at most 64 feature
-// channels). sasaw.hip calls it when `supports()` says so and keeps its
-// general kernels for everything else.
+// passing (at most 16 values of every component index; any number of feature
+// channels, taken 64 at a time). sasaw.hip calls it when `supports()` says so
+// and keeps its general kernels for everything else.
 #ifndef MOPS_AMD_SASAW_MFMA_HPP
 #define MOPS_AMD_SASAW_MFMA_HPP
 
