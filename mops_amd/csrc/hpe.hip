@@ -181,9 +181,12 @@ __global__ __launch_bounds__(256) void forward_ordered_kernel(
 }
 
 // ---------------------------------------------------------------------------
-// vjp. One wavefront per workgroup. LDS: a[nA][R] accumulator[G][nA][R]
+// vjp. One wavefront per workgroup. LDS: a[nA][R] accumulator[G][span][R]
 // Thread (r, g) adds its monomials' terms into its private accumulator row
 // set; afterwards the G copies are added in group order.
+// `span` = nA when the accumulators of all features fit in LDS; otherwise the
+// features are split into ranges of `span`, blockIdx.y picks the range, and a
+// workgroup walks all monomials but keeps only the terms for its range.
 // ---------------------------------------------------------------------------
 template <typename T>
 __global__ __launch_bounds__(WAVE) void vjp_kernel(
@@ -196,11 +199,14 @@ __global__ __launch_bounds__(WAVE) void vjp_kernel(
     int32_t nA,
     int32_t n_monomials,
     int32_t order,
-    int32_t R
+    int32_t R,
+    int32_t span
 ) {
     extern __shared__ __align__(16) unsigned char lds_bytes[];
     T* a_stage = reinterpret_cast<T*>(lds_bytes);
     T* accumulator = a_stage + static_cast<size_t>(nA) * R;
+    const int32_t feature_begin = blockIdx.y * span;
+    const int32_t feature_count = min(span, nA - feature_begin);
 
     const int tid = threadIdx.x;
     const int G = WAVE / R;
@@ -214,20 +220,20 @@ __global__ __launch_bounds__(WAVE) void vjp_kernel(
         int32_t row = i / nA;
         a_stage[(i - row * nA) * R + row] = a_src[i];
     }
-    for (int32_t i = tid; i < G * nA * R; i += WAVE) {
+    for (int32_t i = tid; i < G * feature_count * R; i += WAVE) {
         accumulator[i] = T(0);
     }
     __syncthreads();
 
     if (r < rows) {
-        T* mine = accumulator + static_cast<size_t>(g) * nA * R + r;
+        T* mine = accumulator + static_cast<size_t>(g) * feature_count * R + r;
         const T upstream = grad_output[row0 + r];
         for (int32_t j = g; j < n_monomials; j += G) {
             const int32_t* factors = P + static_cast<size_t>(j) * order;
             const T base = C[j] * upstream;
             for (int32_t f = 0; f < order; f++) {
-                int32_t target = factors[f];
-                if (!in_bounds(target, nA)) {
+                int32_t target = factors[f] - feature_begin;
+                if (!in_bounds(target, feature_count)) {
                     continue;
                 }
                 T term = base;
@@ -244,15 +250,15 @@ __global__ __launch_bounds__(WAVE) void vjp_kernel(
     }
     __syncthreads();
 
-    T* dst = grad_A + static_cast<size_t>(row0) * nA;
-    for (int32_t i = tid; i < rows * nA; i += WAVE) {
-        int32_t row = i / nA;
-        int32_t feature = i - row * nA;
+    T* dst = grad_A + static_cast<size_t>(row0) * nA + feature_begin;
+    for (int32_t i = tid; i < rows * feature_count; i += WAVE) {
+        int32_t row = i / feature_count;
+        int32_t feature = i - row * feature_count;
         T total = T(0);
         for (int group = 0; group < G; group++) {
-            total += accumulator[(static_cast<size_t>(group) * nA + feature) * R + row];
+            total += accumulator[(static_cast<size_t>(group) * feature_count + feature) * R + row];
         }
-        dst[i] = total;
+        dst[static_cast<size_t>(row) * nA + feature] = total;
     }
 }
 
@@ -272,11 +278,14 @@ __global__ __launch_bounds__(WAVE) void vjp_ordered_kernel(
     int32_t n_rows,
     int32_t nA,
     int32_t n_monomials,
-    int32_t R
+    int32_t R,
+    int32_t span
 ) {
     extern __shared__ __align__(16) unsigned char lds_bytes[];
     T* a_stage = reinterpret_cast<T*>(lds_bytes);
     T* accumulator = a_stage + static_cast<size_t>(nA) * R;
+    const int32_t feature_begin = blockIdx.y * span;
+    const int32_t feature_count = min(span, nA - feature_begin);
 
     const int tid = threadIdx.x;
     const int G = WAVE / R;
@@ -290,13 +299,13 @@ __global__ __launch_bounds__(WAVE) void vjp_ordered_kernel(
         int32_t row = i / nA;
         a_stage[(i - row * nA) * R + row] = a_src[i];
     }
-    for (int32_t i = tid; i < G * nA * R; i += WAVE) {
+    for (int32_t i = tid; i < G * feature_count * R; i += WAVE) {
         accumulator[i] = T(0);
     }
     __syncthreads();
 
     if (r < rows) {
-        T* mine = accumulator + static_cast<size_t>(g) * nA * R + r;
+        T* mine = accumulator + static_cast<size_t>(g) * feature_count * R + r;
         const T upstream = grad_output[row0 + r];
         struct Monomial {
             int32_t factor[ORDER];
@@ -335,23 +344,24 @@ __global__ __launch_bounds__(WAVE) void vjp_ordered_kernel(
             for (int f = ORDER - 1; f >= 0; f--) {
                 const T term = prefix[f] * suffix;
                 suffix *= value[f];
-                if (valid[f]) {
-                    unsafeAtomicAdd(&mine[now.factor[f] * R], term); // a slot of my own: an add without the round trip of read, add, write
+                const int32_t slot = now.factor[f] - feature_begin;
+                if (in_bounds(slot, feature_count)) {
+                    unsafeAtomicAdd(&mine[slot * R], term); // a slot of my own: an add without the round trip of read, add, write
                 }
             }
         }
     }
     __syncthreads();
 
-    T* dst = grad_A + static_cast<size_t>(row0) * nA;
-    for (int32_t i = tid; i < rows * nA; i += WAVE) {
-        int32_t row = i / nA;
-        int32_t feature = i - row * nA;
+    T* dst = grad_A + static_cast<size_t>(row0) * nA + feature_begin;
+    for (int32_t i = tid; i < rows * feature_count; i += WAVE) {
+        int32_t row = i / feature_count;
+        int32_t feature = i - row * feature_count;
         T total = T(0);
         for (int group = 0; group < G; group++) {
-            total += accumulator[(static_cast<size_t>(group) * nA + feature) * R + row];
+            total += accumulator[(static_cast<size_t>(group) * feature_count + feature) * R + row];
         }
-        dst[i] = total;
+        dst[static_cast<size_t>(row) * nA + feature] = total;
     }
 }
 
@@ -746,12 +756,26 @@ void homogeneous_polynomial_evaluation_vjp(MOPS_HPE_VJP_PARAMS(MOPS_CXX_FIRST, M
             R <<= 1;
         }
     }
+    int32_t span = nA; // features whose accumulators one workgroup keeps
+    if (R == 0 && static_cast<size_t>(nA) * sizeof(scalar_t) <= LDS_BUDGET / 2) {
+        // the accumulators of all features do not fit: one row per workgroup,
+        // the features in ranges that do
+        R = 1;
+        span = static_cast<int32_t>(
+            (LDS_BUDGET - static_cast<size_t>(nA) * sizeof(scalar_t)) / (WAVE * sizeof(scalar_t))
+        );
+    }
     if (R > 0) {
-        size_t lds = accumulator_bytes + static_cast<size_t>(nA) * R * sizeof(scalar_t);
-        unsigned blocks = static_cast<unsigned>(ceil_div(static_cast<size_t>(n_rows), R));
+        size_t lds =
+            static_cast<size_t>(span) * WAVE * sizeof(scalar_t) + static_cast<size_t>(nA) * R * sizeof(scalar_t);
+        const dim3 blocks(
+            static_cast<unsigned>(ceil_div(static_cast<size_t>(n_rows), R)),
+            static_cast<unsigned>(ceil_div(static_cast<size_t>(nA), span))
+        );
 #define MOPS_LAUNCH_ORDERED(ORDER)                                                                  \
     vjp_ordered_kernel<scalar_t, ORDER><<<blocks, WAVE, lds, stream>>>(                            \
-        grad_A.data, grad_output.data, A.data, C.data, indices_A.data, n_rows, nA, n_monomials, R  \
+        grad_A.data, grad_output.data, A.data, C.data, indices_A.data, n_rows, nA, n_monomials, R, \
+        span                                                                                       \
     )
         switch (n_monomials > 0 ? order : 0) {
         case 1:
@@ -775,7 +799,7 @@ void homogeneous_polynomial_evaluation_vjp(MOPS_HPE_VJP_PARAMS(MOPS_CXX_FIRST, M
         default:
             vjp_kernel<scalar_t><<<blocks, WAVE, lds, stream>>>(
                 grad_A.data, grad_output.data, A.data, C.data, indices_A.data, n_rows, nA, n_monomials,
-                order, R
+                order, R, span
             );
             break;
         }

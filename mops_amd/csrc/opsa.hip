@@ -835,6 +835,7 @@ __global__ __launch_bounds__(WAVE) void edge_rows_vjp_kernel(
 // flight. Used when a row of W fits one value per lane and register.
 constexpr int GATHER_SENDERS = 8;
 constexpr int GATHER_COLUMNS = 4; // values of a row per lane
+constexpr size_t SENDER_SCAN_LIMIT = 100u * 1000 * 1000; // index reads of the in-kernel gather, all workgroups together
 
 template <typename T>
 __global__ __launch_bounds__(GATHER_SENDERS* WAVE) void sum_by_sender_kernel(
@@ -1051,7 +1052,11 @@ void launch_vjp(
     // scratch: edge_W | sender buckets   (only when grad_W is wanted)
     const size_t edge_w_bytes =
         want_W ? align256(static_cast<size_t>(n_edges) * L * sizeof(T)) : 0;
-    const bool gather_in_kernel = L <= GATHER_COLUMNS * WAVE && n_edges > 0;
+    // Every workgroup of the in-kernel gather reads the whole sender index: fine while
+    // (edges x workgroups) is small, quadratic in the size of the graph beyond
+    const size_t index_reads =
+        static_cast<size_t>(n_edges) * ceil_div(static_cast<size_t>(std::max(n_output, 1)), GATHER_SENDERS);
+    const bool gather_in_kernel = L <= GATHER_COLUMNS * WAVE && n_edges > 0 && index_reads <= SENDER_SCAN_LIMIT;
     const size_t buckets_bytes =
         want_W && !gather_in_kernel ? sender_buckets_bytes(n_output, n_edges) : 0;
     char* workspace =

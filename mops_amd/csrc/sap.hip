@@ -52,7 +52,8 @@ namespace {
 
 constexpr int ROWS = WAVE;            // batch rows per workgroup (one per lane)
 constexpr int ROW_STRIDE = ROWS + 1;  // odd: transposing stores hit distinct banks
-constexpr size_t LDS_BUDGET = 60 * 1024;
+constexpr size_t LDS_BUDGET = 60 * 1024;       // what a workgroup takes by choice
+constexpr size_t LARGE_LDS_BUDGET = 150 * 1024; // what it may take before the kernels without LDS are used (160 KB per compute unit)
 constexpr int GROUP = 8;              // packed entries fetched together
 constexpr int TABLE_PAD = WAVE;       // readable slack after the last packed entry
 
@@ -690,7 +691,7 @@ void sparse_accumulation_of_products(MOPS_SAP_PARAMS(MOPS_CXX_FIRST, MOPS_CXX_NE
     const size_t n_blocks = ceil_div(static_cast<size_t>(n_rows), ROWS);
     const size_t tile_elements = (static_cast<size_t>(nA) + nB + nO) * ROW_STRIDE + ROWS;
     const size_t product_elements = static_cast<size_t>(nA) * nB * ROWS;
-    const bool fits = tile_elements * sizeof(scalar_t) <= LDS_BUDGET && nO <= MAX_BUCKETS;
+    const bool fits = tile_elements * sizeof(scalar_t) <= LARGE_LDS_BUDGET && nO <= MAX_BUCKETS;
     if (!fits) {
         unsigned blocks = static_cast<unsigned>(ceil_div(static_cast<size_t>(n_rows), 256));
         forward_global_kernel<scalar_t><<<blocks, 256, 0, stream>>>(
@@ -715,6 +716,13 @@ void sparse_accumulation_of_products(MOPS_SAP_PARAMS(MOPS_CXX_FIRST, MOPS_CXX_NE
     const int waves = pick_waves(n_blocks, nO);
     const size_t lds = (tile_elements + (use_products ? product_elements : 0)) * sizeof(scalar_t);
     MainKernelTimer timer(stream);
+    if (lds > 64 * 1024) {
+        // (only without the product table: with it the tiles stay below LDS_BUDGET)
+        MOPS_HIP_CHECK(hipFuncSetAttribute(
+            reinterpret_cast<const void*>(forward_kernel<scalar_t, false>),
+            hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)
+        ));
+    }
     if (use_products) {
         forward_kernel<scalar_t, true><<<static_cast<unsigned>(n_blocks), waves * WAVE, lds, stream>>>(
             output.data, A.data, B.data, table, n_rows, FastDivisor::make(nA), FastDivisor::make(nB),
@@ -766,7 +774,7 @@ void sparse_accumulation_of_products_vjp(MOPS_SAP_VJP_PARAMS(MOPS_CXX_FIRST, MOP
     const size_t tile_elements =
         (static_cast<size_t>(nO) + 2 * (static_cast<size_t>(nA) + nB)) * ROW_STRIDE + ROWS;
     const bool fits =
-        tile_elements * sizeof(scalar_t) <= LDS_BUDGET && nA <= MAX_BUCKETS && nB <= MAX_BUCKETS;
+        tile_elements * sizeof(scalar_t) <= LARGE_LDS_BUDGET && nA <= MAX_BUCKETS && nB <= MAX_BUCKETS;
     if (!fits) {
         unsigned blocks = static_cast<unsigned>(ceil_div(static_cast<size_t>(n_rows), 256));
         vjp_global_kernel<scalar_t><<<blocks, 256, 0, stream>>>(
@@ -796,6 +804,12 @@ void sparse_accumulation_of_products_vjp(MOPS_SAP_VJP_PARAMS(MOPS_CXX_FIRST, MOP
     const int waves = pick_waves(n_blocks, (want_A ? nA : 0) + (want_B ? nB : 0));
     const size_t lds = tile_elements * sizeof(scalar_t);
     MainKernelTimer timer(stream);
+    if (lds > 64 * 1024) {
+        MOPS_HIP_CHECK(hipFuncSetAttribute(
+            reinterpret_cast<const void*>(vjp_kernel<scalar_t>), hipFuncAttributeMaxDynamicSharedMemorySize,
+            static_cast<int>(lds)
+        ));
+    }
     vjp_kernel<scalar_t><<<static_cast<unsigned>(n_blocks), waves * WAVE, lds, stream>>>(
         grad_A.data, grad_B.data, grad_output.data, A.data, B.data, by_A, by_B, n_rows,
         FastDivisor::make(nA), FastDivisor::make(nB), FastDivisor::make(nO)

@@ -51,6 +51,7 @@
 #include "mfma.hpp"
 #include "runtime.hpp"
 #include "segment_walk.hpp"
+#include "sender_buckets.hpp"
 #include "sender_gather.hpp"
 
 namespace mops::amd::sasaw_mfma {
@@ -67,6 +68,7 @@ constexpr int TILE_GROUP = 3;    // tiles of 16 cells handled together
 constexpr int STEP_GROUP = 8;    // steps of 4 cells handled together
 constexpr size_t LDS_BUDGET = 64 * 1024;
 constexpr size_t WEIGHT_LDS_BUDGET = 96 * 1024; // the weight-gradient kernel asks for more than 64 KB
+constexpr size_t SENDER_SCAN_LIMIT = 100u * 1000 * 1000; // index reads of the in-kernel gather, all workgroups together
 
 template <typename T>
 __device__ __forceinline__ T load_at(const T* __restrict__ base, uint32_t byte_offset) {
@@ -476,9 +478,13 @@ constexpr int32_t FORWARD_RESIDENT_GROUPS = 256 * 6;
 /// Segments whose partial sums wait in LDS before the wavefronts meet.
 template <typename T> constexpr int round_segments() { return sizeof(T) == 4 ? 2 : 1; }
 
-template <typename T, int NT, int RS, int FORWARD_CHUNK>
+/// PERMUTED: position q of the sorted index stands for edge edge_of_position[q]
+/// (grad_W of a large graph: the index is the sender of every edge, put in
+/// order by sender_buckets.hpp); otherwise for edge q.
+template <typename T, int NT, int RS, int FORWARD_CHUNK, bool PERMUTED>
 __global__ __launch_bounds__(forward_waves<T>() * WAVE) void forward_kernel(
-    T* __restrict__ output, const int32_t* __restrict__ receivers, int32_t n_edges, const Contraction<T> p
+    T* __restrict__ output, const int32_t* __restrict__ receivers,
+    const int32_t* __restrict__ edge_of_position, int32_t n_edges, const Contraction<T> p
 ) {
     constexpr int FORWARD_WAVES = forward_waves<T>();
     constexpr int ROUND_SEGMENTS = round_segments<T>();
@@ -496,8 +502,12 @@ __global__ __launch_bounds__(forward_waves<T>() * WAVE) void forward_kernel(
     // is known about the segments
     const int32_t chunk_begin = blockIdx.x * FORWARD_CHUNK;
     const int32_t chunk_position = chunk_begin + lane;
-    const int32_t chunk_source =
-        lane < FORWARD_CHUNK && chunk_position < n_edges ? p.gather_index[chunk_position] : -1;
+    const bool chunk_valid = lane < FORWARD_CHUNK && chunk_position < n_edges;
+    int32_t chunk_edge = chunk_valid ? chunk_position : -1;
+    if constexpr (PERMUTED) {
+        chunk_edge = chunk_valid ? edge_of_position[chunk_position] : -1;
+    }
+    const int32_t chunk_source = chunk_valid ? p.gather_index[chunk_edge] : -1;
 
     ContractionLane<T, NT, RS> mine;
     mine.setup(p, lane);
@@ -554,10 +564,14 @@ __global__ __launch_bounds__(forward_waves<T>() * WAVE) void forward_kernel(
             for (int32_t st = rank; st < n_stages; st += FORWARD_WAVES) {
                 const int32_t s0 = first + st * STAGE;
                 const int32_t n = min(STAGE, last - s0);
-                const int32_t my_edge = i < n ? s0 + i : -1;
+                int32_t my_edge = i < n ? s0 + i : -1;
                 const int32_t offset = s0 + i - chunk_begin; // >= 0: owned segments start in the chunk
                 const bool at_hand = i < n && offset < FORWARD_CHUNK;
                 int32_t my_source = __shfl(chunk_source, at_hand ? offset : 0);
+                if constexpr (PERMUTED) {
+                    const int32_t listed = __shfl(chunk_edge, at_hand ? offset : 0);
+                    my_edge = at_hand ? listed : (i < n ? edge_of_position[s0 + i] : -1);
+                }
                 if (!at_hand) {
                     my_source = i < n ? p.gather_index[my_edge] : -1;
                 }
@@ -1146,8 +1160,19 @@ bool supports(const Shape& full, size_t element_size) {
            edge_gradients_lds(s, element_size) <= LDS_BUDGET;
 }
 
+/// grad_W: whether the edges are first put in the order of their senders
+/// (sender_buckets.hpp) and walked like the forward pass walks the receivers.
+/// Otherwise every workgroup finds the edges of its senders by reading the
+/// whole sender index (sender_gather.hpp): no preparation, which is what a
+/// small graph wants, but edges x workgroups reads.
+bool orders_edges_by_sender(const Shape& s) {
+    const size_t groups = (static_cast<size_t>(s.n_nodes) + senders_per_group<float>() - 1) / senders_per_group<float>();
+    return static_cast<size_t>(s.n_edges) * groups > SENDER_SCAN_LIMIT;
+}
+
 size_t workspace_bytes(const Shape& s, size_t element_size) {
-    return dense_bytes(dense_layout(s), element_size);
+    return align256(dense_bytes(dense_layout(s), element_size)) +
+           (orders_edges_by_sender(s) ? edges_by_sender_bytes(s.n_nodes, s.n_edges) : 0);
 }
 
 template <typename T>
@@ -1170,11 +1195,15 @@ void forward(
         T* target = output + first;
         with_shape_constants(tiles_for(block.L), (s.n2 + 3) / 4, [&](auto tiles, auto steps) {
             if (short_chunks) {
-                forward_kernel<T, decltype(tiles)::value, decltype(steps)::value, SHORT_CHUNK>
-                    <<<grid, forward_waves<T>() * WAVE, lds, stream>>>(target, indices.output_1, s.n_edges, c);
+                forward_kernel<T, decltype(tiles)::value, decltype(steps)::value, SHORT_CHUNK, false>
+                    <<<grid, forward_waves<T>() * WAVE, lds, stream>>>(
+                        target, indices.output_1, nullptr, s.n_edges, c
+                    );
             } else {
-                forward_kernel<T, decltype(tiles)::value, decltype(steps)::value, LONG_CHUNK>
-                    <<<grid, forward_waves<T>() * WAVE, lds, stream>>>(target, indices.output_1, s.n_edges, c);
+                forward_kernel<T, decltype(tiles)::value, decltype(steps)::value, LONG_CHUNK, false>
+                    <<<grid, forward_waves<T>() * WAVE, lds, stream>>>(
+                        target, indices.output_1, nullptr, s.n_edges, c
+                    );
             }
         });
         MOPS_HIP_CHECK(hipGetLastError());
@@ -1189,6 +1218,25 @@ void vjp(
     const DenseLayout layout = dense_layout(s);
     const DenseBuffers<T> dense = enqueue_dense<T>(workspace, layout, C, indices, s, stream);
     const bool want_edges = grad_A != nullptr || grad_B != nullptr;
+    const bool by_sender = grad_W != nullptr && orders_edges_by_sender(s);
+    void* order_workspace = static_cast<char*>(workspace) + align256(dense_bytes(layout, sizeof(T)));
+
+    // large graphs: the forward kernel over the edges in the order of their senders
+    auto launch_ordered_weights = [&](hipStream_t on, const EdgesBySender& order, int32_t first, const Shape& block) {
+        const Contraction<T> c = contraction<T>(
+            A, B + first, grad_output + first, indices.output_1, dense.to_cells, layout, block, s.L, s.n2,
+            s.n3, 1, s.n2
+        );
+        const int32_t grid = (s.n_edges + LONG_CHUNK - 1) / LONG_CHUNK;
+        const size_t lds = forward_lds(block, sizeof(T));
+        with_shape_constants(tiles_for(block.L), (s.n3 + 3) / 4, [&](auto tiles, auto steps) {
+            forward_kernel<T, decltype(tiles)::value, decltype(steps)::value, LONG_CHUNK, true>
+                <<<grid, forward_waves<T>() * WAVE, lds, on>>>(
+                    grad_W + first, order.sender, order.edge, s.n_edges, c
+                );
+        });
+        MOPS_HIP_CHECK(hipGetLastError());
+    };
 
     auto launch_weights = [&](hipStream_t on, int32_t first, const Shape& block) {
         const Contraction<T> c = contraction<T>(
@@ -1257,14 +1305,32 @@ void vjp(
         // that forks from `stream` after the dense table and joins it again.
         // (weights first: the other order is slower, 109 instead of 97 us in f32)
         SideStream side(stream);
+        EdgesBySender order{};
+        if (by_sender) {
+            order = order_edges_by_sender(indices.W_1, s.n_edges, s.n_nodes, order_workspace, side.get());
+        }
         for_each_column_block(s, [&](int32_t first, const Shape& block) {
-            launch_weights(side.get(), first, block);
+            if (by_sender) {
+                launch_ordered_weights(side.get(), order, first, block);
+            } else {
+                launch_weights(side.get(), first, block);
+            }
             launch_edges(first, block);
         });
     } else if (want_edges) {
         for_each_column_block(s, launch_edges);
     } else if (grad_W != nullptr) {
-        for_each_column_block(s, [&](int32_t first, const Shape& block) { launch_weights(stream, first, block); });
+        EdgesBySender order{};
+        if (by_sender) {
+            order = order_edges_by_sender(indices.W_1, s.n_edges, s.n_nodes, order_workspace, stream);
+        }
+        for_each_column_block(s, [&](int32_t first, const Shape& block) {
+            if (by_sender) {
+                launch_ordered_weights(stream, order, first, block);
+            } else {
+                launch_weights(stream, first, block);
+            }
+        });
     }
 }
 

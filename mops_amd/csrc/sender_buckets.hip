@@ -90,7 +90,50 @@ __global__ __launch_bounds__(THREADS) void fill_kernel(
     }
 }
 
+// workgroup `node` writes its list, sorted, and its own number next to every
+// entry; workgroup n_nodes fills what is left after the last list
+constexpr int LIST_THREADS = 64;
+
+__global__ __launch_bounds__(LIST_THREADS) void write_lists_kernel(
+    SenderBuckets buckets, int32_t n_nodes, int32_t n_edges, int32_t* __restrict__ sender_of_position,
+    int32_t* __restrict__ edge_of_position
+) {
+    __shared__ int32_t list[BUCKET_LDS_CAPACITY];
+    const int32_t node = blockIdx.x;
+    if (node == n_nodes) {
+        for (int32_t at = buckets.offsets[n_nodes] + threadIdx.x; at < n_edges; at += LIST_THREADS) {
+            sender_of_position[at] = n_nodes;
+            edge_of_position[at] = 0;
+        }
+        return;
+    }
+    const int32_t begin = buckets.offsets[node];
+    const SortedBucket sorted = sorted_bucket(buckets, node, list);
+    for (int32_t at = threadIdx.x; at < sorted.count; at += LIST_THREADS) {
+        sender_of_position[begin + at] = node;
+        edge_of_position[begin + at] = sorted.edges[at];
+    }
+}
+
 } // namespace
+
+size_t edges_by_sender_bytes(int32_t n_nodes, int32_t n_edges) {
+    return sender_buckets_bytes(n_nodes, n_edges) + 2 * align256(static_cast<size_t>(n_edges) * 4);
+}
+
+EdgesBySender order_edges_by_sender(
+    const int32_t* senders, int32_t n_edges, int32_t n_nodes, void* workspace, hipStream_t stream
+) {
+    const SenderBuckets buckets = build_sender_buckets(senders, n_edges, n_nodes, workspace, stream);
+    char* base = static_cast<char*>(workspace) + sender_buckets_bytes(n_nodes, n_edges);
+    int32_t* sender_of_position = reinterpret_cast<int32_t*>(base);
+    int32_t* edge_of_position = reinterpret_cast<int32_t*>(base + align256(static_cast<size_t>(n_edges) * 4));
+    write_lists_kernel<<<static_cast<unsigned>(n_nodes) + 1, LIST_THREADS, 0, stream>>>(
+        buckets, n_nodes, n_edges, sender_of_position, edge_of_position
+    );
+    MOPS_HIP_CHECK(hipGetLastError());
+    return EdgesBySender{sender_of_position, edge_of_position};
+}
 
 size_t sender_buckets_bytes(int32_t n_nodes, int32_t n_edges) {
     size_t nodes = static_cast<size_t>(n_nodes);

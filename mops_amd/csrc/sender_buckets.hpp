@@ -41,6 +41,27 @@ SenderBuckets build_sender_buckets(
     const int32_t* senders, int32_t n_edges, int32_t n_nodes, void* workspace, hipStream_t stream
 );
 
+/// The edges in the order of their senders, edges of one sender in ascending
+/// edge number: what a kernel needs that walks a SORTED index
+/// (segment_walk.hpp) over the senders.
+struct EdgesBySender {
+    /// [n_edges] sender of position p, non-decreasing; positions after the
+    /// last listed edge (edges whose sender is out of range are not listed)
+    /// hold n_nodes
+    const int32_t* sender;
+    /// [n_edges] edge number of position p (0 after the last listed edge)
+    const int32_t* edge;
+};
+
+/// Bytes of scratch memory order_edges_by_sender needs.
+size_t edges_by_sender_bytes(int32_t n_nodes, int32_t n_edges);
+
+/// Enqueue the kernels that order the edges by senders[e]. `workspace` must
+/// hold edges_by_sender_bytes() bytes of device memory.
+EdgesBySender order_edges_by_sender(
+    const int32_t* senders, int32_t n_edges, int32_t n_nodes, void* workspace, hipStream_t stream
+);
+
 /// Capacity (in edges) of the LDS array passed to sorted_bucket.
 constexpr int BUCKET_LDS_CAPACITY = 1024;
 
