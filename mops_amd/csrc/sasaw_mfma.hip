@@ -66,7 +66,7 @@ constexpr int MAX_L = 64;
 constexpr int T_ROW = STAGE + 1; // LDS row of one cell: 16 edges, one more to spread the banks
 constexpr int TILE_GROUP = 3;    // tiles of 16 cells handled together
 constexpr int STEP_GROUP = 8;    // steps of 4 cells handled together
-constexpr size_t LDS_BUDGET = 64 * 1024;
+constexpr size_t LDS_BUDGET = 150 * 1024; // of the 160 KB of a compute unit (beyond 64 KB a kernel has to ask)
 constexpr size_t WEIGHT_LDS_BUDGET = 96 * 1024; // the weight-gradient kernel asks for more than 64 KB
 constexpr size_t SENDER_SCAN_LIMIT = 100u * 1000 * 1000; // index reads of the in-kernel gather, all workgroups together
 
@@ -1103,6 +1103,16 @@ Contraction<T> contraction(
     return c;
 }
 
+/// A kernel that wants more than 64 KB of dynamic LDS has to say so first.
+template <typename Kernel> void allow_lds(Kernel kernel, size_t bytes) {
+    if (bytes > 64 * 1024) {
+        MOPS_HIP_CHECK(hipFuncSetAttribute(
+            reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+            static_cast<int>(bytes)
+        ));
+    }
+}
+
 /// Calls `launch(tiles, steps)` with the two shape parameters the kernels are
 /// compiled for as integral constants.
 template <typename Launch> void with_shape_constants(int tiles, int steps, Launch&& launch) {
@@ -1156,8 +1166,8 @@ bool supports(const Shape& full, size_t element_size) {
         s.n3 > MAX_INDEX || s.L < 1) {
         return false;
     }
-    return forward_lds(s, element_size) <= LDS_BUDGET && weight_gradient_lds(s, element_size) <= WEIGHT_LDS_BUDGET &&
-           edge_gradients_lds(s, element_size) <= LDS_BUDGET;
+    // (the weight-gradient kernel has the forward kernel to fall back on)
+    return forward_lds(s, element_size) <= LDS_BUDGET && edge_gradients_lds(s, element_size) <= LDS_BUDGET;
 }
 
 /// grad_W: whether the edges are first put in the order of their senders
@@ -1165,14 +1175,15 @@ bool supports(const Shape& full, size_t element_size) {
 /// Otherwise every workgroup finds the edges of its senders by reading the
 /// whole sender index (sender_gather.hpp): no preparation, which is what a
 /// small graph wants, but edges x workgroups reads.
-bool orders_edges_by_sender(const Shape& s) {
+bool orders_edges_by_sender(const Shape& s, size_t element_size) {
     const size_t groups = (static_cast<size_t>(s.n_nodes) + senders_per_group<float>() - 1) / senders_per_group<float>();
-    return static_cast<size_t>(s.n_edges) * groups > SENDER_SCAN_LIMIT;
+    return static_cast<size_t>(s.n_edges) * groups > SENDER_SCAN_LIMIT ||
+           weight_gradient_lds(widest_block(s), element_size) > WEIGHT_LDS_BUDGET;
 }
 
 size_t workspace_bytes(const Shape& s, size_t element_size) {
     return align256(dense_bytes(dense_layout(s), element_size)) +
-           (orders_edges_by_sender(s) ? edges_by_sender_bytes(s.n_nodes, s.n_edges) : 0);
+           (orders_edges_by_sender(s, element_size) ? edges_by_sender_bytes(s.n_nodes, s.n_edges) : 0);
 }
 
 template <typename T>
@@ -1195,15 +1206,17 @@ void forward(
         T* target = output + first;
         with_shape_constants(tiles_for(block.L), (s.n2 + 3) / 4, [&](auto tiles, auto steps) {
             if (short_chunks) {
-                forward_kernel<T, decltype(tiles)::value, decltype(steps)::value, SHORT_CHUNK, false>
-                    <<<grid, forward_waves<T>() * WAVE, lds, stream>>>(
-                        target, indices.output_1, nullptr, s.n_edges, c
-                    );
+                auto kernel = forward_kernel<T, decltype(tiles)::value, decltype(steps)::value, SHORT_CHUNK, false>;
+                allow_lds(kernel, lds);
+                kernel<<<grid, forward_waves<T>() * WAVE, lds, stream>>>(
+                    target, indices.output_1, nullptr, s.n_edges, c
+                );
             } else {
-                forward_kernel<T, decltype(tiles)::value, decltype(steps)::value, LONG_CHUNK, false>
-                    <<<grid, forward_waves<T>() * WAVE, lds, stream>>>(
-                        target, indices.output_1, nullptr, s.n_edges, c
-                    );
+                auto kernel = forward_kernel<T, decltype(tiles)::value, decltype(steps)::value, LONG_CHUNK, false>;
+                allow_lds(kernel, lds);
+                kernel<<<grid, forward_waves<T>() * WAVE, lds, stream>>>(
+                    target, indices.output_1, nullptr, s.n_edges, c
+                );
             }
         });
         MOPS_HIP_CHECK(hipGetLastError());
@@ -1218,7 +1231,7 @@ void vjp(
     const DenseLayout layout = dense_layout(s);
     const DenseBuffers<T> dense = enqueue_dense<T>(workspace, layout, C, indices, s, stream);
     const bool want_edges = grad_A != nullptr || grad_B != nullptr;
-    const bool by_sender = grad_W != nullptr && orders_edges_by_sender(s);
+    const bool by_sender = grad_W != nullptr && orders_edges_by_sender(s, sizeof(T));
     void* order_workspace = static_cast<char*>(workspace) + align256(dense_bytes(layout, sizeof(T)));
 
     // large graphs: the forward kernel over the edges in the order of their senders
@@ -1230,10 +1243,11 @@ void vjp(
         const int32_t grid = (s.n_edges + LONG_CHUNK - 1) / LONG_CHUNK;
         const size_t lds = forward_lds(block, sizeof(T));
         with_shape_constants(tiles_for(block.L), (s.n3 + 3) / 4, [&](auto tiles, auto steps) {
-            forward_kernel<T, decltype(tiles)::value, decltype(steps)::value, LONG_CHUNK, true>
-                <<<grid, forward_waves<T>() * WAVE, lds, on>>>(
-                    grad_W + first, order.sender, order.edge, s.n_edges, c
-                );
+            auto kernel = forward_kernel<T, decltype(tiles)::value, decltype(steps)::value, LONG_CHUNK, true>;
+            allow_lds(kernel, lds);
+            kernel<<<grid, forward_waves<T>() * WAVE, lds, on>>>(
+                grad_W + first, order.sender, order.edge, s.n_edges, c
+            );
         });
         MOPS_HIP_CHECK(hipGetLastError());
     };
@@ -1293,8 +1307,9 @@ void vjp(
         const int32_t grid = (s.n_edges + STAGE - 1) / STAGE;
         const size_t lds = edge_gradients_lds(block, sizeof(T));
         with_shape_constants(tiles_for(block.L), (s.n2 + 3) / 4, [&](auto tiles_constant, auto steps) {
-            edge_gradients_kernel<T, decltype(tiles_constant)::value, decltype(steps)::value>
-                <<<grid, WAVE, lds, stream>>>(args);
+            auto kernel = edge_gradients_kernel<T, decltype(tiles_constant)::value, decltype(steps)::value>;
+            allow_lds(kernel, lds);
+            kernel<<<grid, WAVE, lds, stream>>>(args);
         });
         MOPS_HIP_CHECK(hipGetLastError());
     };
