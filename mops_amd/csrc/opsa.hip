@@ -201,6 +201,112 @@ __global__ __launch_bounds__(BLOCK) void forward_kernel(
     );
 }
 
+// ---------------------------------------------------------------------------
+// forward for LONG segments (pooling over whole structures: a few output rows,
+// thousands of edges each). One wavefront per segment would leave the device
+// idle, so segments are cut every SPLIT positions (segment_walk.hpp); a piece
+// that is a whole segment goes to its output row as above, the others to
+//   tail[b]  the piece that begins its segment inside block b and leaves it
+//   head[b]  the piece that entered block b from the block before
+// (at most one of each per block of SPLIT positions), and
+// combine_pieces_kernel adds tail[b] + head[b + 1] + head[b + 2] + ... in that
+// order for every cut segment: no atomics, one fixed order.
+// ---------------------------------------------------------------------------
+constexpr int SPLIT = 256;
+
+template <typename T, int NT, bool WEIGHTED>
+__global__ __launch_bounds__(BLOCK) void forward_split_kernel(
+    T* __restrict__ output,
+    T* __restrict__ tails,
+    T* __restrict__ heads,
+    const T* __restrict__ A,
+    const T* __restrict__ B,
+    const T* __restrict__ W,
+    const int32_t* __restrict__ indices_W,
+    const int32_t* __restrict__ indices_output,
+    int32_t n_edges,
+    int32_t n_output,
+    int32_t K,
+    int32_t L
+) {
+    const int32_t wave_index =
+        __builtin_amdgcn_readfirstlane(blockIdx.x * WAVES_PER_BLOCK + (threadIdx.x >> 6));
+    const int lane = threadIdx.x & (WAVE - 1);
+    const size_t row_elements = static_cast<size_t>(K) * L;
+    walk_split_segments<CHUNK, SPLIT>(
+        indices_output,
+        n_edges,
+        n_output,
+        wave_index,
+        [&](int32_t row, int32_t first, int32_t last, bool from_start, bool to_end) {
+            const int32_t block = first / SPLIT;
+            T* target = from_start && to_end ? output + row * row_elements
+                        : from_start         ? tails + block * row_elements
+                                             : heads + block * row_elements;
+            forward_segment<T, NT, WEIGHTED>(target, A, B, W, indices_W, n_output, first, last, K, L);
+        },
+        [&](int32_t begin, int32_t end) {
+            T* base = output + begin * row_elements;
+            const size_t count = (end - begin) * row_elements;
+            for (size_t i = lane; i < count; i += WAVE) {
+                base[i] = T(0);
+            }
+        }
+    );
+}
+
+constexpr int COMBINE_THREADS = 256;
+
+/// Workgroup b: if a segment begins in block b of SPLIT positions and goes on
+/// into block b + 1, its output row = tail[b] + head[b + 1] + ... (all its pieces).
+template <typename T>
+__global__ __launch_bounds__(COMBINE_THREADS) void combine_pieces_kernel(
+    T* __restrict__ output,
+    const T* __restrict__ tails,
+    const T* __restrict__ heads,
+    const int32_t* __restrict__ indices_output,
+    int32_t n_edges,
+    int32_t n_output,
+    int32_t row_elements
+) {
+    const int32_t block = blockIdx.x;
+    const int32_t cut = (block + 1) * SPLIT; // first position of the next block
+    if (cut >= n_edges) {
+        return;
+    }
+    const int32_t row = indices_output[cut];
+    if (indices_output[cut - 1] != row || !in_bounds(row, n_output)) {
+        return; // nothing crosses this cut
+    }
+    if (block > 0 && indices_output[block * SPLIT - 1] == row) {
+        return; // the segment began before this block: another workgroup adds it up
+    }
+    // blocks block + 1 .. last_block hold head pieces of this row
+    int32_t last_block = block + 1;
+    while ((last_block + 1) * SPLIT < n_edges && indices_output[(last_block + 1) * SPLIT] == row) {
+        last_block++;
+    }
+    constexpr int AHEAD = 8;
+    for (int32_t element = threadIdx.x; element < row_elements; element += COMBINE_THREADS) {
+        T sum = tails[static_cast<size_t>(block) * row_elements + element];
+        for (int32_t b0 = block + 1; b0 <= last_block; b0 += AHEAD) {
+            T piece[AHEAD];
+#pragma unroll
+            for (int u = 0; u < AHEAD; u++) {
+                const int32_t b = min(b0 + u, last_block);
+                piece[u] = heads[static_cast<size_t>(b) * row_elements + element];
+            }
+#pragma unroll
+            for (int u = 0; u < AHEAD; u++) {
+                if (b0 + u <= last_block) {
+                    sum += piece[u];
+                }
+            }
+        }
+        output[static_cast<size_t>(row) * row_elements + element] = sum;
+    }
+}
+
 // every element of `data` := 0 (used when there is no edge at all)
 template <typename T>
 __global__ __launch_bounds__(256) void zero_kernel(T* __restrict__ data, size_t count) {
@@ -1008,6 +1114,35 @@ void launch_forward(
         return;
     }
     const unsigned blocks = blocks_for(n_edges);
+    // few rows with many edges each: cut the segments and add the pieces up
+    // (twice SPLIT edges per row on average, or it is not worth a second kernel)
+    if (static_cast<size_t>(n_edges) >= static_cast<size_t>(n_output) * 2 * SPLIT && n_edges > SPLIT) {
+        const size_t row_elements = static_cast<size_t>(K) * L;
+        const size_t n_split_blocks = ceil_div(static_cast<size_t>(n_edges), SPLIT);
+        const size_t pieces_bytes = align256(n_split_blocks * row_elements * sizeof(T));
+        char* workspace = static_cast<char*>(scratch(2 * pieces_bytes));
+        T* tails = reinterpret_cast<T*>(workspace);
+        T* heads = reinterpret_cast<T*>(workspace + pieces_bytes);
+#define MOPS_LAUNCH_SPLIT(NT)                                                                      \
+    forward_split_kernel<T, NT, WEIGHTED><<<blocks, BLOCK, 0, stream>>>(                           \
+        output.data, tails, heads, A.data, B.data, W, indices_W, indices_output.data, n_edges,     \
+        n_output, K, L                                                                             \
+    )
+        if (L <= 16) {
+            MOPS_LAUNCH_SPLIT(1);
+        } else if (L <= 32) {
+            MOPS_LAUNCH_SPLIT(2);
+        } else {
+            MOPS_LAUNCH_SPLIT(4);
+        }
+#undef MOPS_LAUNCH_SPLIT
+        combine_pieces_kernel<T><<<static_cast<unsigned>(n_split_blocks), COMBINE_THREADS, 0, stream>>>(
+            output.data, tails, heads, indices_output.data, n_edges, n_output,
+            static_cast<int32_t>(row_elements)
+        );
+        finish_call(operation);
+        return;
+    }
 #define MOPS_LAUNCH_FORWARD(NT)                                                                    \
     forward_kernel<T, NT, WEIGHTED><<<blocks, BLOCK, 0, stream>>>(                                 \
         output.data, A.data, B.data, W, indices_W, indices_output.data, n_edges, n_output, K, L    \

@@ -14,6 +14,12 @@
 // owner of position 0 learns the rows before the first value and the owner of
 // the last position the rows after the last value. Calling `on_empty_rows`
 // for these ranges lets a kernel write every output row exactly once.
+//
+// SPLIT > 0 (walk_split_segments): segments are additionally cut at every
+// multiple of SPLIT positions, so that no piece is longer than SPLIT and a
+// long segment is shared by many wavefronts. A piece is reported with whether
+// it begins where its segment begins and ends where its segment ends; whoever
+// calls this has to add up the pieces of a cut segment afterwards.
 #ifndef MOPS_AMD_SEGMENT_WALK_HPP
 #define MOPS_AMD_SEGMENT_WALK_HPP
 
@@ -29,16 +35,18 @@ namespace mops::amd {
 /// the wavefront (uniform). CHUNK <= 64.
 ///   on_segment(row, first, last)  all lanes, uniform arguments, 0 <= row < n_rows
 ///   on_empty_rows(begin, end)     all lanes, rows in [begin, end) receive nothing
-template <int CHUNK, typename SegmentFn, typename EmptyRowsFn>
-__device__ __forceinline__ void walk_owned_segments(
+///   on_piece(row, first, last, from_start, to_end)   (walk_split_segments)
+template <int CHUNK, int SPLIT, typename PieceFn, typename EmptyRowsFn>
+__device__ __forceinline__ void walk_pieces(
     const int32_t* __restrict__ sorted_index,
     int32_t n_input,
     int32_t n_rows,
     int32_t wave_index,
-    SegmentFn&& on_segment,
+    PieceFn&& on_piece,
     EmptyRowsFn&& on_empty_rows
 ) {
     static_assert(CHUNK >= 1 && CHUNK <= WAVE, "one index value per lane");
+    static_assert(SPLIT == 0 || SPLIT % CHUNK == 0, "cuts fall on chunk boundaries");
     const int lane = threadIdx.x & (WAVE - 1);
     const int32_t chunk_begin = wave_index * CHUNK;
     if (chunk_begin >= n_input) {
@@ -53,9 +61,11 @@ __device__ __forceinline__ void walk_owned_segments(
     // another round trip to memory
     const int32_t ahead_position = chunk_begin + CHUNK + lane;
     const int32_t ahead = load_or_zero(sorted_index, static_cast<size_t>(ahead_position), ahead_position < n_input);
-    const bool starts_here = inside && (position == 0 || mine != before);
+    const bool segment_starts_here = inside && (position == 0 || mine != before);
+    const bool starts_here = segment_starts_here || (SPLIT > 0 && inside && position % (SPLIT > 0 ? SPLIT : 1) == 0);
 
     unsigned long long starts = __ballot(starts_here);
+    const unsigned long long segment_starts = __ballot(segment_starts_here);
     while (starts != 0) {
         const int start_lane = __ffsll(static_cast<long long>(starts)) - 1;
         starts &= starts - 1;
@@ -63,32 +73,50 @@ __device__ __forceinline__ void walk_owned_segments(
         const int32_t row = __shfl(mine, start_lane);
         const int32_t previous_row = __shfl(before, start_lane); // -1 at position 0
 
+        const bool from_start = ((segment_starts >> start_lane) & 1) != 0;
+        bool to_end = true;
         int32_t last;
         if (starts != 0) {
-            last = chunk_begin + __ffsll(static_cast<long long>(starts)) - 1;
+            const int next_lane = __ffsll(static_cast<long long>(starts)) - 1;
+            last = chunk_begin + next_lane;
+            to_end = ((segment_starts >> next_lane) & 1) != 0;
         } else {
-            // the run reaches the end of the chunk: follow it
-            last = n_input;
-            for (int32_t probe = chunk_begin + CHUNK; probe < n_input; probe += WAVE) {
+            // the run reaches the end of the chunk: follow it (to the next cut at most)
+            int32_t limit = n_input;
+            if constexpr (SPLIT > 0) {
+                limit = min(n_input, (first / SPLIT + 1) * SPLIT);
+            }
+            last = limit;
+            bool found_end = false;
+            for (int32_t probe = chunk_begin + CHUNK; probe < limit; probe += WAVE) {
                 const int32_t at = probe + lane;
                 const bool first_look = probe == chunk_begin + CHUNK; // uniform
                 const int32_t value = first_look ? ahead : load_or_zero(sorted_index, static_cast<size_t>(at), at < n_input);
                 const bool differs = at >= n_input || value != row;
                 const unsigned long long mask = __ballot(differs);
                 if (mask != 0) {
-                    last = min(probe + __ffsll(static_cast<long long>(mask)) - 1, n_input);
+                    const int32_t end = min(probe + __ffsll(static_cast<long long>(mask)) - 1, n_input);
+                    if (end <= limit) {
+                        last = end;
+                        found_end = true;
+                    }
                     break;
+                }
+            }
+            if constexpr (SPLIT > 0) {
+                if (!found_end && last < n_input) {
+                    to_end = sorted_index[last] != row; // the piece stops at a cut: does the segment?
                 }
             }
         }
 
         const int32_t empty_begin = max(previous_row + 1, 0);
         const int32_t empty_end = min(row, n_rows);
-        if (empty_begin < empty_end) {
+        if (from_start && empty_begin < empty_end) {
             on_empty_rows(empty_begin, empty_end);
         }
         if (in_bounds(row, n_rows)) {
-            on_segment(row, first, last);
+            on_piece(row, first, last, from_start, to_end);
         }
     }
 
@@ -99,6 +127,34 @@ __device__ __forceinline__ void walk_owned_segments(
             on_empty_rows(tail_begin, n_rows);
         }
     }
+}
+
+template <int CHUNK, typename SegmentFn, typename EmptyRowsFn>
+__device__ __forceinline__ void walk_owned_segments(
+    const int32_t* __restrict__ sorted_index,
+    int32_t n_input,
+    int32_t n_rows,
+    int32_t wave_index,
+    SegmentFn&& on_segment,
+    EmptyRowsFn&& on_empty_rows
+) {
+    walk_pieces<CHUNK, 0>(
+        sorted_index, n_input, n_rows, wave_index,
+        [&](int32_t row, int32_t first, int32_t last, bool, bool) { on_segment(row, first, last); }, on_empty_rows
+    );
+}
+
+template <int CHUNK, int SPLIT, typename PieceFn, typename EmptyRowsFn>
+__device__ __forceinline__ void walk_split_segments(
+    const int32_t* __restrict__ sorted_index,
+    int32_t n_input,
+    int32_t n_rows,
+    int32_t wave_index,
+    PieceFn&& on_piece,
+    EmptyRowsFn&& on_empty_rows
+) {
+    static_assert(SPLIT > 0, "distance between cuts");
+    walk_pieces<CHUNK, SPLIT>(sorted_index, n_input, n_rows, wave_index, on_piece, on_empty_rows);
 }
 
 } // namespace mops::amd

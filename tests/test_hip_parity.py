@@ -45,6 +45,10 @@ CASES = {
         "long_segments": lambda s, d: support.opsa_case(s, d, J=3000, K=5, L=7, n_out=6),
         "wide": lambda s, d: support.opsa_case(s, d, J=400, K=40, L=33, n_out=21, allow_empty=True),
         "mostly_empty": lambda s, d: support.opsa_case(s, d, J=20, K=4, L=4, n_out=300, allow_empty=True),
+        "pooling": lambda s, d: support.opsa_case(s, d, J=5000, K=13, L=20, n_out=7),
+        "pooling_mixed_lengths": lambda s, d: _with_lengths(
+            support.opsa_case(s, d, J=sum(MIXED_LENGTHS), K=5, L=40, n_out=len(MIXED_LENGTHS)), "indices_output", MIXED_LENGTHS
+        ),
         "many_columns": lambda s, d: support.opsa_case(s, d, J=700, K=16, L=128, n_out=31, allow_empty=True),
         "ragged_columns": lambda s, d: support.opsa_case(s, d, J=500, K=20, L=70, n_out=23, allow_empty=True),
     },
@@ -54,6 +58,10 @@ CASES = {
         "long_segments": lambda s, d: support.opsaw_case(s, d, E=3000, K=5, L=7, n_nodes=6),
         "hub_sender": lambda s, d: _hub(support.opsaw_case(s, d, E=2600, K=3, L=5, n_nodes=9), "indices_W"),
         "mostly_empty": lambda s, d: support.opsaw_case(s, d, E=20, K=4, L=4, n_nodes=300, allow_empty=True),
+        "pooling": lambda s, d: support.opsaw_case(s, d, E=5000, K=13, L=32, n_nodes=7),
+        "pooling_mixed_lengths": lambda s, d: _with_lengths(
+            support.opsaw_case(s, d, E=sum(MIXED_LENGTHS), K=3, L=17, n_nodes=len(MIXED_LENGTHS)), "indices_output", MIXED_LENGTHS
+        ),
         "many_columns": lambda s, d: support.opsaw_case(s, d, E=700, K=32, L=192, n_nodes=31, allow_empty=True),
         "ragged_columns": lambda s, d: support.opsaw_case(s, d, E=500, K=9, L=131, n_nodes=23, allow_empty=True),
     },
@@ -117,6 +125,18 @@ def _one_receiver(case, key):
     index[len(index) // 20 : len(index) * 19 // 20] = 3
     case[key] = np.sort(index)
     return case
+
+
+def _with_lengths(case, key, lengths):
+    """Scatter index with exactly these segment lengths (row r gets lengths[r] edges)."""
+    index = np.repeat(np.arange(len(lengths)), lengths).astype(np.int32)
+    assert len(index) == len(case[key])
+    case[key] = index
+    return case
+
+
+# lengths around the distance at which long segments are cut (256), rows without edges, one row over many cuts
+MIXED_LENGTHS = [0, 1700, 3, 0, 2300, 255, 256, 257, 512, 1, 0, 1900, 0, 769]
 
 
 def _hub(case, key):
