@@ -30,6 +30,7 @@
 // order is fixed (ascending edge number in steps of four), so results are
 // bit-reproducible.
 #include <algorithm>
+#include <memory>
 
 #include "mops/opsa.hpp"
 #include "mops/opsaw.hpp"
@@ -1198,6 +1199,16 @@ void launch_vjp(
         want_W ? static_cast<char*>(scratch(edge_w_bytes + buckets_bytes)) : nullptr;
     T* edge_W = want_W ? reinterpret_cast<T*>(workspace) : nullptr;
 
+    // the lists of edges per sender do not depend on the kernels below: they are
+    // built beside them, on a side stream that joins before the lists are used
+    SenderBuckets buckets{};
+    const bool use_buckets = want_W && n_output > 0 && L > 0 && !gather_in_kernel;
+    std::unique_ptr<SideStream> beside;
+    if (use_buckets) {
+        beside = std::make_unique<SideStream>(stream);
+        buckets = build_sender_buckets(indices_W, n_edges, n_output, workspace + edge_w_bytes, beside->get());
+    }
+
     // degenerate shapes: a gradient that sums over an empty axis is zero
     if (want_A && L == 0 && n_edges > 0 && K > 0) {
         const size_t count = static_cast<size_t>(n_edges) * K;
@@ -1299,9 +1310,8 @@ void launch_vjp(
         sum_by_sender_kernel<T><<<blocks, GATHER_SENDERS * WAVE, 0, stream>>>(
             grad_W.data, edge_W, indices_W, n_edges, n_output, L, aligned
         );
-    } else if (want_W && n_output > 0 && L > 0) {
-        SenderBuckets buckets =
-            build_sender_buckets(indices_W, n_edges, n_output, workspace + edge_w_bytes, stream);
+    } else if (use_buckets) {
+        beside.reset(); // joins
         int threads = std::min(256, round_up_wave(L));
         gather_weights_kernel<T><<<n_output, threads, 0, stream>>>(grad_W.data, edge_W, buckets, L);
     }
