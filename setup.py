@@ -6,6 +6,7 @@ package data, the way the reference's wheels carry their ``libmops.so``
 (python/mops/setup.py of lab-cosmo/mops builds it with CMake).
 """
 import os
+import shutil
 import subprocess
 
 from setuptools import setup
@@ -18,6 +19,10 @@ class build_py_with_library(build_py):
     def run(self):
         subprocess.run(["make", "-C", os.path.join(ROOT, "mops_amd", "csrc"), "-j8"], check=True)
         super().run()
+        # the C / C++ headers travel inside the package, where cmake/mops/mops-config.cmake looks first
+        target = os.path.join(self.build_lib, "mops_amd", "include")
+        shutil.rmtree(target, ignore_errors=True)
+        shutil.copytree(os.path.join(ROOT, "include"), target)
 
 
 setup(
@@ -25,7 +30,7 @@ setup(
     version="0.1.0",
     description="lab-cosmo/mops operations on AMD MI355X (gfx950): HIP kernels behind the mops C ABI",
     packages=["mops_amd"],
-    package_data={"mops_amd": ["lib/libmops.so"]},
+    package_data={"mops_amd": ["lib/libmops.so", "cmake/mops/*.cmake"]},
     python_requires=">=3.9",
     install_requires=["numpy"],
     extras_require={"torch": ["torch"]},
