@@ -22,12 +22,24 @@ CASES = {
     "opsa": lambda d: support.opsa_case(23, d, J=2000, K=13, L=20, n_out=70, allow_empty=True),
     "opsaw": lambda d: support.opsaw_case(24, d, E=2000, K=13, L=32, n_nodes=70, allow_empty=True),
     "sasaw": lambda d: support.sasaw_case(25, d, E=2000, nA=9, L=32, n_nodes=70, allow_empty=True),
+    # paths with more than one kernel per call and with scratch memory between them:
+    # segments cut into pieces and added up (OPSA forward of long segments)
+    "opsa_pooling": lambda d: support.opsa_case(26, d, J=6000, K=13, L=20, n_out=8),
+    # blocks of 64 columns, grad_A added to by one launch after the other
+    "sasaw_many_columns": lambda d: support.sasaw_case(27, d, E=1500, nA=9, L=160, n_nodes=50, allow_empty=True),
+    # edges ordered by sender on a side stream (edges x nodes / 4 beyond the in-kernel gather)
+    "sasaw_many_senders": lambda d: support.sasaw_case(28, d, E=30000, nA=4, L=16, n_nodes=16000, n2=4, n3=4, N=30, allow_empty=True),
 }
+
+
+def _operation(name):
+    return name.split("_")[0]
 
 
 def _call(op, case):
     import mops_amd
 
+    op = _operation(op)
     spec = OPS[op]
     forward = getattr(mops_amd, spec.function)
     backward = getattr(mops_amd, spec.function + "_vjp")
