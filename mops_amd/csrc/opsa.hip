@@ -1009,6 +1009,71 @@ __global__ __launch_bounds__(GATHER_SENDERS* WAVE) void sum_by_sender_kernel(
     }
 }
 
+// The same sum over lists that are already there (sender_buckets.hpp: the edges in
+// the order of their senders, built beside the per-edge kernel on a side
+// stream): one wavefront per sender, sixteen rows in flight.
+constexpr int LISTED_WAVES = 4;
+
+template <typename T>
+__global__ __launch_bounds__(LISTED_WAVES* WAVE) void sum_listed_rows_kernel(
+    T* __restrict__ grad_W, const T* __restrict__ edge_W, const int32_t* __restrict__ offsets,
+    const int32_t* __restrict__ edge_of_position, int32_t n_nodes, int32_t L
+) {
+    const int lane = threadIdx.x & (WAVE - 1);
+    const int32_t node = __builtin_amdgcn_readfirstlane(blockIdx.x * LISTED_WAVES + (threadIdx.x >> 6));
+    if (node >= n_nodes) {
+        return;
+    }
+    const int32_t begin = offsets[node];
+    const int32_t end = offsets[node + 1];
+    T sum[GATHER_COLUMNS];
+    uint32_t column[GATHER_COLUMNS];
+#pragma unroll
+    for (int c = 0; c < GATHER_COLUMNS; c++) {
+        sum[c] = T(0);
+        column[c] = min(lane + c * WAVE, L - 1);
+    }
+    constexpr int ROWS = sizeof(T) == 8 ? 8 : 16;
+    for (int32_t p0 = begin; p0 < end; p0 += WAVE) {
+        const int32_t n = min(WAVE, end - p0);
+        const int32_t my_edge = lane < n ? edge_of_position[p0 + lane] : 0;
+#pragma unroll 1
+        for (int32_t k0 = 0; k0 < n; k0 += ROWS) {
+            T values[ROWS][GATHER_COLUMNS];
+#pragma unroll
+            for (int k = 0; k < ROWS; k++) {
+                // beyond n: some row that exists, left out of the sum
+                const int32_t edge = __builtin_amdgcn_readlane(my_edge, min(k0 + k, WAVE - 1));
+                const T* row = edge_W + static_cast<size_t>(edge) * L;
+#pragma unroll
+                for (int c = 0; c < GATHER_COLUMNS; c++) {
+                    if (c * WAVE < L) {
+                        values[k][c] = row[column[c]];
+                    }
+                }
+            }
+#pragma unroll
+            for (int k = 0; k < ROWS; k++) {
+                if (k0 + k < n) {
+#pragma unroll
+                    for (int c = 0; c < GATHER_COLUMNS; c++) {
+                        if (c * WAVE < L) {
+                            sum[c] += values[k][c];
+                        }
+                    }
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int c = 0; c < GATHER_COLUMNS; c++) {
+        const int32_t l = lane + c * WAVE;
+        if (l < L) {
+            grad_W[static_cast<size_t>(node) * L + l] = sum[c];
+        }
+    }
+}
+
 // vjp for rows too wide for the LDS tile of vjp_kernel: one wavefront per
 // edge, lanes over l in chunks of 64, the receiver's grad_output row read
 // from global memory (L2). grad_A[e, k] is a fixed shuffle tree over the
@@ -1192,9 +1257,11 @@ void launch_vjp(
     // (edges x workgroups) is small, quadratic in the size of the graph beyond
     const size_t index_reads =
         static_cast<size_t>(n_edges) * ceil_div(static_cast<size_t>(std::max(n_output, 1)), GATHER_SENDERS);
-    const bool gather_in_kernel = L <= GATHER_COLUMNS * WAVE && n_edges > 0 && index_reads <= SENDER_SCAN_LIMIT;
+    const bool narrow_rows = L <= GATHER_COLUMNS * WAVE;
+    // (at 60 000 edges the lists cost more than the scans: 52 us against 32 for the whole vjp)
+    const bool gather_in_kernel = narrow_rows && n_edges > 0 && index_reads <= SENDER_SCAN_LIMIT;
     const size_t buckets_bytes =
-        want_W && !gather_in_kernel ? sender_buckets_bytes(n_output, n_edges) : 0;
+        want_W && !gather_in_kernel ? edges_by_sender_bytes(n_output, n_edges) : 0;
     char* workspace =
         want_W ? static_cast<char*>(scratch(edge_w_bytes + buckets_bytes)) : nullptr;
     T* edge_W = want_W ? reinterpret_cast<T*>(workspace) : nullptr;
@@ -1202,11 +1269,16 @@ void launch_vjp(
     // the lists of edges per sender do not depend on the kernels below: they are
     // built beside them, on a side stream that joins before the lists are used
     SenderBuckets buckets{};
+    EdgesBySender by_sender{};
     const bool use_buckets = want_W && n_output > 0 && L > 0 && !gather_in_kernel;
     std::unique_ptr<SideStream> beside;
     if (use_buckets) {
         beside = std::make_unique<SideStream>(stream);
-        buckets = build_sender_buckets(indices_W, n_edges, n_output, workspace + edge_w_bytes, beside->get());
+        if (narrow_rows) {
+            by_sender = order_edges_by_sender(indices_W, n_edges, n_output, workspace + edge_w_bytes, beside->get());
+        } else {
+            buckets = build_sender_buckets(indices_W, n_edges, n_output, workspace + edge_w_bytes, beside->get());
+        }
     }
 
     // degenerate shapes: a gradient that sums over an empty axis is zero
@@ -1312,8 +1384,15 @@ void launch_vjp(
         );
     } else if (use_buckets) {
         beside.reset(); // joins
-        int threads = std::min(256, round_up_wave(L));
-        gather_weights_kernel<T><<<n_output, threads, 0, stream>>>(grad_W.data, edge_W, buckets, L);
+        if (narrow_rows) {
+            const unsigned blocks = static_cast<unsigned>(ceil_div(static_cast<size_t>(n_output), LISTED_WAVES));
+            sum_listed_rows_kernel<T><<<blocks, LISTED_WAVES * WAVE, 0, stream>>>(
+                grad_W.data, edge_W, by_sender.offsets, by_sender.edge, n_output, L
+            );
+        } else {
+            int threads = std::min(256, round_up_wave(L));
+            gather_weights_kernel<T><<<n_output, threads, 0, stream>>>(grad_W.data, edge_W, buckets, L);
+        }
     }
     finish_call(operation);
 }

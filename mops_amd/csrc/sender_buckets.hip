@@ -132,7 +132,7 @@ EdgesBySender order_edges_by_sender(
         buckets, n_nodes, n_edges, sender_of_position, edge_of_position
     );
     MOPS_HIP_CHECK(hipGetLastError());
-    return EdgesBySender{sender_of_position, edge_of_position};
+    return EdgesBySender{sender_of_position, edge_of_position, buckets.offsets};
 }
 
 size_t sender_buckets_bytes(int32_t n_nodes, int32_t n_edges) {

@@ -51,6 +51,8 @@ struct EdgesBySender {
     const int32_t* sender;
     /// [n_edges] edge number of position p (0 after the last listed edge)
     const int32_t* edge;
+    /// [n_nodes + 1] first position of every sender's edges
+    const int32_t* offsets;
 };
 
 /// Bytes of scratch memory order_edges_by_sender needs.
