@@ -30,11 +30,14 @@
 #include "index_validation.hpp"
 #include "elementwise.hpp"
 #include "runtime.hpp"
+#include "sender_buckets.hpp"
 
 namespace mops::amd {
 namespace {
 
 constexpr size_t LDS_BUDGET = 60 * 1024;
+constexpr int32_t MANY_ROWS = 4096;                     // from here on the vjp goes by feature
+constexpr size_t BY_FEATURE_LDS_BUDGET = 140 * 1024;    // its two tiles, of the 160 KB of a compute unit
 
 // ---------------------------------------------------------------------------
 // forward. LDS: a[nA][R] partial[G][R]
@@ -362,6 +365,123 @@ __global__ __launch_bounds__(WAVE) void vjp_ordered_kernel(
             total += accumulator[(static_cast<size_t>(group) * feature_count + feature) * R + row];
         }
         dst[static_cast<size_t>(row) * nA + feature] = total;
+    }
+}
+
+// ---------------------------------------------------------------------------
+// vjp for MANY rows, by feature. With thousands of rows the kernel above is
+// bound by its LDS add instructions (one per factor of every monomial and
+// row). Here nothing is scattered: the table is first turned round on the
+// device (sender_buckets.hpp, the same counting sort that orders edges by
+// sender: for every feature a the list of pairs q = j * ORDER + f with
+// P[j, f] = a, in ascending q), and then a wavefront owns (64 rows, one
+// feature at a time): a lane is a row, walks the feature's list, multiplies
+// up the OTHER factors of its row from an LDS tile of A and adds the terms in
+// a register:
+//
+//   grad_A[i, a] = gO[i] * sum over (j, f) in list(a) of C[j] * prod_{k != f} A[i, P[j, k]]
+//
+// The list entries are read 64 at a time, one per lane, and handed out to all
+// lanes through readlane. One fixed order (ascending q), no atomics.
+// LDS: a[nA][ROW_PITCH] out[64][out_pitch]
+// ---------------------------------------------------------------------------
+constexpr int FEATURE_ROWS = WAVE;          // rows per workgroup
+constexpr int FEATURE_ROW_PITCH = WAVE + 1; // distance between features in the tile of A
+constexpr int FEATURE_WAVES = 16;
+
+template <typename T, int ORDER>
+__global__ __launch_bounds__(FEATURE_WAVES* WAVE) void vjp_by_feature_kernel(
+    T* __restrict__ grad_A,
+    const T* __restrict__ grad_output,
+    const T* __restrict__ A,
+    const T* __restrict__ C,
+    const int32_t* __restrict__ P,
+    const int32_t* __restrict__ list_begin, // [nA + 1]
+    const int32_t* __restrict__ list,       // pairs q = j * ORDER + f, grouped by feature
+    int32_t n_rows,
+    int32_t nA,
+    int32_t out_pitch
+) {
+    extern __shared__ __align__(16) unsigned char lds_bytes[];
+    T* a_stage = reinterpret_cast<T*>(lds_bytes);
+    T* out = a_stage + static_cast<size_t>(nA) * FEATURE_ROW_PITCH;
+    constexpr int THREADS = FEATURE_WAVES * WAVE;
+    constexpr int OTHERS = ORDER - 1;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & (WAVE - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int32_t row0 = blockIdx.x * FEATURE_ROWS;
+    const int32_t rows = min(FEATURE_ROWS, n_rows - row0);
+
+    const T* a_src = A + static_cast<size_t>(row0) * nA;
+    constexpr int STAGE_LOADS = 4;
+    for (int32_t i0 = tid; i0 < FEATURE_ROWS * nA; i0 += STAGE_LOADS * THREADS) {
+        T value[STAGE_LOADS];
+#pragma unroll
+        for (int u = 0; u < STAGE_LOADS; u++) {
+            const int32_t i = i0 + u * THREADS;
+            value[u] = load_or_zero(a_src, static_cast<size_t>(i), i < rows * nA); // rows beyond the end: zeros
+        }
+#pragma unroll
+        for (int u = 0; u < STAGE_LOADS; u++) {
+            const int32_t i = i0 + u * THREADS;
+            if (i < FEATURE_ROWS * nA) {
+                const int32_t row = i / nA;
+                a_stage[(i - row * nA) * FEATURE_ROW_PITCH + row] = value[u];
+            }
+        }
+    }
+    const T upstream = load_or_zero(grad_output, static_cast<size_t>(row0 + lane), lane < rows);
+    __syncthreads();
+
+    const T* mine = a_stage + lane;
+    for (int32_t feature = wave; feature < nA; feature += FEATURE_WAVES) {
+        const int32_t begin = list_begin[feature];
+        const int32_t end = list_begin[feature + 1];
+        T sum = T(0);
+        for (int32_t p0 = begin; p0 < end; p0 += WAVE) {
+            const int32_t n = min(WAVE, end - p0);
+            // my entry of the batch: coefficient (zero: no entry, or a factor out of range) and
+            // where the other factors' values are in the tile
+            const int32_t q = lane < n ? list[p0 + lane] : 0;
+            const int32_t j = q / ORDER;
+            const int32_t f = q - j * ORDER;
+            T coefficient = lane < n ? C[j] : T(0);
+            int32_t other[OTHERS > 0 ? OTHERS : 1];
+#pragma unroll
+            for (int k = 0; k < OTHERS; k++) {
+                const int32_t factor = P[static_cast<size_t>(j) * ORDER + (k < f ? k : k + 1)];
+                const bool valid = in_bounds(factor, nA);
+                other[k] = (valid ? factor : 0) * FEATURE_ROW_PITCH;
+                coefficient = valid ? coefficient : T(0);
+            }
+            int32_t words[sizeof(T) / 4];
+            __builtin_memcpy(words, &coefficient, sizeof(T));
+#pragma unroll 4
+            for (int32_t u = 0; u < n; u++) {
+                int32_t uniform[sizeof(T) / 4];
+#pragma unroll
+                for (int w = 0; w < static_cast<int>(sizeof(T) / 4); w++) {
+                    uniform[w] = __builtin_amdgcn_readlane(words[w], u);
+                }
+                T term;
+                __builtin_memcpy(&term, uniform, sizeof(T));
+#pragma unroll
+                for (int k = 0; k < OTHERS; k++) {
+                    term *= mine[__builtin_amdgcn_readlane(other[k], u)];
+                }
+                sum += term;
+            }
+        }
+        out[lane * out_pitch + feature] = upstream * sum;
+    }
+    __syncthreads();
+    // the 64 rows of grad_A are one contiguous piece of memory
+    T* target = grad_A + static_cast<size_t>(row0) * nA;
+    for (int32_t i = tid; i < rows * nA; i += THREADS) {
+        const int32_t row = i / nA;
+        target[i] = out[row * out_pitch + (i - row * nA)];
     }
 }
 
@@ -732,6 +852,55 @@ void homogeneous_polynomial_evaluation_vjp(MOPS_HPE_VJP_PARAMS(MOPS_CXX_FIRST, M
         return;
     }
     hipStream_t stream = current_stream();
+    // many rows: by feature (vjp_by_feature_kernel), after the table has been turned round
+    const int32_t out_pitch = nA | 1;
+    const size_t by_feature_lds =
+        (static_cast<size_t>(nA) * FEATURE_ROW_PITCH + static_cast<size_t>(FEATURE_ROWS) * out_pitch) * sizeof(scalar_t);
+    const size_t n_pairs = static_cast<size_t>(n_monomials) * static_cast<size_t>(std::max(order, 0));
+    if (n_rows >= MANY_ROWS && order >= 1 && order <= 6 && n_pairs > 0 && n_pairs < (size_t(1) << 30) &&
+        by_feature_lds <= BY_FEATURE_LDS_BUDGET) {
+        void* workspace = scratch(edges_by_sender_bytes(nA, static_cast<int32_t>(n_pairs)));
+        const EdgesBySender lists =
+            order_edges_by_sender(indices_A.data, static_cast<int32_t>(n_pairs), nA, workspace, stream);
+        const unsigned blocks = static_cast<unsigned>(ceil_div(static_cast<size_t>(n_rows), FEATURE_ROWS));
+#define MOPS_LAUNCH_BY_FEATURE(ORDER)                                                               \
+    {                                                                                              \
+        auto kernel = vjp_by_feature_kernel<scalar_t, ORDER>;                                      \
+        if (by_feature_lds > 64 * 1024) {                                                          \
+            MOPS_HIP_CHECK(hipFuncSetAttribute(                                                    \
+                reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, \
+                static_cast<int>(by_feature_lds)                                                   \
+            ));                                                                                    \
+        }                                                                                          \
+        kernel<<<blocks, FEATURE_WAVES * WAVE, by_feature_lds, stream>>>(                          \
+            grad_A.data, grad_output.data, A.data, C.data, indices_A.data, lists.offsets, lists.edge, \
+            n_rows, nA, out_pitch                                                                  \
+        );                                                                                         \
+    }
+        switch (order) {
+        case 1:
+            MOPS_LAUNCH_BY_FEATURE(1);
+            break;
+        case 2:
+            MOPS_LAUNCH_BY_FEATURE(2);
+            break;
+        case 3:
+            MOPS_LAUNCH_BY_FEATURE(3);
+            break;
+        case 4:
+            MOPS_LAUNCH_BY_FEATURE(4);
+            break;
+        case 5:
+            MOPS_LAUNCH_BY_FEATURE(5);
+            break;
+        default:
+            MOPS_LAUNCH_BY_FEATURE(6);
+            break;
+        }
+#undef MOPS_LAUNCH_BY_FEATURE
+        finish_call(operation);
+        return;
+    }
     // LDS holds R rows of A and WAVE private accumulator rows, whatever R is
     const size_t accumulator_bytes = static_cast<size_t>(nA) * WAVE * sizeof(scalar_t);
     // Rows per workgroup: the fewest for which all workgroups are on the

@@ -92,13 +92,19 @@ __global__ __launch_bounds__(THREADS) void fill_kernel(
 
 // workgroup `node` writes its list, sorted, and its own number next to every
 // entry; workgroup n_nodes fills what is left after the last list
-constexpr int LIST_THREADS = 64;
+// (threads, entries sorted in LDS; longer lists take the slow way through global memory):
+// small workgroups for the short lists of a graph, large ones where lists are long on average
+constexpr int SHORT_LIST_THREADS = 64;
+constexpr int SHORT_LIST_CAPACITY = BUCKET_LDS_CAPACITY;
+constexpr int LONG_LIST_THREADS = 256;
+constexpr int LONG_LIST_CAPACITY = 8192;
 
+template <int LIST_THREADS, int LIST_LDS_CAPACITY>
 __global__ __launch_bounds__(LIST_THREADS) void write_lists_kernel(
     SenderBuckets buckets, int32_t n_nodes, int32_t n_edges, int32_t* __restrict__ sender_of_position,
     int32_t* __restrict__ edge_of_position
 ) {
-    __shared__ int32_t list[BUCKET_LDS_CAPACITY];
+    __shared__ int32_t list[LIST_LDS_CAPACITY];
     const int32_t node = blockIdx.x;
     if (node == n_nodes) {
         for (int32_t at = buckets.offsets[n_nodes] + threadIdx.x; at < n_edges; at += LIST_THREADS) {
@@ -108,7 +114,7 @@ __global__ __launch_bounds__(LIST_THREADS) void write_lists_kernel(
         return;
     }
     const int32_t begin = buckets.offsets[node];
-    const SortedBucket sorted = sorted_bucket(buckets, node, list);
+    const SortedBucket sorted = sorted_bucket(buckets, node, list, LIST_LDS_CAPACITY);
     for (int32_t at = threadIdx.x; at < sorted.count; at += LIST_THREADS) {
         sender_of_position[begin + at] = node;
         edge_of_position[begin + at] = sorted.edges[at];
@@ -128,9 +134,17 @@ EdgesBySender order_edges_by_sender(
     char* base = static_cast<char*>(workspace) + sender_buckets_bytes(n_nodes, n_edges);
     int32_t* sender_of_position = reinterpret_cast<int32_t*>(base);
     int32_t* edge_of_position = reinterpret_cast<int32_t*>(base + align256(static_cast<size_t>(n_edges) * 4));
-    write_lists_kernel<<<static_cast<unsigned>(n_nodes) + 1, LIST_THREADS, 0, stream>>>(
-        buckets, n_nodes, n_edges, sender_of_position, edge_of_position
-    );
+    if (static_cast<size_t>(n_edges) <= static_cast<size_t>(n_nodes) * 256) {
+        write_lists_kernel<SHORT_LIST_THREADS, SHORT_LIST_CAPACITY>
+            <<<static_cast<unsigned>(n_nodes) + 1, SHORT_LIST_THREADS, 0, stream>>>(
+                buckets, n_nodes, n_edges, sender_of_position, edge_of_position
+            );
+    } else {
+        write_lists_kernel<LONG_LIST_THREADS, LONG_LIST_CAPACITY>
+            <<<static_cast<unsigned>(n_nodes) + 1, LONG_LIST_THREADS, 0, stream>>>(
+                buckets, n_nodes, n_edges, sender_of_position, edge_of_position
+            );
+    }
     MOPS_HIP_CHECK(hipGetLastError());
     return EdgesBySender{sender_of_position, edge_of_position, buckets.offsets};
 }

@@ -78,13 +78,16 @@ struct SortedBucket {
 /// the reference's CPU loops). Lists of up to BUCKET_LDS_CAPACITY edges are
 /// sorted in `lds` (a bitonic network); longer ones by counting ranks through
 /// the global spare buffer.
-__device__ inline SortedBucket sorted_bucket(const SenderBuckets& buckets, int32_t node, int32_t* lds) {
+/// `capacity`: entries `lds` has room for (BUCKET_LDS_CAPACITY unless the caller has more).
+__device__ inline SortedBucket sorted_bucket(
+    const SenderBuckets& buckets, int32_t node, int32_t* lds, int32_t capacity = BUCKET_LDS_CAPACITY
+) {
     const int32_t begin = buckets.offsets[node];
     const int32_t count = buckets.offsets[node + 1] - begin;
     const int tid = threadIdx.x;
     const int nthreads = blockDim.x;
 
-    if (count <= BUCKET_LDS_CAPACITY) {
+    if (count <= capacity) {
         int padded = 1;
         while (padded < count) {
             padded <<= 1;
