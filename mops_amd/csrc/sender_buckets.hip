@@ -121,6 +121,123 @@ __global__ __launch_bounds__(LIST_THREADS) void write_lists_kernel(
     }
 }
 
+// Small problems (a table of a few thousand entries over a few hundred values:
+// the monomial table of HPE turned round) in ONE workgroup, without atomics on
+// shared counters and without a sort afterwards: wavefront w looks after a
+// contiguous share of the edges; counts per (wavefront, value) in LDS, a scan
+// over them, and then every edge takes the next free place of its value, edges
+// of one group of 64 with the same value in lane order (ranks from ballots
+// over the bits of the value). The places are handed out in ascending edge
+// order, so every list comes out sorted.
+constexpr int SMALL_WAVES = 16;
+constexpr int SMALL_THREADS = SMALL_WAVES * WAVE;
+constexpr int32_t SMALL_MAX_NODES = 896; // (SMALL_WAVES + 1) counters per value in 64 KB of LDS
+constexpr int32_t SMALL_MAX_EDGES = 16384;
+
+/// LDS: counts[SMALL_WAVES][n_nodes] totals[n_nodes] (ints).
+__global__ __launch_bounds__(SMALL_THREADS) void order_small_kernel(
+    const int32_t* __restrict__ senders, int32_t n_edges, int32_t n_nodes, int32_t value_bits,
+    int32_t* __restrict__ offsets, int32_t* __restrict__ sender_of_position, int32_t* __restrict__ edge_of_position
+) {
+    extern __shared__ __align__(16) unsigned char lds_bytes[];
+    int32_t* counts = reinterpret_cast<int32_t*>(lds_bytes);
+    int32_t* totals = counts + SMALL_WAVES * n_nodes;
+    const int tid = threadIdx.x;
+    const int lane = tid & (WAVE - 1);
+    const int wave = tid >> 6;
+    constexpr int GROUPS = SMALL_MAX_EDGES / SMALL_THREADS;
+    const int32_t share = (n_edges + SMALL_THREADS - 1) / SMALL_THREADS * WAVE;
+    const int32_t my_begin = min(wave * share, n_edges);
+    const int32_t my_end = min(my_begin + share, n_edges);
+
+    int32_t value[GROUPS]; // negative: no such edge, or a value out of range
+#pragma unroll
+    for (int c = 0; c < GROUPS; c++) {
+        const int32_t e = my_begin + c * WAVE + lane;
+        const int32_t loaded = load_or_zero(senders, static_cast<size_t>(e), e < my_end);
+        value[c] = e < my_end && in_bounds(loaded, n_nodes) ? loaded : -1;
+    }
+    for (int32_t i = tid; i < SMALL_WAVES * n_nodes; i += SMALL_THREADS) {
+        counts[i] = 0;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int c = 0; c < GROUPS; c++) {
+        if (value[c] >= 0) {
+            atomicAdd(&counts[wave * n_nodes + value[c]], 1); // integer counts in LDS: no order involved
+        }
+    }
+    __syncthreads();
+    // counts[w][v] := edges of value v in the shares before w; totals[v] := all of them
+    if (tid < n_nodes) {
+        int32_t running = 0;
+        for (int w = 0; w < SMALL_WAVES; w++) {
+            const int32_t here = counts[w * n_nodes + tid];
+            counts[w * n_nodes + tid] = running;
+            running += here;
+        }
+        totals[tid] = running;
+    }
+    __syncthreads();
+    // inclusive scan of totals over the values (at most one per thread)
+    for (int32_t step = 1; step < n_nodes; step <<= 1) {
+        const int32_t mine = tid < n_nodes ? totals[tid] : 0;
+        const int32_t left = tid < n_nodes && tid >= step ? totals[tid - step] : 0;
+        __syncthreads();
+        if (tid < n_nodes) {
+            totals[tid] = mine + left;
+        }
+        __syncthreads();
+    }
+    const int32_t listed = totals[n_nodes - 1];
+    if (tid < n_nodes) {
+        const int32_t before = tid > 0 ? totals[tid - 1] : 0;
+        offsets[tid] = before;
+        if (tid == n_nodes - 1) {
+            offsets[n_nodes] = totals[tid];
+        }
+        for (int w = 0; w < SMALL_WAVES; w++) {
+            counts[w * n_nodes + tid] += before;
+        }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int c = 0; c < GROUPS; c++) {
+        if (my_begin + c * WAVE < my_end) { // uniform
+            const bool valid = value[c] >= 0;
+            // the lanes with my value: agreement on every bit of it
+            unsigned long long match = __ballot(valid);
+            for (int32_t bit = 0; bit < value_bits; bit++) {
+                const bool set = ((value[c] >> bit) & 1) != 0;
+                const unsigned long long with_bit = __ballot(valid && set);
+                match &= set ? with_bit : ~with_bit;
+            }
+            const int32_t rank = __popcll(match & ((1ull << lane) - 1ull));
+            const int32_t same = __popcll(match);
+            int32_t place = -1;
+            if (valid) {
+                place = counts[wave * n_nodes + value[c]] + rank;
+            }
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            if (valid && rank == same - 1) {
+                counts[wave * n_nodes + value[c]] += same; // one lane per value of the group
+            }
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+            if (place >= 0) {
+                sender_of_position[place] = value[c];
+                edge_of_position[place] = my_begin + c * WAVE + lane;
+            }
+        }
+    }
+    for (int32_t at = listed + tid; at < n_edges; at += SMALL_THREADS) {
+        sender_of_position[at] = n_nodes;
+        edge_of_position[at] = 0;
+    }
+}
+
 } // namespace
 
 size_t edges_by_sender_bytes(int32_t n_nodes, int32_t n_edges) {
@@ -130,6 +247,24 @@ size_t edges_by_sender_bytes(int32_t n_nodes, int32_t n_edges) {
 EdgesBySender order_edges_by_sender(
     const int32_t* senders, int32_t n_edges, int32_t n_nodes, void* workspace, hipStream_t stream
 ) {
+    if (n_nodes >= 1 && n_nodes <= SMALL_MAX_NODES && n_edges >= 1 && n_edges <= SMALL_MAX_EDGES) {
+        // same places in the workspace as below
+        char* at = static_cast<char*>(workspace);
+        int32_t* offsets = reinterpret_cast<int32_t*>(at + align256(static_cast<size_t>(n_nodes) * 4));
+        at += sender_buckets_bytes(n_nodes, n_edges);
+        int32_t* sender_of_position = reinterpret_cast<int32_t*>(at);
+        int32_t* edge_of_position = reinterpret_cast<int32_t*>(at + align256(static_cast<size_t>(n_edges) * 4));
+        int32_t value_bits = 0;
+        while ((1 << value_bits) < n_nodes) {
+            value_bits++;
+        }
+        const size_t lds = static_cast<size_t>(SMALL_WAVES + 1) * n_nodes * sizeof(int32_t);
+        order_small_kernel<<<1, SMALL_THREADS, lds, stream>>>(
+            senders, n_edges, n_nodes, value_bits, offsets, sender_of_position, edge_of_position
+        );
+        MOPS_HIP_CHECK(hipGetLastError());
+        return EdgesBySender{sender_of_position, edge_of_position, offsets};
+    }
     const SenderBuckets buckets = build_sender_buckets(senders, n_edges, n_nodes, workspace, stream);
     char* base = static_cast<char*>(workspace) + sender_buckets_bytes(n_nodes, n_edges);
     int32_t* sender_of_position = reinterpret_cast<int32_t*>(base);
