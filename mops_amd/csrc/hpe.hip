@@ -36,7 +36,7 @@ namespace mops::amd {
 namespace {
 
 constexpr size_t LDS_BUDGET = 60 * 1024;
-constexpr int32_t MANY_ROWS = 4096;                     // from here on the vjp goes by feature
+constexpr int32_t MANY_ROWS = 4096;                     // from here on the vjp goes by feature (at 1000 rows: 31.6 us against 27.5)
 constexpr size_t BY_FEATURE_LDS_BUDGET = 140 * 1024;    // its two tiles, of the 160 KB of a compute unit
 
 // ---------------------------------------------------------------------------
@@ -400,11 +400,14 @@ __global__ __launch_bounds__(FEATURE_WAVES* WAVE) void vjp_by_feature_kernel(
     const int32_t* __restrict__ list,       // pairs q = j * ORDER + f, grouped by feature
     int32_t n_rows,
     int32_t nA,
+    int32_t features_per_group, // blockIdx.y takes the features [y, y + 1) * features_per_group
     int32_t out_pitch
 ) {
     extern __shared__ __align__(16) unsigned char lds_bytes[];
     T* a_stage = reinterpret_cast<T*>(lds_bytes);
     T* out = a_stage + static_cast<size_t>(nA) * FEATURE_ROW_PITCH;
+    const int32_t first_feature = blockIdx.y * features_per_group;
+    const int32_t n_features = min(features_per_group, nA - first_feature);
     constexpr int THREADS = FEATURE_WAVES * WAVE;
     constexpr int OTHERS = ORDER - 1;
 
@@ -436,7 +439,8 @@ __global__ __launch_bounds__(FEATURE_WAVES* WAVE) void vjp_by_feature_kernel(
     __syncthreads();
 
     const T* mine = a_stage + lane;
-    for (int32_t feature = wave; feature < nA; feature += FEATURE_WAVES) {
+    for (int32_t local = wave; local < n_features; local += FEATURE_WAVES) {
+        const int32_t feature = first_feature + local;
         const int32_t begin = list_begin[feature];
         const int32_t end = list_begin[feature + 1];
         T sum = T(0);
@@ -474,14 +478,15 @@ __global__ __launch_bounds__(FEATURE_WAVES* WAVE) void vjp_by_feature_kernel(
                 sum += term;
             }
         }
-        out[lane * out_pitch + feature] = upstream * sum;
+        out[lane * out_pitch + local] = upstream * sum;
     }
     __syncthreads();
-    // the 64 rows of grad_A are one contiguous piece of memory
-    T* target = grad_A + static_cast<size_t>(row0) * nA;
-    for (int32_t i = tid; i < rows * nA; i += THREADS) {
-        const int32_t row = i / nA;
-        target[i] = out[row * out_pitch + (i - row * nA)];
+    // row by row, this group's features next to each other (all of them: one contiguous piece)
+    T* target = grad_A + static_cast<size_t>(row0) * nA + first_feature;
+    for (int32_t i = tid; i < rows * n_features; i += THREADS) {
+        const int32_t row = i / n_features;
+        const int32_t local = i - row * n_features;
+        target[static_cast<size_t>(row) * nA + local] = out[row * out_pitch + local];
     }
 }
 
@@ -853,7 +858,15 @@ void homogeneous_polynomial_evaluation_vjp(MOPS_HPE_VJP_PARAMS(MOPS_CXX_FIRST, M
     }
     hipStream_t stream = current_stream();
     // many rows: by feature (vjp_by_feature_kernel), after the table has been turned round
-    const int32_t out_pitch = nA | 1;
+    // workgroup = (64 rows, a group of features): groups of 16 features (one per wavefront)
+    // while that brings the launch to a few hundred workgroups, all features in one otherwise
+    const size_t row_groups = ceil_div(static_cast<size_t>(n_rows), FEATURE_ROWS);
+    const size_t wanted_groups = std::max<size_t>(1, ceil_div(512, row_groups));
+    const size_t feature_groups = std::min(wanted_groups, ceil_div(static_cast<size_t>(nA), FEATURE_WAVES));
+    const int32_t features_per_group = static_cast<int32_t>(
+        ceil_div(ceil_div(static_cast<size_t>(nA), feature_groups), FEATURE_WAVES) * FEATURE_WAVES
+    );
+    const int32_t out_pitch = features_per_group | 1;
     const size_t by_feature_lds =
         (static_cast<size_t>(nA) * FEATURE_ROW_PITCH + static_cast<size_t>(FEATURE_ROWS) * out_pitch) * sizeof(scalar_t);
     const size_t n_pairs = static_cast<size_t>(n_monomials) * static_cast<size_t>(std::max(order, 0));
@@ -862,7 +875,10 @@ void homogeneous_polynomial_evaluation_vjp(MOPS_HPE_VJP_PARAMS(MOPS_CXX_FIRST, M
         void* workspace = scratch(edges_by_sender_bytes(nA, static_cast<int32_t>(n_pairs)));
         const EdgesBySender lists =
             order_edges_by_sender(indices_A.data, static_cast<int32_t>(n_pairs), nA, workspace, stream);
-        const unsigned blocks = static_cast<unsigned>(ceil_div(static_cast<size_t>(n_rows), FEATURE_ROWS));
+        const dim3 blocks(
+            static_cast<unsigned>(row_groups),
+            static_cast<unsigned>(ceil_div(static_cast<size_t>(nA), static_cast<size_t>(features_per_group)))
+        );
 #define MOPS_LAUNCH_BY_FEATURE(ORDER)                                                               \
     {                                                                                              \
         auto kernel = vjp_by_feature_kernel<scalar_t, ORDER>;                                      \
@@ -874,7 +890,7 @@ void homogeneous_polynomial_evaluation_vjp(MOPS_HPE_VJP_PARAMS(MOPS_CXX_FIRST, M
         }                                                                                          \
         kernel<<<blocks, FEATURE_WAVES * WAVE, by_feature_lds, stream>>>(                          \
             grad_A.data, grad_output.data, A.data, C.data, indices_A.data, lists.offsets, lists.edge, \
-            n_rows, nA, out_pitch                                                                  \
+            n_rows, nA, features_per_group, out_pitch                                              \
         );                                                                                         \
     }
         switch (order) {
