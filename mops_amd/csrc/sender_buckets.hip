@@ -121,7 +121,7 @@ __global__ __launch_bounds__(LIST_THREADS) void write_lists_kernel(
     }
 }
 
-// Small problems (a table of a few thousand entries over a few hundred values:
+// Small problems (a table of some thousands of entries over a few hundred values:
 // the monomial table of HPE turned round) in ONE workgroup, without atomics on
 // shared counters and without a sort afterwards: wavefront w looks after a
 // contiguous share of the edges; counts per (wavefront, value) in LDS, a scan
@@ -132,7 +132,7 @@ __global__ __launch_bounds__(LIST_THREADS) void write_lists_kernel(
 constexpr int SMALL_WAVES = 16;
 constexpr int SMALL_THREADS = SMALL_WAVES * WAVE;
 constexpr int32_t SMALL_MAX_NODES = 896; // (SMALL_WAVES + 1) counters per value in 64 KB of LDS
-constexpr int32_t SMALL_MAX_EDGES = 16384;
+constexpr int32_t SMALL_MAX_EDGES = 131072;
 
 /// LDS: counts[SMALL_WAVES][n_nodes] totals[n_nodes] (ints).
 __global__ __launch_bounds__(SMALL_THREADS) void order_small_kernel(
@@ -145,26 +145,31 @@ __global__ __launch_bounds__(SMALL_THREADS) void order_small_kernel(
     const int tid = threadIdx.x;
     const int lane = tid & (WAVE - 1);
     const int wave = tid >> 6;
-    constexpr int GROUPS = SMALL_MAX_EDGES / SMALL_THREADS;
     const int32_t share = (n_edges + SMALL_THREADS - 1) / SMALL_THREADS * WAVE;
     const int32_t my_begin = min(wave * share, n_edges);
     const int32_t my_end = min(my_begin + share, n_edges);
-
-    int32_t value[GROUPS]; // negative: no such edge, or a value out of range
-#pragma unroll
-    for (int c = 0; c < GROUPS; c++) {
-        const int32_t e = my_begin + c * WAVE + lane;
+    // the value of edge e for this lane: negative if there is no such edge or the value is out of range
+    auto value_of = [&](int32_t e) {
         const int32_t loaded = load_or_zero(senders, static_cast<size_t>(e), e < my_end);
-        value[c] = e < my_end && in_bounds(loaded, n_nodes) ? loaded : -1;
-    }
+        return e < my_end && in_bounds(loaded, n_nodes) ? loaded : -1;
+    };
+
     for (int32_t i = tid; i < SMALL_WAVES * n_nodes; i += SMALL_THREADS) {
         counts[i] = 0;
     }
     __syncthreads();
+    constexpr int AHEAD = 8; // loads in flight
+    for (int32_t e0 = my_begin; e0 < my_end; e0 += AHEAD * WAVE) {
+        int32_t value[AHEAD];
 #pragma unroll
-    for (int c = 0; c < GROUPS; c++) {
-        if (value[c] >= 0) {
-            atomicAdd(&counts[wave * n_nodes + value[c]], 1); // integer counts in LDS: no order involved
+        for (int c = 0; c < AHEAD; c++) {
+            value[c] = value_of(e0 + c * WAVE + lane);
+        }
+#pragma unroll
+        for (int c = 0; c < AHEAD; c++) {
+            if (value[c] >= 0) {
+                atomicAdd(&counts[wave * n_nodes + value[c]], 1); // integer counts in LDS: no order involved
+            }
         }
     }
     __syncthreads();
@@ -201,34 +206,41 @@ __global__ __launch_bounds__(SMALL_THREADS) void order_small_kernel(
         }
     }
     __syncthreads();
+    for (int32_t e0 = my_begin; e0 < my_end; e0 += AHEAD * WAVE) {
+        int32_t value[AHEAD];
 #pragma unroll
-    for (int c = 0; c < GROUPS; c++) {
-        if (my_begin + c * WAVE < my_end) { // uniform
-            const bool valid = value[c] >= 0;
-            // the lanes with my value: agreement on every bit of it
-            unsigned long long match = __ballot(valid);
-            for (int32_t bit = 0; bit < value_bits; bit++) {
-                const bool set = ((value[c] >> bit) & 1) != 0;
-                const unsigned long long with_bit = __ballot(valid && set);
-                match &= set ? with_bit : ~with_bit;
-            }
-            const int32_t rank = __popcll(match & ((1ull << lane) - 1ull));
-            const int32_t same = __popcll(match);
-            int32_t place = -1;
-            if (valid) {
-                place = counts[wave * n_nodes + value[c]] + rank;
-            }
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-            __builtin_amdgcn_wave_barrier();
-            if (valid && rank == same - 1) {
-                counts[wave * n_nodes + value[c]] += same; // one lane per value of the group
-            }
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-            __builtin_amdgcn_wave_barrier();
-            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-            if (place >= 0) {
-                sender_of_position[place] = value[c];
-                edge_of_position[place] = my_begin + c * WAVE + lane;
+        for (int c = 0; c < AHEAD; c++) {
+            value[c] = value_of(e0 + c * WAVE + lane);
+        }
+#pragma unroll
+        for (int c = 0; c < AHEAD; c++) {
+            if (e0 + c * WAVE < my_end) { // uniform
+                const bool valid = value[c] >= 0;
+                // the lanes with my value: agreement on every bit of it
+                unsigned long long match = __ballot(valid);
+                for (int32_t bit = 0; bit < value_bits; bit++) {
+                    const bool set = ((value[c] >> bit) & 1) != 0;
+                    const unsigned long long with_bit = __ballot(valid && set);
+                    match &= set ? with_bit : ~with_bit;
+                }
+                const int32_t rank = __popcll(match & ((1ull << lane) - 1ull));
+                const int32_t same = __popcll(match);
+                int32_t place = -1;
+                if (valid) {
+                    place = counts[wave * n_nodes + value[c]] + rank;
+                }
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                __builtin_amdgcn_wave_barrier();
+                if (valid && rank == same - 1) {
+                    counts[wave * n_nodes + value[c]] += same; // one lane per value of the group
+                }
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                __builtin_amdgcn_wave_barrier();
+                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+                if (place >= 0) {
+                    sender_of_position[place] = value[c];
+                    edge_of_position[place] = e0 + c * WAVE + lane;
+                }
             }
         }
     }

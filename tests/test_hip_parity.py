@@ -89,6 +89,7 @@ LARGE = {
         "many_monomials": lambda s, d: support.hpe_case(s, d, I=500, nA=60, J=40000, K=5),
         "many_rows_long_table": lambda s, d: support.hpe_case(s, d, I=5000, nA=30, J=6000, K=3),
         "many_rows_order1": lambda s, d: support.hpe_case(s, d, I=4100, nA=7, J=50, K=1),
+        "many_rows_very_long_table": lambda s, d: support.hpe_case(s, d, I=4096, nA=20, J=45000, K=3),
     },
     "sap": {
         "many_rows": lambda s, d: support.sap_case(s, d, I=1000003, nA=13, nB=7, K=900, nO=20),
