@@ -462,20 +462,38 @@ __global__ __launch_bounds__(FEATURE_WAVES* WAVE) void vjp_by_feature_kernel(
             }
             int32_t words[sizeof(T) / 4];
             __builtin_memcpy(words, &coefficient, sizeof(T));
-#pragma unroll 4
-            for (int32_t u = 0; u < n; u++) {
-                int32_t uniform[sizeof(T) / 4];
+            // BATCH entries at a time: first every LDS read, then the products (a read that
+            // is waited for before the next one is asked for costs its whole latency)
+            constexpr int BATCH = 8;
+            for (int32_t u0 = 0; u0 < n; u0 += BATCH) {
+                T term[BATCH];
+                T value[BATCH][OTHERS > 0 ? OTHERS : 1];
 #pragma unroll
-                for (int w = 0; w < static_cast<int>(sizeof(T) / 4); w++) {
-                    uniform[w] = __builtin_amdgcn_readlane(words[w], u);
-                }
-                T term;
-                __builtin_memcpy(&term, uniform, sizeof(T));
+                for (int b = 0; b < BATCH; b++) {
+                    // entries beyond n: lanes beyond n hold coefficient zero and a place that exists
+                    const int32_t u = min(u0 + b, WAVE - 1);
+                    int32_t uniform[sizeof(T) / 4];
 #pragma unroll
-                for (int k = 0; k < OTHERS; k++) {
-                    term *= mine[__builtin_amdgcn_readlane(other[k], u)];
+                    for (int w = 0; w < static_cast<int>(sizeof(T) / 4); w++) {
+                        uniform[w] = __builtin_amdgcn_readlane(words[w], u);
+                    }
+                    __builtin_memcpy(&term[b], uniform, sizeof(T));
+                    if (u0 + b >= WAVE) {
+                        term[b] = T(0);
+                    }
+#pragma unroll
+                    for (int k = 0; k < OTHERS; k++) {
+                        value[b][k] = mine[__builtin_amdgcn_readlane(other[k], u)];
+                    }
                 }
-                sum += term;
+#pragma unroll
+                for (int b = 0; b < BATCH; b++) {
+#pragma unroll
+                    for (int k = 0; k < OTHERS; k++) {
+                        term[b] *= value[b][k];
+                    }
+                    sum += term[b];
+                }
             }
         }
         out[lane * out_pitch + local] = upstream * sum;
