@@ -385,11 +385,14 @@ __global__ __launch_bounds__(WAVE) void vjp_ordered_kernel(
 // lanes through readlane. One fixed order (ascending q), no atomics.
 // LDS: a[nA][ROW_PITCH] out[64][out_pitch]
 // ---------------------------------------------------------------------------
-constexpr int FEATURE_ROWS = WAVE;          // rows per workgroup
-constexpr int FEATURE_ROW_PITCH = WAVE + 1; // distance between features in the tile of A
 constexpr int FEATURE_WAVES = 16;
+/// Rows per workgroup when a lane has RPL rows (lane, lane + 64, ...: the table entry a
+/// wavefront is at then serves RPL rows per lane for the same readlanes and address)
+__host__ __device__ constexpr int feature_rows(int rpl) { return WAVE * rpl; }
+/// Distance between features in the tile of A
+__host__ __device__ constexpr int feature_row_pitch(int rpl) { return WAVE * rpl + 1; }
 
-template <typename T, int ORDER>
+template <typename T, int ORDER, int RPL>
 __global__ __launch_bounds__(FEATURE_WAVES* WAVE) void vjp_by_feature_kernel(
     T* __restrict__ grad_A,
     const T* __restrict__ grad_output,
@@ -405,10 +408,12 @@ __global__ __launch_bounds__(FEATURE_WAVES* WAVE) void vjp_by_feature_kernel(
 ) {
     extern __shared__ __align__(16) unsigned char lds_bytes[];
     T* a_stage = reinterpret_cast<T*>(lds_bytes);
-    T* out = a_stage + static_cast<size_t>(nA) * FEATURE_ROW_PITCH;
+    T* out = a_stage + static_cast<size_t>(nA) * feature_row_pitch(RPL);
     const int32_t first_feature = blockIdx.y * features_per_group;
     const int32_t n_features = min(features_per_group, nA - first_feature);
     constexpr int THREADS = FEATURE_WAVES * WAVE;
+    constexpr int FEATURE_ROWS = feature_rows(RPL);
+    constexpr int FEATURE_ROW_PITCH = feature_row_pitch(RPL);
     constexpr int OTHERS = ORDER - 1;
 
     const int tid = threadIdx.x;
@@ -435,7 +440,11 @@ __global__ __launch_bounds__(FEATURE_WAVES* WAVE) void vjp_by_feature_kernel(
             }
         }
     }
-    const T upstream = load_or_zero(grad_output, static_cast<size_t>(row0 + lane), lane < rows);
+    T upstream[RPL];
+#pragma unroll
+    for (int r = 0; r < RPL; r++) {
+        upstream[r] = load_or_zero(grad_output, static_cast<size_t>(row0 + lane + r * WAVE), lane + r * WAVE < rows);
+    }
     __syncthreads();
 
     const T* mine = a_stage + lane;
@@ -443,7 +452,11 @@ __global__ __launch_bounds__(FEATURE_WAVES* WAVE) void vjp_by_feature_kernel(
         const int32_t feature = first_feature + local;
         const int32_t begin = list_begin[feature];
         const int32_t end = list_begin[feature + 1];
-        T sum = T(0);
+        T sum[RPL];
+#pragma unroll
+        for (int r = 0; r < RPL; r++) {
+            sum[r] = T(0);
+        }
         for (int32_t p0 = begin; p0 < end; p0 += WAVE) {
             const int32_t n = min(WAVE, end - p0);
             // my entry of the batch: coefficient (zero: no entry, or a factor out of range) and
@@ -467,7 +480,7 @@ __global__ __launch_bounds__(FEATURE_WAVES* WAVE) void vjp_by_feature_kernel(
             constexpr int BATCH = 8;
             for (int32_t u0 = 0; u0 < n; u0 += BATCH) {
                 T term[BATCH];
-                T value[BATCH][OTHERS > 0 ? OTHERS : 1];
+                T value[BATCH][OTHERS > 0 ? OTHERS : 1][RPL];
 #pragma unroll
                 for (int b = 0; b < BATCH; b++) {
                     // entries beyond n: lanes beyond n hold coefficient zero and a place that exists
@@ -483,20 +496,31 @@ __global__ __launch_bounds__(FEATURE_WAVES* WAVE) void vjp_by_feature_kernel(
                     }
 #pragma unroll
                     for (int k = 0; k < OTHERS; k++) {
-                        value[b][k] = mine[__builtin_amdgcn_readlane(other[k], u)];
+                        const T* at = mine + __builtin_amdgcn_readlane(other[k], u);
+#pragma unroll
+                        for (int r = 0; r < RPL; r++) {
+                            value[b][k][r] = at[r * WAVE];
+                        }
                     }
                 }
 #pragma unroll
                 for (int b = 0; b < BATCH; b++) {
 #pragma unroll
-                    for (int k = 0; k < OTHERS; k++) {
-                        term[b] *= value[b][k];
+                    for (int r = 0; r < RPL; r++) {
+                        T product = term[b];
+#pragma unroll
+                        for (int k = 0; k < OTHERS; k++) {
+                            product *= value[b][k][r];
+                        }
+                        sum[r] += product;
                     }
-                    sum += term[b];
                 }
             }
         }
-        out[lane * out_pitch + local] = upstream * sum;
+#pragma unroll
+        for (int r = 0; r < RPL; r++) {
+            out[(lane + r * WAVE) * out_pitch + local] = upstream[r] * sum[r];
+        }
     }
     __syncthreads();
     // row by row, this group's features next to each other (all of them: one contiguous piece)
@@ -878,15 +902,20 @@ void homogeneous_polynomial_evaluation_vjp(MOPS_HPE_VJP_PARAMS(MOPS_CXX_FIRST, M
     // many rows: by feature (vjp_by_feature_kernel), after the table has been turned round
     // workgroup = (64 rows, a group of features): groups of 16 features (one per wavefront)
     // while that brings the launch to a few hundred workgroups, all features in one otherwise
-    const size_t row_groups = ceil_div(static_cast<size_t>(n_rows), FEATURE_ROWS);
+    auto by_feature_bytes = [&](int rpl, int32_t pitch) {
+        return (static_cast<size_t>(nA) * feature_row_pitch(rpl) + static_cast<size_t>(feature_rows(rpl)) * pitch) *
+               sizeof(scalar_t);
+    };
+    // two rows per lane where the tiles of 128 rows fit
+    const int rows_per_lane = by_feature_bytes(2, (FEATURE_WAVES * 4) | 1) <= BY_FEATURE_LDS_BUDGET ? 2 : 1;
+    const size_t row_groups = ceil_div(static_cast<size_t>(n_rows), static_cast<size_t>(feature_rows(rows_per_lane)));
     const size_t wanted_groups = std::max<size_t>(1, ceil_div(512, row_groups));
     const size_t feature_groups = std::min(wanted_groups, ceil_div(static_cast<size_t>(nA), FEATURE_WAVES));
     const int32_t features_per_group = static_cast<int32_t>(
         ceil_div(ceil_div(static_cast<size_t>(nA), feature_groups), FEATURE_WAVES) * FEATURE_WAVES
     );
     const int32_t out_pitch = features_per_group | 1;
-    const size_t by_feature_lds =
-        (static_cast<size_t>(nA) * FEATURE_ROW_PITCH + static_cast<size_t>(FEATURE_ROWS) * out_pitch) * sizeof(scalar_t);
+    const size_t by_feature_lds = by_feature_bytes(rows_per_lane, out_pitch);
     const size_t n_pairs = static_cast<size_t>(n_monomials) * static_cast<size_t>(std::max(order, 0));
     if (n_rows >= MANY_ROWS && order >= 1 && order <= 6 && n_pairs > 0 && n_pairs < (size_t(1) << 30) &&
         by_feature_lds <= BY_FEATURE_LDS_BUDGET) {
@@ -899,7 +928,8 @@ void homogeneous_polynomial_evaluation_vjp(MOPS_HPE_VJP_PARAMS(MOPS_CXX_FIRST, M
         );
 #define MOPS_LAUNCH_BY_FEATURE(ORDER)                                                               \
     {                                                                                              \
-        auto kernel = vjp_by_feature_kernel<scalar_t, ORDER>;                                      \
+        auto kernel = rows_per_lane == 2 ? vjp_by_feature_kernel<scalar_t, ORDER, 2>               \
+                                         : vjp_by_feature_kernel<scalar_t, ORDER, 1>;              \
         if (by_feature_lds > 64 * 1024) {                                                          \
             MOPS_HIP_CHECK(hipFuncSetAttribute(                                                    \
                 reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, \
