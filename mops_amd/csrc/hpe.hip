@@ -37,6 +37,7 @@ namespace {
 
 constexpr size_t LDS_BUDGET = 60 * 1024;
 constexpr int32_t MANY_ROWS = 4096;                     // from here on the vjp goes by feature (at 1000 rows: 31.6 us against 27.5)
+constexpr int32_t FORWARD_MANY_ROWS = 200 * 64;            // from here on the forward pass has a lane per row
 constexpr size_t BY_FEATURE_LDS_BUDGET = 140 * 1024;    // its two tiles, of the 160 KB of a compute unit
 
 // ---------------------------------------------------------------------------
@@ -533,6 +534,135 @@ __global__ __launch_bounds__(FEATURE_WAVES* WAVE) void vjp_by_feature_kernel(
 }
 
 // ---------------------------------------------------------------------------
+// forward for MANY rows, the same way: a lane is RPL rows, all lanes of a
+// wavefront are at the same monomial. The wavefronts of a workgroup share the
+// rows and take contiguous shares of the monomials, 64 at a time (lane u
+// loads monomial u of the batch, readlane hands it out); their partial sums
+// meet in LDS in wave order.
+// LDS: a[nA][pitch] partial[FEATURE_WAVES][rows]
+// ---------------------------------------------------------------------------
+template <typename T, int ORDER, int RPL>
+__global__ __launch_bounds__(FEATURE_WAVES* WAVE) void forward_rows_kernel(
+    T* __restrict__ output,
+    const T* __restrict__ A,
+    const T* __restrict__ C,
+    const int32_t* __restrict__ P,
+    int32_t n_rows,
+    int32_t nA,
+    int32_t n_monomials
+) {
+    extern __shared__ __align__(16) unsigned char lds_bytes[];
+    constexpr int THREADS = FEATURE_WAVES * WAVE;
+    constexpr int ROWS = feature_rows(RPL);
+    constexpr int PITCH = feature_row_pitch(RPL);
+    T* a_stage = reinterpret_cast<T*>(lds_bytes);
+    T* partial = a_stage + static_cast<size_t>(nA) * PITCH;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & (WAVE - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int32_t row0 = blockIdx.x * ROWS;
+    const int32_t rows = min(ROWS, n_rows - row0);
+
+    const T* a_src = A + static_cast<size_t>(row0) * nA;
+    constexpr int STAGE_LOADS = 4;
+    for (int32_t i0 = tid; i0 < ROWS * nA; i0 += STAGE_LOADS * THREADS) {
+        T value[STAGE_LOADS];
+#pragma unroll
+        for (int u = 0; u < STAGE_LOADS; u++) {
+            const int32_t i = i0 + u * THREADS;
+            value[u] = load_or_zero(a_src, static_cast<size_t>(i), i < rows * nA); // rows beyond the end: zeros
+        }
+#pragma unroll
+        for (int u = 0; u < STAGE_LOADS; u++) {
+            const int32_t i = i0 + u * THREADS;
+            if (i < ROWS * nA) {
+                const int32_t row = i / nA;
+                a_stage[(i - row * nA) * PITCH + row] = value[u];
+            }
+        }
+    }
+    __syncthreads();
+
+    const int32_t per_wave = (n_monomials + FEATURE_WAVES - 1) / FEATURE_WAVES;
+    const int32_t begin = min(wave * per_wave, n_monomials);
+    const int32_t end = min(begin + per_wave, n_monomials);
+    const T* mine = a_stage + lane;
+    T sum[RPL];
+#pragma unroll
+    for (int r = 0; r < RPL; r++) {
+        sum[r] = T(0);
+    }
+    for (int32_t j0 = begin; j0 < end; j0 += WAVE) {
+        const int32_t n = min(WAVE, end - j0);
+        // my monomial of the batch: coefficient (zero: none, or a factor out of range) and where
+        // its factors' values are in the tile
+        const int32_t j = lane < n ? j0 + lane : 0;
+        T coefficient = lane < n ? C[j] : T(0);
+        int32_t place[ORDER];
+#pragma unroll
+        for (int k = 0; k < ORDER; k++) {
+            const int32_t factor = P[static_cast<size_t>(j) * ORDER + k];
+            const bool valid = in_bounds(factor, nA);
+            place[k] = (valid ? factor : 0) * PITCH;
+            coefficient = valid ? coefficient : T(0);
+        }
+        int32_t words[sizeof(T) / 4];
+        __builtin_memcpy(words, &coefficient, sizeof(T));
+        constexpr int BATCH = 8;
+        for (int32_t u0 = 0; u0 < n; u0 += BATCH) {
+            T term[BATCH];
+            T value[BATCH][ORDER][RPL];
+#pragma unroll
+            for (int b = 0; b < BATCH; b++) {
+                const int32_t u = min(u0 + b, WAVE - 1);
+                int32_t uniform[sizeof(T) / 4];
+#pragma unroll
+                for (int w = 0; w < static_cast<int>(sizeof(T) / 4); w++) {
+                    uniform[w] = __builtin_amdgcn_readlane(words[w], u);
+                }
+                __builtin_memcpy(&term[b], uniform, sizeof(T));
+                if (u0 + b >= WAVE) {
+                    term[b] = T(0);
+                }
+#pragma unroll
+                for (int k = 0; k < ORDER; k++) {
+                    const T* at = mine + __builtin_amdgcn_readlane(place[k], u);
+#pragma unroll
+                    for (int r = 0; r < RPL; r++) {
+                        value[b][k][r] = at[r * WAVE];
+                    }
+                }
+            }
+#pragma unroll
+            for (int b = 0; b < BATCH; b++) {
+#pragma unroll
+                for (int r = 0; r < RPL; r++) {
+                    T product = term[b];
+#pragma unroll
+                    for (int k = 0; k < ORDER; k++) {
+                        product *= value[b][k][r];
+                    }
+                    sum[r] += product;
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < RPL; r++) {
+        partial[wave * ROWS + lane + r * WAVE] = sum[r];
+    }
+    __syncthreads();
+    if (tid < rows) {
+        T total = T(0);
+        for (int w = 0; w < FEATURE_WAVES; w++) {
+            total += partial[w * ROWS + tid];
+        }
+        output[row0 + tid] = total;
+    }
+}
+
+// ---------------------------------------------------------------------------
 // Fallbacks for feature counts whose tiles do not fit in LDS: one thread per
 // batch row, everything in global memory.
 // ---------------------------------------------------------------------------
@@ -833,6 +963,58 @@ void homogeneous_polynomial_evaluation(MOPS_HPE_PARAMS(MOPS_CXX_FIRST, MOPS_CXX_
     }
     hipStream_t stream = current_stream();
     constexpr int THREADS = 256;
+    // many rows: a lane per row (forward_rows_kernel), two where the tile of 128 rows fits
+    auto rows_bytes = [&](int rpl) {
+        return (static_cast<size_t>(nA) * feature_row_pitch(rpl) + static_cast<size_t>(FEATURE_WAVES) * feature_rows(rpl)) *
+               sizeof(scalar_t);
+    };
+    // (a workgroup per 64 or 128 rows: fewer workgroups than about one per compute unit leave the
+    // kernel below ahead, 8192 rows: 24 us against 35)
+    if (n_rows >= FORWARD_MANY_ROWS && order >= 1 && order <= 6 && n_monomials > 0 &&
+        rows_bytes(1) <= BY_FEATURE_LDS_BUDGET) {
+        // (two rows per lane also where that halves the workgroups: 20 000 rows, 51 us against 65)
+        const int rows_per_lane = rows_bytes(2) <= BY_FEATURE_LDS_BUDGET ? 2 : 1;
+        const size_t lds = rows_bytes(rows_per_lane);
+        const unsigned blocks =
+            static_cast<unsigned>(ceil_div(static_cast<size_t>(n_rows), static_cast<size_t>(feature_rows(rows_per_lane))));
+#define MOPS_LAUNCH_ROWS(ORDER)                                                                     \
+    {                                                                                              \
+        auto kernel = rows_per_lane == 2 ? forward_rows_kernel<scalar_t, ORDER, 2>                 \
+                                         : forward_rows_kernel<scalar_t, ORDER, 1>;                \
+        if (lds > 64 * 1024) {                                                                     \
+            MOPS_HIP_CHECK(hipFuncSetAttribute(                                                    \
+                reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, \
+                static_cast<int>(lds)                                                              \
+            ));                                                                                    \
+        }                                                                                          \
+        kernel<<<blocks, FEATURE_WAVES * WAVE, lds, stream>>>(                                     \
+            output.data, A.data, C.data, indices_A.data, n_rows, nA, n_monomials                   \
+        );                                                                                         \
+    }
+        switch (order) {
+        case 1:
+            MOPS_LAUNCH_ROWS(1);
+            break;
+        case 2:
+            MOPS_LAUNCH_ROWS(2);
+            break;
+        case 3:
+            MOPS_LAUNCH_ROWS(3);
+            break;
+        case 4:
+            MOPS_LAUNCH_ROWS(4);
+            break;
+        case 5:
+            MOPS_LAUNCH_ROWS(5);
+            break;
+        default:
+            MOPS_LAUNCH_ROWS(6);
+            break;
+        }
+#undef MOPS_LAUNCH_ROWS
+        finish_call(operation);
+        return;
+    }
     // per row: its A values plus one partial sum per group (G <= THREADS)
     int R = pick_rows(n_rows, (static_cast<size_t>(nA) + THREADS) * sizeof(scalar_t));
     if (R > 0) {
