@@ -76,6 +76,8 @@ def build_configs():
         # beyond the BASELINE shapes: feature counts that fill whole 16-wide matrix tiles
         ("wide", "opsa", np.float32, support.opsa_case(5, np.float32, K=32, L=64)),
         ("wide", "opsaw", np.float32, support.opsaw_case(6, np.float32, K=32, L=64)),
+        # many rows: HPE with a lane per row (forward) and by feature (vjp)
+        ("many_rows", "hpe", np.float64, support.hpe_case(10, np.float64, I=20000, nA=50, J=4000, K=3)),
         # 128 feature channels: the kernels take them in blocks of 64 columns
         ("wide128", "opsa", np.float32, support.opsa_case(7, np.float32, K=16, L=128)),
         ("wide128", "opsaw", np.float32, support.opsaw_case(8, np.float32, K=16, L=128)),
@@ -301,7 +303,7 @@ def main():
 
     if args.profile:
         for config, op_name, _, op_case in configs:
-            if not config.startswith("wide") and args.profile in (op_name, "all"):
+            if config.startswith("c") and args.profile in (op_name, "all"):
                 w = DeviceWorkload(op_name, op_case, device)
                 for _ in range(50):
                     w.step()
