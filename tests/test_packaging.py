@@ -100,6 +100,6 @@ def test_setup_ships_library_headers_and_cmake_files(tmp_path):
     )
     assert built.returncode == 0, built.stdout + built.stderr
     package = tmp_path / "mops_amd"
-    for relative in ("lib/libmops.so", "include/mops.h", "include/mops/opsa.hpp", "cmake/mops/mops-config.cmake",
+    for relative in ("lib/libmops.so", "lib/libmops_amd_torch.so", "include/mops.h", "include/mops/opsa.hpp", "cmake/mops/mops-config.cmake",
                      "cmake/mops/mops-config-version.cmake", "torch.py"):
         assert (package / relative).exists(), relative

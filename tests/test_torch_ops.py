@@ -1,4 +1,8 @@
 """torch.ops.mops.*: schemas (as mops-torch/src/register.cpp of the reference), values, autograd."""
+import os
+import subprocess
+import sys
+
 import numpy as np
 import pytest
 import torch
@@ -34,6 +38,29 @@ def arguments(op, case):
 def test_schemas_match_the_reference():
     for name, schema in SCHEMAS.items():
         assert str(getattr(torch.ops.mops, name).default._schema) == schema
+
+
+def test_cpp_operators_are_used_when_built():
+    """mops_amd/lib/libmops_amd_torch.so (mops_amd/csrc/torch_ops.cpp), if there, is what registers the operators."""
+    built = os.path.exists(mops_amd.torch.CPP_OPERATORS_PATH)
+    forced = os.environ.get("MOPS_AMD_TORCH_PYTHON_OPS", "0") not in ("", "0")
+    assert mops_amd.torch.OPERATORS_FROM == ("c++" if built and not forced else "python")
+
+
+@pytest.mark.gpu
+@pytest.mark.skipif(mops_amd.torch.OPERATORS_FROM != "c++", reason="this process already runs the Python operators")
+def test_python_operators_in_a_process_of_their_own():
+    """The operators registered from Python (the fallback without the C++ library): the same tests, in a
+    process that is told to use them."""
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    environment = dict(os.environ, MOPS_AMD_TORCH_PYTHON_OPS="1")
+    done = subprocess.run(
+        [sys.executable, "-m", "pytest", os.path.join(root, "tests", "test_torch_ops.py"), "-m", "gpu", "-q", "-x",
+         "-p", "no:cacheprovider"],
+        cwd=root, env=environment, capture_output=True, text=True,
+    )
+    assert done.returncode == 0, done.stdout[-3000:] + done.stderr[-2000:]
+    assert " passed" in done.stdout
 
 
 def test_host_tensors_are_refused():
