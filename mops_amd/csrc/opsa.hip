@@ -667,8 +667,17 @@ __global__ __launch_bounds__(256) void gather_weights_kernel(
 // 16-byte load per lane replaces VL loads that each touch 16 cache lines,
 // which is what these kernels otherwise spend their time on (address
 // processing, not bandwidth).
-template <typename T, int KT, int NT, bool WEIGHTED, bool VECTORS, bool BLOCKS>
-__global__ __launch_bounds__(WAVE) void edge_rows_vjp_kernel(
+//
+// LISTS: workgroups are four wavefronts (four groups of 16 edges, independent
+// of each other), and the first `list_blocks` workgroups do something else:
+// they list the edges of every sender in its slots (sender_buckets.hpp), which
+// the sum of the per-edge rows of grad_W needs afterwards. That pass over the
+// sender index has no launch of its own then and no time of its own: it runs
+// beside the wavefronts that wait for their rows.
+constexpr int LISTING_WAVES = 2;
+
+template <typename T, int KT, int NT, bool WEIGHTED, bool VECTORS, bool BLOCKS, bool LISTS>
+__global__ __launch_bounds__((LISTS ? LISTING_WAVES : 1) * WAVE) void edge_rows_vjp_kernel(
     T* __restrict__ grad_A,
     T* __restrict__ grad_B,
     T* __restrict__ edge_W,
@@ -681,15 +690,34 @@ __global__ __launch_bounds__(WAVE) void edge_rows_vjp_kernel(
     int32_t n_edges,
     int32_t n_output,
     int32_t K,
-    int32_t L
+    int32_t L,
+    int32_t* __restrict__ slots,
+    int32_t* __restrict__ slot_counts,
+    int32_t list_blocks,
+    bool aligned_senders
 ) {
     using M = Mfma<T>;
     constexpr int K_STEPS = 4 * KT;
     constexpr int L_STEPS = 4 * NT;
-    const int lane = threadIdx.x;
+    constexpr int WAVES = LISTS ? LISTING_WAVES : 1;
+    if constexpr (LISTS) {
+        if (static_cast<int32_t>(blockIdx.x) < list_blocks) {
+            __shared__ SlotLists lists;
+            list_in_slots_block<WAVES * WAVE>(
+                lists, slots, slot_counts, indices_W, n_edges, n_output, aligned_senders, blockIdx.x
+            );
+            return;
+        }
+    }
+    const int lane = threadIdx.x & (WAVE - 1);
+    const int wave = LISTS ? threadIdx.x >> 6 : 0;
     const int i = lane & 15;
     const int q = lane >> 4;
-    const int32_t first_edge = blockIdx.x * 16;
+    const int32_t first_edge =
+        (LISTS ? (static_cast<int32_t>(blockIdx.x) - list_blocks) * WAVES + wave : static_cast<int32_t>(blockIdx.x)) * 16;
+    if (LISTS && first_edge >= n_edges) {
+        return; // (the wavefronts of a workgroup never wait for each other)
+    }
     const int32_t n = min(16, n_edges - first_edge);
     const int32_t my_edge = i < n ? first_edge + i : -1;
     const bool want_A = grad_A != nullptr;
@@ -751,7 +779,8 @@ __global__ __launch_bounds__(WAVE) void edge_rows_vjp_kernel(
     // The 16 rows of A are one contiguous piece of memory: read as such (a few
     // cache lines per load instead of 16) and handed to the operand layout
     // through LDS.
-    __shared__ T a_tile[16 * 16 * KT];
+    __shared__ T a_tiles[WAVES][16 * 16 * KT];
+    T* a_tile = a_tiles[wave];
     {
         constexpr int LOADS = (16 * 16 * KT + WAVE - 1) / WAVE;
         const int32_t tile_elements = n * K;
@@ -1009,10 +1038,124 @@ __global__ __launch_bounds__(GATHER_SENDERS* WAVE) void sum_by_sender_kernel(
     }
 }
 
+// The pass over the sender index needs none of the per-edge rows, so it can
+// run beside the kernel that writes them (sender_buckets.hpp:
+// list_edges_in_slots): used while a sender has SLOT_MEAN_LIMIT edges or fewer
+// on average.
+constexpr int SLOT_MEAN_LIMIT = 32;
+
+// The sum over the slots: one wavefront per sender, ascending edge order, as
+// many rows in flight as 32 registers hold (COLUMNS values of a row per lane).
+// A sender with more edges than places (rare by the choice of SLOT_MEAN_LIMIT)
+// is looked after by its wavefront alone, which then reads the whole sender
+// index itself.
+constexpr int LISTED_WAVES = 4;
+
+template <typename T, int COLUMNS>
+__global__ __launch_bounds__(LISTED_WAVES* WAVE) void sum_slotted_rows_kernel(
+    T* __restrict__ grad_W, const T* __restrict__ edge_W, const int32_t* __restrict__ slots,
+    const int32_t* __restrict__ counts, const int32_t* __restrict__ senders, int32_t n_edges,
+    int32_t n_nodes, int32_t L
+) {
+    const int lane = threadIdx.x & (WAVE - 1);
+    const int32_t node = __builtin_amdgcn_readfirstlane(blockIdx.x * LISTED_WAVES + (threadIdx.x >> 6));
+    if (node >= n_nodes) {
+        return;
+    }
+    const int32_t* mine = slots + static_cast<size_t>(node) * SLOT_CAPACITY;
+    // all places asked for before the counts are known
+    const int32_t first_half = mine[lane];
+    const int32_t second_half = mine[lane + WAVE];
+    static_assert(SLOT_PARTS == 4 && SLOT_CAPACITY == 2 * WAVE, "the four parts of a sender's places in two registers");
+    const int4 part_counts = reinterpret_cast<const int4*>(counts)[node];
+    const int32_t c0 = __builtin_amdgcn_readfirstlane(part_counts.x);
+    const int32_t c1 = __builtin_amdgcn_readfirstlane(part_counts.y);
+    const int32_t c2 = __builtin_amdgcn_readfirstlane(part_counts.z);
+    const int32_t c3 = __builtin_amdgcn_readfirstlane(part_counts.w);
+    const bool listed = max(max(c0, c1), max(c2, c3)) <= SLOT_PART_CAPACITY;
+    const int32_t count = c0 + c1 + c2 + c3;
+    T sum[COLUMNS];
+    uint32_t column[COLUMNS];
+#pragma unroll
+    for (int c = 0; c < COLUMNS; c++) {
+        sum[c] = T(0);
+        column[c] = min(lane + c * WAVE, L - 1);
+    }
+    constexpr int ROWS = 32 / (COLUMNS * static_cast<int>(sizeof(T) / 4));
+    // adds the rows of the first n <= 64 edges held by the lanes of `my_edge`
+    auto add_rows = [&](int32_t my_edge, int32_t n) {
+#pragma unroll 1
+        for (int32_t k0 = 0; k0 < n; k0 += ROWS) {
+            T values[ROWS][COLUMNS];
+#pragma unroll
+            for (int k = 0; k < ROWS; k++) {
+                // beyond n: some row that exists, left out of the sum
+                const int32_t edge = __builtin_amdgcn_readlane(my_edge, min(k0 + k, WAVE - 1));
+                const T* row = edge_W + static_cast<size_t>(edge) * L;
+#pragma unroll
+                for (int c = 0; c < COLUMNS; c++) {
+                    values[k][c] = row[column[c]];
+                }
+            }
+#pragma unroll
+            for (int k = 0; k < ROWS; k++) {
+                if (k0 + k < n) {
+#pragma unroll
+                    for (int c = 0; c < COLUMNS; c++) {
+                        sum[c] += values[k][c];
+                    }
+                }
+            }
+        }
+    };
+    if (listed) {
+        // the parts moved together: position p of the list is in part `part`, place p - before
+        auto edge_at = [&](int32_t position) {
+            const int32_t part = (position >= c0 ? 1 : 0) + (position >= c0 + c1 ? 1 : 0) +
+                                 (position >= c0 + c1 + c2 ? 1 : 0);
+            const int32_t before = part == 0 ? 0 : part == 1 ? c0 : part == 2 ? c0 + c1 : c0 + c1 + c2;
+            const int32_t place = part * SLOT_PART_CAPACITY + position - before;
+            const int32_t low = __shfl(first_half, place & (WAVE - 1));
+            const int32_t high = __shfl(second_half, place & (WAVE - 1));
+            return place < WAVE ? low : high;
+        };
+        const int32_t n_first = min(count, WAVE);
+        const int32_t first = edge_at(lane);
+        add_rows(lane < n_first ? first : 0, n_first);
+        if (count > WAVE) {
+            const int32_t n_second = count - WAVE;
+            const int32_t second = edge_at(lane + WAVE);
+            add_rows(lane < n_second ? second : 0, n_second);
+        }
+    } else {
+        const unsigned long long below = (1ull << lane) - 1ull;
+        for (int32_t base = 0; base < n_edges; base += WAVE) {
+            const int32_t e = base + lane;
+            const bool named = e < n_edges && senders[min(e, n_edges - 1)] == node;
+            const unsigned long long mask = __ballot(named);
+            if (mask != 0) {
+                // the matches moved to the first lanes, in edge order
+                // (a permutation of the lanes: the others follow, in their order)
+                const int32_t n = __popcll(mask);
+                const int32_t named_below = __popcll(mask & below);
+                const int32_t place = named ? named_below : n + lane - named_below;
+                const int32_t packed = __builtin_amdgcn_ds_permute(place << 2, e);
+                add_rows(lane < n ? packed : 0, n);
+            }
+        }
+    }
+#pragma unroll
+    for (int c = 0; c < COLUMNS; c++) {
+        const int32_t l = lane + c * WAVE;
+        if (l < L) {
+            grad_W[static_cast<size_t>(node) * L + l] = sum[c];
+        }
+    }
+}
+
 // The same sum over lists that are already there (sender_buckets.hpp: the edges in
 // the order of their senders, built beside the per-edge kernel on a side
 // stream): one wavefront per sender, sixteen rows in flight.
-constexpr int LISTED_WAVES = 4;
 
 template <typename T>
 __global__ __launch_bounds__(LISTED_WAVES* WAVE) void sum_listed_rows_kernel(
@@ -1260,8 +1403,14 @@ void launch_vjp(
     const bool narrow_rows = L <= GATHER_COLUMNS * WAVE;
     // (at 60 000 edges the lists cost more than the scans: 52 us against 32 for the whole vjp)
     const bool gather_in_kernel = narrow_rows && n_edges > 0 && index_reads <= SENDER_SCAN_LIMIT;
+    // sparse graphs: the pass over the sender index runs beside the per-edge kernel
+    // and leaves every sender's edges in places of its own
+    // (c3 shape, f32: 33 us -> see the design notes; hubs with thousands of edges keep the gather)
+    const bool slotted = want_W && gather_in_kernel && n_output > 0 && L > 0 &&
+                         static_cast<size_t>(n_edges) <= static_cast<size_t>(n_output) * SLOT_MEAN_LIMIT;
+    const size_t slots_bytes = slotted ? sender_slots_bytes(n_output) : 0;
     const size_t buckets_bytes =
-        want_W && !gather_in_kernel ? edges_by_sender_bytes(n_output, n_edges) : 0;
+        want_W && !gather_in_kernel ? edges_by_sender_bytes(n_output, n_edges) : slots_bytes;
     char* workspace =
         want_W ? static_cast<char*>(scratch(edge_w_bytes + buckets_bytes)) : nullptr;
     T* edge_W = want_W ? reinterpret_cast<T*>(workspace) : nullptr;
@@ -1270,8 +1419,10 @@ void launch_vjp(
     // built beside them, on a side stream that joins before the lists are used
     SenderBuckets buckets{};
     EdgesBySender by_sender{};
+    SenderSlots slots{};
     const bool use_buckets = want_W && n_output > 0 && L > 0 && !gather_in_kernel;
     std::unique_ptr<SideStream> beside;
+    bool listed = false; // the slots are being filled by a kernel that is already enqueued
     if (use_buckets) {
         beside = std::make_unique<SideStream>(stream);
         if (narrow_rows) {
@@ -1326,11 +1477,22 @@ void launch_vjp(
                                  reinterpret_cast<uintptr_t>(B.data) % 16 == 0 &&
                                  reinterpret_cast<uintptr_t>(grad_output.data) % 16 == 0 &&
                                  (!WEIGHTED || reinterpret_cast<uintptr_t>(W) % 16 == 0);
-#define MOPS_LAUNCH_ROWS_AS(KT, NT, VECTORS, BLOCKS)                                                \
-    edge_rows_vjp_kernel<T, KT, NT, WEIGHTED, VECTORS, BLOCKS><<<groups, WAVE, 0, stream>>>(       \
+#define MOPS_LAUNCH_ROWS_WITH(KT, NT, VECTORS, BLOCKS, LISTS, GRID, WAVES)                          \
+    edge_rows_vjp_kernel<T, KT, NT, WEIGHTED, VECTORS, BLOCKS, LISTS><<<GRID, (WAVES) * WAVE, 0, stream>>>( \
         grad_A.data, grad_B.data, edge_W, grad_output.data, A.data, B.data, W, indices_W,          \
-        indices_output.data, n_edges, n_output, K, L                                               \
+        indices_output.data, n_edges, n_output, K, L, const_cast<int32_t*>(slots.edges),           \
+        const_cast<int32_t*>(slots.counts), static_cast<int32_t>(list_blocks), aligned_senders     \
     )
+#define MOPS_LAUNCH_ROWS_AS(KT, NT, VECTORS, BLOCKS)                                                \
+    if constexpr (WEIGHTED) {                                                                      \
+        if (list_blocks > 0) {                                                                     \
+            MOPS_LAUNCH_ROWS_WITH(KT, NT, VECTORS, BLOCKS, true, listing_grid, LISTING_WAVES);     \
+        } else {                                                                                   \
+            MOPS_LAUNCH_ROWS_WITH(KT, NT, VECTORS, BLOCKS, false, groups, 1);                      \
+        }                                                                                          \
+    } else {                                                                                       \
+        MOPS_LAUNCH_ROWS_WITH(KT, NT, VECTORS, BLOCKS, false, groups, 1);                          \
+    }
 #define MOPS_LAUNCH_ROWS(KT, NT)                                                                   \
     if (vectors) {                                                                                 \
         MOPS_LAUNCH_ROWS_AS(KT, NT, true, false);                                                  \
@@ -1343,6 +1505,15 @@ void launch_vjp(
     } else {                                                                                       \
         MOPS_LAUNCH_ROWS_AS(KT, 4, false, true);                                                   \
     }
+            // the listing of the senders' edges rides along in this launch
+            const unsigned list_blocks = slotted ? sender_slots_blocks(n_output) : 0;
+            const unsigned listing_grid =
+                list_blocks + static_cast<unsigned>(ceil_div(static_cast<size_t>(groups), LISTING_WAVES));
+            const bool aligned_senders = reinterpret_cast<uintptr_t>(indices_W) % 16 == 0;
+            if (slotted) {
+                slots = sender_slots_in(workspace + edge_w_bytes, n_output);
+                listed = true;
+            }
             if (K <= 16) {
                 if (L <= 16) {
                     MOPS_LAUNCH_ROWS(1, 1);
@@ -1367,6 +1538,7 @@ void launch_vjp(
 #undef MOPS_LAUNCH_ROW_PASSES
 #undef MOPS_LAUNCH_ROWS
 #undef MOPS_LAUNCH_ROWS_AS
+#undef MOPS_LAUNCH_ROWS_WITH
         } else {
             MainKernelTimer timer(stream);
             vjp_kernel<T, WEIGHTED><<<waves, WAVE, lds, stream>>>(
@@ -1376,7 +1548,24 @@ void launch_vjp(
         }
     }
 
-    if (want_W && n_output > 0 && L > 0 && gather_in_kernel) {
+    if (slotted) {
+        if (!listed) {
+            slots = list_edges_in_slots(indices_W, n_edges, n_output, workspace + edge_w_bytes, stream);
+        }
+        const unsigned blocks = static_cast<unsigned>(ceil_div(static_cast<size_t>(n_output), LISTED_WAVES));
+#define MOPS_LAUNCH_SLOTTED(COLUMNS)                                                                \
+    sum_slotted_rows_kernel<T, COLUMNS><<<blocks, LISTED_WAVES * WAVE, 0, stream>>>(               \
+        grad_W.data, edge_W, slots.edges, slots.counts, indices_W, n_edges, n_output, L                   \
+    )
+        if (L <= WAVE) {
+            MOPS_LAUNCH_SLOTTED(1);
+        } else if (L <= 2 * WAVE) {
+            MOPS_LAUNCH_SLOTTED(2);
+        } else {
+            MOPS_LAUNCH_SLOTTED(4);
+        }
+#undef MOPS_LAUNCH_SLOTTED
+    } else if (want_W && n_output > 0 && L > 0 && gather_in_kernel) {
         const bool aligned = reinterpret_cast<uintptr_t>(indices_W) % 16 == 0;
         const unsigned blocks = static_cast<unsigned>(ceil_div(static_cast<size_t>(n_output), GATHER_SENDERS));
         sum_by_sender_kernel<T><<<blocks, GATHER_SENDERS * WAVE, 0, stream>>>(

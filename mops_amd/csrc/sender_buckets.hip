@@ -1,5 +1,7 @@
 #include "sender_buckets.hpp"
 
+#include <algorithm>
+
 #include "runtime.hpp"
 
 namespace mops::amd {
@@ -250,7 +252,50 @@ __global__ __launch_bounds__(SMALL_THREADS) void order_small_kernel(
     }
 }
 
+// Sparse graphs: one launch of list_in_slots_block (sender_buckets.hpp), four
+// wavefronts per workgroup.
+constexpr int SLOT_THREADS = 4 * WAVE;
+
+__global__ __launch_bounds__(SLOT_THREADS) void list_in_slots_kernel(
+    int32_t* __restrict__ slots, int32_t* __restrict__ counts, const int32_t* __restrict__ senders,
+    int32_t n_edges, int32_t n_nodes, bool aligned
+) {
+    __shared__ SlotLists lists;
+    list_in_slots_block<SLOT_THREADS>(lists, slots, counts, senders, n_edges, n_nodes, aligned, blockIdx.x);
+}
+
 } // namespace
+
+size_t sender_slots_bytes(int32_t n_nodes) {
+    return align256(static_cast<size_t>(n_nodes) * SLOT_CAPACITY * 4) +
+           align256(static_cast<size_t>(n_nodes) * SLOT_PARTS * 4);
+}
+
+SenderSlots sender_slots_in(void* workspace, int32_t n_nodes) {
+    int32_t* slots = static_cast<int32_t*>(workspace);
+    int32_t* counts = reinterpret_cast<int32_t*>(
+        static_cast<char*>(workspace) + align256(static_cast<size_t>(n_nodes) * SLOT_CAPACITY * 4)
+    );
+    return SenderSlots{slots, counts};
+}
+
+unsigned sender_slots_blocks(int32_t n_nodes) {
+    return static_cast<unsigned>(ceil_div(static_cast<size_t>(std::max(n_nodes, 0)), SLOT_SENDERS)) * SLOT_PARTS;
+}
+
+SenderSlots list_edges_in_slots(
+    const int32_t* senders, int32_t n_edges, int32_t n_nodes, void* workspace, hipStream_t stream
+) {
+    const SenderSlots slots = sender_slots_in(workspace, n_nodes);
+    if (n_nodes > 0) {
+        const bool aligned = reinterpret_cast<uintptr_t>(senders) % 16 == 0;
+        list_in_slots_kernel<<<sender_slots_blocks(n_nodes), SLOT_THREADS, 0, stream>>>(
+            const_cast<int32_t*>(slots.edges), const_cast<int32_t*>(slots.counts), senders, n_edges, n_nodes, aligned
+        );
+        MOPS_HIP_CHECK(hipGetLastError());
+    }
+    return slots;
+}
 
 size_t edges_by_sender_bytes(int32_t n_nodes, int32_t n_edges) {
     return sender_buckets_bytes(n_nodes, n_edges) + 2 * align256(static_cast<size_t>(n_edges) * 4);

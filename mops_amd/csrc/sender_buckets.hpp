@@ -64,6 +64,158 @@ EdgesBySender order_edges_by_sender(
     const int32_t* senders, int32_t n_edges, int32_t n_nodes, void* workspace, hipStream_t stream
 );
 
+/// Sparse graphs (a few dozen edges per sender): every sender owns
+/// SLOT_CAPACITY places, so no offsets have to be known before the lists are
+/// written and ONE launch does it, without counters shared between workgroups
+/// and without anything to clear first. The index is cut into SLOT_PARTS parts
+/// of consecutive edges, each looked at by workgroups of its own, and so are a
+/// sender's places: its edges in part p go to places [32 p, 32 p + 32). The
+/// parts one after the other are the sender's edges in ascending order.
+constexpr int SLOT_PARTS = 4;
+constexpr int SLOT_PART_CAPACITY = 32;
+constexpr int SLOT_CAPACITY = SLOT_PARTS * SLOT_PART_CAPACITY;
+struct SenderSlots {
+    /// [n_nodes][SLOT_PARTS][SLOT_PART_CAPACITY] the edges that name the node in
+    /// each part of the index, ascending, in the first counts[node][part] places
+    /// (nothing in a part whose count exceeds SLOT_PART_CAPACITY)
+    const int32_t* edges;
+    /// [n_nodes][SLOT_PARTS] number of edges of the part that name the node (may
+    /// exceed SLOT_PART_CAPACITY: the consumer then has to find the node's edges
+    /// itself)
+    const int32_t* counts;
+};
+
+/// Bytes of scratch memory list_edges_in_slots needs.
+size_t sender_slots_bytes(int32_t n_nodes);
+
+/// Where the two arrays lie in a workspace of sender_slots_bytes() bytes (for a
+/// kernel that does the listing among other work: list_in_slots_block).
+SenderSlots sender_slots_in(void* workspace, int32_t n_nodes);
+
+/// Workgroups the listing takes: SLOT_PARTS for every 16 senders.
+unsigned sender_slots_blocks(int32_t n_nodes);
+
+/// Enqueue the kernel that lists the edges of every sender in its slots
+/// (values outside [0, n_nodes) are dropped). A workgroup serves 16 senders and
+/// reads a quarter of the index: meant for graphs where n_edges * n_nodes / 16
+/// is small.
+SenderSlots list_edges_in_slots(
+    const int32_t* senders, int32_t n_edges, int32_t n_nodes, void* workspace, hipStream_t stream
+);
+
+/// Senders per workgroup of the listing.
+constexpr int SLOT_SENDERS = 16;
+/// LDS of one workgroup of the listing.
+struct SlotLists {
+    int32_t edges[SLOT_SENDERS][SLOT_PART_CAPACITY];
+    int32_t found[SLOT_SENDERS];
+};
+
+/// The listing itself, called by ALL threads of a workgroup of THREADS threads
+/// (a multiple of 64): workgroup `block` lists the edges of senders
+/// [16 g, 16 g + 16), g = block / SLOT_PARTS, in part block % SLOT_PARTS of the
+/// index. Every thread looks at its share of the part, sixteen loads in flight
+/// (128-bit loads when `aligned`: `senders` on a 16-byte boundary); an edge that
+/// names one of the sixteen takes the next place of that sender's list in LDS
+/// (integer LDS atomic: the places depend on the order of arrival, the set of
+/// edges does not); a wavefront then puts a list in ascending order (the rank of
+/// an edge is the number of smaller ones: edge numbers are distinct) and writes
+/// it to the sender's slots. A device function so that a kernel with other work
+/// can give some of its workgroups to it: no launch of its own then.
+template <int THREADS>
+__device__ __forceinline__ void list_in_slots_block(
+    SlotLists& lds, int32_t* __restrict__ slots, int32_t* __restrict__ counts,
+    const int32_t* __restrict__ senders, int32_t n_edges, int32_t n_nodes, bool aligned, int32_t block
+) {
+    constexpr int WAVES = THREADS / WAVE;
+    const int tid = threadIdx.x;
+    const int lane = tid & (WAVE - 1);
+    const int wave = tid >> 6;
+    const int32_t part = block % SLOT_PARTS;
+    const int32_t node0 = block / SLOT_PARTS * SLOT_SENDERS;
+    const int32_t served = min(SLOT_SENDERS, n_nodes - node0);
+    if (tid < SLOT_SENDERS) {
+        lds.found[tid] = 0;
+    }
+    __syncthreads();
+    auto look = [&](int32_t value, int32_t edge) {
+        const int32_t which = value - node0;
+        if (in_bounds(which, served)) {
+            const int32_t place = atomicAdd(&lds.found[which], 1);
+            if (place < SLOT_PART_CAPACITY) {
+                lds.edges[which][place] = edge;
+            }
+        }
+    };
+    constexpr int AHEAD = 16;
+    if (aligned) {
+        // parts of whole groups of four; the last part also takes the n_edges % 4 edges after them
+        const int32_t groups = n_edges >> 2;
+        const int32_t per_part = (groups + SLOT_PARTS - 1) / SLOT_PARTS;
+        const int32_t begin = min(part * per_part, groups);
+        const int32_t end = min(begin + per_part, groups);
+        for (int32_t g0 = begin; g0 < end; g0 += AHEAD * THREADS) {
+            int4 values[AHEAD];
+#pragma unroll
+            for (int u = 0; u < AHEAD; u++) {
+                // beyond the end: a group that exists, and values that name nobody
+                // (a conditional load would make every load wait for the one before)
+                const int32_t g = g0 + u * THREADS + tid;
+                const bool ok = g < end;
+                const int4 loaded = reinterpret_cast<const int4*>(senders)[ok ? g : 0];
+                values[u].x = ok ? loaded.x : -1;
+                values[u].y = ok ? loaded.y : -1;
+                values[u].z = ok ? loaded.z : -1;
+                values[u].w = ok ? loaded.w : -1;
+            }
+#pragma unroll
+            for (int u = 0; u < AHEAD; u++) {
+                const int32_t edge = (g0 + u * THREADS + tid) << 2;
+                look(values[u].x, edge);
+                look(values[u].y, edge + 1);
+                look(values[u].z, edge + 2);
+                look(values[u].w, edge + 3);
+            }
+        }
+        const int32_t e = (n_edges & ~3) + tid;
+        if (part == SLOT_PARTS - 1 && tid < 4 && e < n_edges) {
+            look(senders[e], e);
+        }
+    } else {
+        const int32_t per_part = (n_edges + SLOT_PARTS - 1) / SLOT_PARTS;
+        const int32_t begin = min(part * per_part, n_edges);
+        const int32_t end = min(begin + per_part, n_edges);
+        for (int32_t e0 = begin; e0 < end; e0 += AHEAD * THREADS) {
+            int32_t values[AHEAD];
+#pragma unroll
+            for (int u = 0; u < AHEAD; u++) {
+                const int32_t e = e0 + u * THREADS + tid;
+                const int32_t loaded = load_or_zero(senders, static_cast<size_t>(e), e < end);
+                values[u] = e < end ? loaded : -1;
+            }
+#pragma unroll
+            for (int u = 0; u < AHEAD; u++) {
+                look(values[u], e0 + u * THREADS + tid);
+            }
+        }
+    }
+    __syncthreads();
+    for (int32_t which = wave; which < served; which += WAVES) {
+        const int32_t n = lds.found[which];
+        if (lane < n && n <= SLOT_PART_CAPACITY) {
+            const int32_t edge = lds.edges[which][lane];
+            int32_t rank = 0;
+            for (int32_t other = 0; other < n; other++) {
+                rank += lds.edges[which][other] < edge ? 1 : 0; // the same address for all lanes
+            }
+            slots[(static_cast<size_t>(node0 + which) * SLOT_PARTS + part) * SLOT_PART_CAPACITY + rank] = edge;
+        }
+        if (lane == 0) {
+            counts[static_cast<size_t>(node0 + which) * SLOT_PARTS + part] = n;
+        }
+    }
+}
+
 /// Capacity (in edges) of the LDS array passed to sorted_bucket.
 constexpr int BUCKET_LDS_CAPACITY = 1024;
 

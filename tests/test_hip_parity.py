@@ -58,6 +58,9 @@ CASES = {
         "long_segments": lambda s, d: support.opsaw_case(s, d, E=3000, K=5, L=7, n_nodes=6),
         "hub_sender": lambda s, d: _hub(support.opsaw_case(s, d, E=2600, K=3, L=5, n_nodes=9), "indices_W"),
         "mostly_empty": lambda s, d: support.opsaw_case(s, d, E=20, K=4, L=4, n_nodes=300, allow_empty=True),
+        "sparse_with_hubs": lambda s, d: _with_sender_counts(
+            support.opsaw_case(s, d, E=6000, K=4, L=32, n_nodes=300, allow_empty=True), "indices_W", SENDER_COUNTS
+        ),
         "pooling": lambda s, d: support.opsaw_case(s, d, E=5000, K=13, L=32, n_nodes=7),
         "pooling_mixed_lengths": lambda s, d: _with_lengths(
             support.opsaw_case(s, d, E=sum(MIXED_LENGTHS), K=3, L=17, n_nodes=len(MIXED_LENGTHS)), "indices_output", MIXED_LENGTHS
@@ -140,6 +143,28 @@ def _with_lengths(case, key, lengths):
 
 # lengths around the distance at which long segments are cut (256), rows without edges, one row over many cuts
 MIXED_LENGTHS = [0, 1700, 3, 0, 2300, 255, 256, 257, 512, 1, 0, 1900, 0, 769]
+
+
+# senders of a sparse graph (20 edges per sender on average) named by exactly this many edges:
+# around the 64 edges one wavefront holds, around the 128 places a sender owns, and far beyond
+SENDER_COUNTS = {5: 1000, 7: 128, 9: 129, 11: 64, 13: 65, 15: 0, 299: 127}
+
+
+def _with_sender_counts(case, key, counts):
+    """Sender index in which sender v is named by exactly counts[v] edges, at random positions."""
+    index = case[key]
+    n_nodes = int(index.max()) + 1
+    for value in counts:
+        index[index == value] = (value + 1) % n_nodes
+    assert not set(counts) & {(value + 1) % n_nodes for value in counts}
+    positions = np.random.default_rng(len(index)).permutation(len(index))
+    used = 0
+    for value, count in counts.items():
+        index[positions[used : used + count]] = value
+        used += count
+    for value, count in counts.items():
+        assert int((index == value).sum()) == count
+    return case
 
 
 def _hub(case, key):
