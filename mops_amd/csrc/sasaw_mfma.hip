@@ -113,6 +113,17 @@ DenseLayout dense_layout(const Shape& s) {
 constexpr int DENSE_THREADS = 256;
 constexpr int TABLE_TILE = 1024;
 
+/// What the workgroups of dense_coupling_kernel from `first_block` on list
+/// (nothing: first_block beyond the grid).
+struct SlotListing {
+    int32_t first_block;
+    int32_t* edges;
+    int32_t* counts;
+    const int32_t* senders;
+    int32_t n_edges, n_nodes;
+    bool aligned;
+};
+
 // Every thread owns one operand slot and adds up, in ascending entry order,
 // the coefficients of the entries that fall on it.
 //   to_cells[(tile * MAX_A_STEPS + step) * 64 + lane] = D[16 * tile + (lane & 15)][4 * step + (lane >> 4)]
@@ -129,8 +140,21 @@ __global__ __launch_bounds__(DENSE_THREADS) void dense_coupling_kernel(
     int32_t nA,
     int32_t n2,
     int32_t n3,
-    DenseLayout layout
+    DenseLayout layout,
+    SlotListing listing
 ) {
+    // Workgroups after the table's own list the edges of every sender in its
+    // slots (sender_buckets.hpp) for the weight-gradient kernel of a vjp: the
+    // pass over the sender index needs no launch of its own that way, and no
+    // time of its own either (this launch is a few microseconds of latency).
+    if (static_cast<int32_t>(blockIdx.x) >= listing.first_block) {
+        __shared__ SlotLists lists;
+        list_in_slots_block<DENSE_THREADS>(
+            lists, listing.edges, listing.counts, listing.senders, listing.n_edges, listing.n_nodes,
+            listing.aligned, static_cast<int32_t>(blockIdx.x) - listing.first_block
+        );
+        return;
+    }
     __shared__ int32_t keys[TABLE_TILE];
     __shared__ T coefficients[TABLE_TILE];
 
@@ -639,10 +663,86 @@ __global__ __launch_bounds__(forward_waves<T>() * WAVE) void forward_kernel(
 /// Wavefronts (= senders) per workgroup.
 template <typename T> constexpr int senders_per_group() { return 4; } // (8: 1 % faster at c4, twice the LDS)
 
+/// grad_W of ONE sender by one wavefront, the sender's edges read from its
+/// slots (sender_buckets.hpp; listed by workgroups of the launch that made the
+/// dense table). `t_area`: this wavefront's T area in LDS.
+template <typename T, int NT, int RS>
+__device__ __forceinline__ void weight_gradient_of_sender(
+    T* __restrict__ grad_W, const int32_t* __restrict__ senders, int32_t n_edges, const Contraction<T>& p,
+    const int32_t* __restrict__ slot_edges, const int32_t* __restrict__ slot_counts, int32_t node,
+    T* t_area, int lane
+) {
+    ContractionLane<T, NT, RS> mine_lane;
+    mine_lane.setup(p, lane);
+    clear_zero_row(t_area, p.layout, lane);
+    Accumulators<T, NT> acc;
+    acc.clear();
+    auto on_stage = [&](int32_t my_edge, int32_t n) {
+        const int32_t my_source = my_edge >= 0 ? p.gather_index[my_edge] : -1;
+        contract_batch<T, NT, RS>(acc, p, mine_lane, t_area, my_edge, my_source, n, lane);
+    };
+    const int32_t* mine = slot_edges + static_cast<size_t>(node) * SLOT_CAPACITY;
+    const int32_t first_half = mine[lane];
+    const int32_t second_half = mine[lane + WAVE];
+    static_assert(SLOT_PARTS == 4 && SLOT_CAPACITY == 2 * WAVE, "the four parts of a sender's places in two registers");
+    const int4 part_counts = reinterpret_cast<const int4*>(slot_counts)[node];
+    const int32_t c0 = __builtin_amdgcn_readfirstlane(part_counts.x);
+    const int32_t c1 = __builtin_amdgcn_readfirstlane(part_counts.y);
+    const int32_t c2 = __builtin_amdgcn_readfirstlane(part_counts.z);
+    const int32_t c3 = __builtin_amdgcn_readfirstlane(part_counts.w);
+    const int32_t count = c0 + c1 + c2 + c3;
+    // lane p of `edges` holds edge p of n <= 64: handed on 16 at a time
+    auto hand_on = [&](int32_t edges, int32_t n) {
+        for (int32_t k0 = 0; k0 < n; k0 += STAGE) {
+            const int32_t m = min(STAGE, n - k0);
+            const int k = lane & (STAGE - 1);
+            const int32_t edge = __shfl(edges, k0 + k);
+            on_stage(k < m ? edge : -1, m);
+        }
+    };
+    if (max(max(c0, c1), max(c2, c3)) <= SLOT_PART_CAPACITY) {
+        // the parts moved together: position p of the list is in part `part`, place p - before
+        auto edge_at = [&](int32_t position) {
+            const int32_t part = (position >= c0 ? 1 : 0) + (position >= c0 + c1 ? 1 : 0) +
+                                 (position >= c0 + c1 + c2 ? 1 : 0);
+            const int32_t before = part == 0 ? 0 : part == 1 ? c0 : part == 2 ? c0 + c1 : c0 + c1 + c2;
+            const int32_t place = part * SLOT_PART_CAPACITY + position - before;
+            const int32_t low = __shfl(first_half, place & (WAVE - 1));
+            const int32_t high = __shfl(second_half, place & (WAVE - 1));
+            return place < WAVE ? low : high;
+        };
+        hand_on(edge_at(lane), min(count, WAVE));
+        if (count > WAVE) {
+            hand_on(edge_at(lane + WAVE), count - WAVE);
+        }
+    } else {
+        // more edges in a part than places (a hub of a sparse graph): this
+        // wavefront reads the whole sender index itself
+        const unsigned long long below = (1ull << lane) - 1ull;
+        for (int32_t base = 0; base < n_edges; base += WAVE) {
+            const int32_t e = base + lane;
+            const bool named = e < n_edges && senders[min(e, n_edges - 1)] == node;
+            const unsigned long long mask = __ballot(named);
+            if (mask != 0) {
+                // the matches moved to the first lanes, in edge order
+                // (a permutation of the lanes: the others follow, in their order)
+                const int32_t n = __popcll(mask);
+                const int32_t named_below = __popcll(mask & below);
+                const int32_t place = named ? named_below : n + lane - named_below;
+                hand_on(__builtin_amdgcn_ds_permute(place << 2, e), n);
+            }
+        }
+    }
+    store_block<T, NT>(
+        grad_W + static_cast<size_t>(node) * p.n_out * p.ld, [&](int t, int r) { return acc.total(t, r); },
+        p.n_out, p.L, p.ld, lane
+    );
+}
+
 template <typename T, int NT, int RS>
 __global__ __launch_bounds__(senders_per_group<T>() * WAVE) void weight_gradient_kernel(
     T* __restrict__ grad_W, const int32_t* __restrict__ senders, int32_t n_edges, bool aligned_senders,
-    const Contraction<T> p
+    const Contraction<T> p, const int32_t* __restrict__ slot_edges, const int32_t* __restrict__ slot_counts
 ) {
     constexpr int SENDERS_PER_GROUP = senders_per_group<T>();
     using Gather = SenderGather<SENDERS_PER_GROUP>;
@@ -654,6 +754,13 @@ __global__ __launch_bounds__(senders_per_group<T>() * WAVE) void weight_gradient
                 wave * p.layout.t_elements();
     const int32_t node0 = blockIdx.x * SENDERS_PER_GROUP;
     const int32_t node = node0 + wave;
+    if (slot_edges != nullptr) {
+        // the edges of every sender are listed already: a wavefront needs nobody else
+        if (node < p.n_blocks) {
+            weight_gradient_of_sender<T, NT, RS>(grad_W, senders, n_edges, p, slot_edges, slot_counts, node, t_area, lane);
+        }
+        return;
+    }
 
     ContractionLane<T, NT, RS> mine;
     mine.setup(p, lane);
@@ -703,8 +810,22 @@ template <typename T> struct EdgeGradArgs {
 constexpr int EDGE_BATCH = 2; // edges whose W blocks are in LDS together (4: more LDS and registers
                               // per wavefront, 98 instead of 89 us for the whole vjp; 1: 112 us)
 
-template <typename T, int NT, int M2S>
-__global__ __launch_bounds__(WAVE) void edge_gradients_kernel(const EdgeGradArgs<T> p) {
+/// grad_W in the same launch (WITH_WEIGHTS): the first `n_senders` workgroups
+/// are one sender each (weight_gradient_of_sender), the others 16 edges each.
+/// The two halves of a vjp do not depend on each other and both wait for
+/// memory most of the time; as one launch they share the device without a
+/// second stream (forking and joining streams costs about 10 us per call,
+/// also as nodes of a graph).
+template <typename T> struct WeightGradArgs {
+    T* grad_W;
+    Contraction<T> contraction;
+    const int32_t* slot_edges;
+    const int32_t* slot_counts;
+    int32_t n_senders;
+};
+
+template <typename T, int NT, int M2S, bool WITH_WEIGHTS>
+__global__ __launch_bounds__(WAVE) void edge_gradients_kernel(const EdgeGradArgs<T> p, const WeightGradArgs<T> w) {
     using M = Mfma<T>;
     constexpr int L_STEPS = 4 * NT;
     constexpr uint32_t ELEMENT = sizeof(T);
@@ -716,12 +837,22 @@ __global__ __launch_bounds__(WAVE) void edge_gradients_kernel(const EdgeGradArgs
     const int32_t lds_elements = p.layout.t_elements() + EDGE_BATCH * (p.n2 + 1) * p.Ls;
 
     const int lane = threadIdx.x;
+    if constexpr (WITH_WEIGHTS) {
+        // (M2S steps of four cover n3 as well as n2 here: the host sees to it)
+        if (static_cast<int32_t>(blockIdx.x) < w.n_senders) {
+            weight_gradient_of_sender<T, NT, M2S>(
+                w.grad_W, p.senders, p.n_edges, w.contraction, w.slot_edges, w.slot_counts,
+                static_cast<int32_t>(blockIdx.x), t_area, lane
+            );
+            return;
+        }
+    }
     const int i = lane & 15;
     const int q = lane >> 4;
     const bool want_A = p.grad_A != nullptr;
     const bool want_B = p.grad_B != nullptr;
 
-    const int32_t chunk_begin = blockIdx.x * STAGE;
+    const int32_t chunk_begin = (static_cast<int32_t>(blockIdx.x) - (WITH_WEIGHTS ? w.n_senders : 0)) * STAGE;
     const int32_t n = min(STAGE, p.n_edges - chunk_begin);
     const int32_t my_edge = i < n ? chunk_begin + i : -1;
     const int32_t my_source = my_edge >= 0 ? p.senders[my_edge] : -1;
@@ -1023,16 +1154,29 @@ size_t dense_bytes(const DenseLayout& layout, size_t element_size) {
 template <typename T>
 DenseBuffers<T> enqueue_dense(
     void* workspace, const DenseLayout& layout, const T* C, const Indices& indices, const Shape& s,
-    hipStream_t stream
+    hipStream_t stream, const SenderSlots* slots_wanted = nullptr
 ) {
     DenseBuffers<T> buffers;
     char* base = static_cast<char*>(workspace);
     buffers.to_cells = reinterpret_cast<T*>(base);
     buffers.to_A = reinterpret_cast<T*>(base + align256(static_cast<size_t>(layout.to_cells_slots()) * sizeof(T)));
     const int32_t slots = layout.to_cells_slots() + layout.to_A_slots();
-    dense_coupling_kernel<T><<<(slots + DENSE_THREADS - 1) / DENSE_THREADS, DENSE_THREADS, 0, stream>>>(
+    const int32_t dense_blocks = (slots + DENSE_THREADS - 1) / DENSE_THREADS;
+    SlotListing listing{};
+    listing.first_block = dense_blocks;
+    unsigned listing_blocks = 0;
+    if (slots_wanted != nullptr) {
+        listing.edges = const_cast<int32_t*>(slots_wanted->edges);
+        listing.counts = const_cast<int32_t*>(slots_wanted->counts);
+        listing.senders = indices.W_1;
+        listing.n_edges = s.n_edges;
+        listing.n_nodes = s.n_nodes;
+        listing.aligned = reinterpret_cast<uintptr_t>(indices.W_1) % 16 == 0;
+        listing_blocks = sender_slots_blocks(s.n_nodes);
+    }
+    dense_coupling_kernel<T><<<dense_blocks + listing_blocks, DENSE_THREADS, 0, stream>>>(
         buffers.to_cells, buffers.to_A, C, indices.A, indices.W_2, indices.output_2, s.N, s.nA, s.n2, s.n3,
-        layout
+        layout, listing
     );
     MOPS_HIP_CHECK(hipGetLastError());
     return buffers;
@@ -1181,9 +1325,19 @@ bool orders_edges_by_sender(const Shape& s, size_t element_size) {
            weight_gradient_lds(widest_block(s), element_size) > WEIGHT_LDS_BUDGET;
 }
 
+/// Sparse graphs that take the in-kernel path: the edges of every sender are
+/// listed in slots (sender_buckets.hpp) beside the dense table, and the
+/// weight-gradient kernel reads the lists instead of the whole index.
+constexpr int32_t SLOT_MEAN_LIMIT = 32; // edges per sender on average
+bool lists_edges_in_slots(const Shape& s) {
+    return s.n_nodes > 0 && static_cast<size_t>(s.n_edges) <= static_cast<size_t>(s.n_nodes) * SLOT_MEAN_LIMIT;
+}
+
 size_t workspace_bytes(const Shape& s, size_t element_size) {
     return align256(dense_bytes(dense_layout(s), element_size)) +
-           (orders_edges_by_sender(s, element_size) ? edges_by_sender_bytes(s.n_nodes, s.n_edges) : 0);
+           (orders_edges_by_sender(s, element_size) ? edges_by_sender_bytes(s.n_nodes, s.n_edges)
+            : lists_edges_in_slots(s)               ? sender_slots_bytes(s.n_nodes)
+                                                    : 0);
 }
 
 template <typename T>
@@ -1229,10 +1383,12 @@ void vjp(
     const T* W, const Indices& indices, const Shape& s, void* workspace, hipStream_t stream
 ) {
     const DenseLayout layout = dense_layout(s);
-    const DenseBuffers<T> dense = enqueue_dense<T>(workspace, layout, C, indices, s, stream);
     const bool want_edges = grad_A != nullptr || grad_B != nullptr;
     const bool by_sender = grad_W != nullptr && orders_edges_by_sender(s, sizeof(T));
     void* order_workspace = static_cast<char*>(workspace) + align256(dense_bytes(layout, sizeof(T)));
+    const bool slotted = grad_W != nullptr && !by_sender && lists_edges_in_slots(s);
+    const SenderSlots slots = slotted ? sender_slots_in(order_workspace, s.n_nodes) : SenderSlots{nullptr, nullptr};
+    const DenseBuffers<T> dense = enqueue_dense<T>(workspace, layout, C, indices, s, stream, slotted ? &slots : nullptr);
 
     // large graphs: the forward kernel over the edges in the order of their senders
     auto launch_ordered_weights = [&](hipStream_t on, const EdgesBySender& order, int32_t first, const Shape& block) {
@@ -1270,13 +1426,14 @@ void vjp(
                 ));
             }
             kernel<<<grid, SENDERS_PER_GROUP * WAVE, lds, on>>>(
-                grad_W + first, indices.W_1, s.n_edges, aligned, c
+                grad_W + first, indices.W_1, s.n_edges, aligned, c, slots.edges, slots.counts
             );
         });
         MOPS_HIP_CHECK(hipGetLastError());
     };
 
-    auto launch_edges = [&](int32_t first, const Shape& block) {
+    // with_weights: grad_W of this block of columns in the same launch (needs the slots)
+    auto launch_edges = [&](int32_t first, const Shape& block, bool with_weights) {
         const bool vectors = block.L % 4 == 0 && s.L % 4 == 0 && aligned_for_vectors(W + first, sizeof(T));
         const int vec = vectors ? 4 : 1;
         EdgeGradArgs<T> args{};
@@ -1304,17 +1461,38 @@ void vjp(
         args.by_items = FastDivisor::make(s.n2 * block.L / vec);
         args.by_lvec = FastDivisor::make(block.L / vec);
         args.by_L = FastDivisor::make(block.L);
-        const int32_t grid = (s.n_edges + STAGE - 1) / STAGE;
-        const size_t lds = edge_gradients_lds(block, sizeof(T));
+        WeightGradArgs<T> weights{};
+        if (with_weights) {
+            weights.grad_W = grad_W + first;
+            weights.contraction = contraction<T>(
+                A, B + first, grad_output + first, indices.output_1, dense.to_cells, layout, block, s.L, s.n2,
+                s.n3, 1, s.n2
+            );
+            weights.slot_edges = slots.edges;
+            weights.slot_counts = slots.counts;
+            weights.n_senders = s.n_nodes;
+        }
+        const int32_t grid = (s.n_edges + STAGE - 1) / STAGE + weights.n_senders;
+        const size_t lds =
+            std::max(edge_gradients_lds(block, sizeof(T)), with_weights ? t_area_bytes(block, sizeof(T)) : 0);
         with_shape_constants(tiles_for(block.L), (s.n2 + 3) / 4, [&](auto tiles_constant, auto steps) {
-            auto kernel = edge_gradients_kernel<T, decltype(tiles_constant)::value, decltype(steps)::value>;
-            allow_lds(kernel, lds);
-            kernel<<<grid, WAVE, lds, stream>>>(args);
+            if (with_weights) {
+                auto kernel = edge_gradients_kernel<T, decltype(tiles_constant)::value, decltype(steps)::value, true>;
+                allow_lds(kernel, lds);
+                kernel<<<grid, WAVE, lds, stream>>>(args, weights);
+            } else {
+                auto kernel = edge_gradients_kernel<T, decltype(tiles_constant)::value, decltype(steps)::value, false>;
+                allow_lds(kernel, lds);
+                kernel<<<grid, WAVE, lds, stream>>>(args, weights);
+            }
         });
         MOPS_HIP_CHECK(hipGetLastError());
     };
 
-    if (want_edges && grad_W != nullptr) {
+    if (want_edges && slotted && (s.n2 + 3) / 4 == (s.n3 + 3) / 4) {
+        // sparse graphs: one launch for all three gradients
+        for_each_column_block(s, [&](int32_t first, const Shape& block) { launch_edges(first, block, true); });
+    } else if (want_edges && grad_W != nullptr) {
         // The two kernels are independent and both wait for memory most of
         // the time: they share the device, the weight kernel on a side stream
         // that forks from `stream` after the dense table and joins it again.
@@ -1330,10 +1508,10 @@ void vjp(
             } else {
                 launch_weights(side.get(), first, block);
             }
-            launch_edges(first, block);
+            launch_edges(first, block, false);
         });
     } else if (want_edges) {
-        for_each_column_block(s, launch_edges);
+        for_each_column_block(s, [&](int32_t first, const Shape& block) { launch_edges(first, block, false); });
     } else if (grad_W != nullptr) {
         EdgesBySender order{};
         if (by_sender) {

@@ -76,6 +76,10 @@ CASES = {
             support.sasaw_case(s, d, E=2300, nA=3, L=4, n_nodes=7, n2=2, n3=3, N=10), "indices_W_1"
         ),
         "mostly_empty": lambda s, d: support.sasaw_case(s, d, E=15, nA=3, L=5, n_nodes=200, n2=3, n3=2, N=7, allow_empty=True),
+        "sparse_with_hubs": lambda s, d: _with_sender_counts(
+            support.sasaw_case(s, d, E=6000, nA=4, L=8, n_nodes=300, n2=3, n3=5, N=40, allow_empty=True),
+            "indices_W_1", SENDER_COUNTS
+        ),
         "many_columns": lambda s, d: support.sasaw_case(s, d, E=500, nA=9, L=128, n_nodes=21, n2=9, n3=9, N=120, allow_empty=True),
         "ragged_columns": lambda s, d: support.sasaw_case(s, d, E=400, nA=4, L=70, n_nodes=17, n2=6, n3=11, N=80, allow_empty=True),
         "three_blocks": lambda s, d: support.sasaw_case(s, d, E=300, nA=16, L=164, n_nodes=40, n2=16, n3=16, N=300, allow_empty=True),
