@@ -147,6 +147,25 @@ __device__ __forceinline__ void list_in_slots_block(
             }
         }
     };
+    // four positions at once: the four places are asked for together, so that a
+    // thread waits for the LDS once and not four times
+    auto look4 = [&](const int4& values, int32_t edge) {
+        const int32_t which[4] = {values.x - node0, values.y - node0, values.z - node0, values.w - node0};
+        int32_t place[4];
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+            place[c] = SLOT_PART_CAPACITY;
+            if (in_bounds(which[c], served)) {
+                place[c] = atomicAdd(&lds.found[which[c]], 1);
+            }
+        }
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+            if (place[c] < SLOT_PART_CAPACITY) {
+                lds.edges[which[c]][place[c]] = edge + c;
+            }
+        }
+    };
     constexpr int AHEAD = 16;
     if (aligned) {
         // parts of whole groups of four; the last part also takes the n_edges % 4 edges after them
@@ -170,11 +189,7 @@ __device__ __forceinline__ void list_in_slots_block(
             }
 #pragma unroll
             for (int u = 0; u < AHEAD; u++) {
-                const int32_t edge = (g0 + u * THREADS + tid) << 2;
-                look(values[u].x, edge);
-                look(values[u].y, edge + 1);
-                look(values[u].z, edge + 2);
-                look(values[u].w, edge + 3);
+                look4(values[u], (g0 + u * THREADS + tid) << 2);
             }
         }
         const int32_t e = (n_edges & ~3) + tid;

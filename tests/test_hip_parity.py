@@ -61,6 +61,7 @@ CASES = {
         "sparse_with_hubs": lambda s, d: _with_sender_counts(
             support.opsaw_case(s, d, E=6000, K=4, L=32, n_nodes=300, allow_empty=True), "indices_W", SENDER_COUNTS
         ),
+        "sparse_tall": lambda s, d: support.opsaw_case(s, d, E=700, K=40, L=24, n_nodes=60, allow_empty=True),
         "pooling": lambda s, d: support.opsaw_case(s, d, E=5000, K=13, L=32, n_nodes=7),
         "pooling_mixed_lengths": lambda s, d: _with_lengths(
             support.opsaw_case(s, d, E=sum(MIXED_LENGTHS), K=3, L=17, n_nodes=len(MIXED_LENGTHS)), "indices_output", MIXED_LENGTHS
@@ -199,6 +200,29 @@ def test_vjp(oracle, device, op, name, dtype):
     actual = hip_vjp(op, to_device(case, device))
     for key in OPS[op].differentiable:
         assert_close(actual[key].cpu().numpy(), expected[key], dtype, f"{op}/{name} grad_{key}")
+
+
+@pytest.mark.parametrize("shift", [1, 2, 3])
+@pytest.mark.parametrize("op,key", [("opsaw", "indices_W"), ("sasaw", "indices_W_1")])
+def test_sender_index_off_the_vector_boundary(oracle, device, op, key, shift):
+    """The sender index starts 4, 8 or 12 bytes after a 16-byte boundary: the kernels that read
+    it 128 bits at a time must take their other way, with the same results."""
+    import torch
+
+    for name in ("ragged", "sparse_with_hubs"):
+        case = CASES[op][name](707, np.float32)
+        expected = cpu_vjp(oracle, op, case)
+        on_device = to_device(case, device)
+        index = on_device[key]
+        longer = torch.zeros(len(index) + 8, dtype=index.dtype, device=index.device)
+        base = (-longer.data_ptr() // 4) % 4  # elements up to the next 16-byte boundary
+        view = longer[base + shift : base + shift + len(index)]
+        view.copy_(index)
+        assert view.data_ptr() % 16 == 4 * shift
+        on_device[key] = view
+        actual = hip_vjp(op, on_device)
+        for gradient in OPS[op].differentiable:
+            assert_close(actual[gradient].cpu().numpy(), expected[gradient], np.float32, f"{op}/{name} grad_{gradient}")
 
 
 @pytest.mark.parametrize("op", list(OPS))
