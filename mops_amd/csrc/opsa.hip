@@ -1042,7 +1042,7 @@ __global__ __launch_bounds__(GATHER_SENDERS* WAVE) void sum_by_sender_kernel(
 // run beside the kernel that writes them (sender_buckets.hpp:
 // list_edges_in_slots): used while a sender has SLOT_MEAN_LIMIT edges or fewer
 // on average.
-constexpr int SLOT_MEAN_LIMIT = 32;
+constexpr int SLOT_MEAN_LIMIT = 48;
 
 // The sum over the slots: one wavefront per sender, ascending edge order, as
 // many rows in flight as 32 registers hold (COLUMNS values of a row per lane).

@@ -61,6 +61,7 @@ CASES = {
         "sparse_with_hubs": lambda s, d: _with_sender_counts(
             support.opsaw_case(s, d, E=6000, K=4, L=32, n_nodes=300, allow_empty=True), "indices_W", SENDER_COUNTS
         ),
+        "forty_five_per_sender": lambda s, d: support.opsaw_case(s, d, E=4500, K=6, L=32, n_nodes=100),
         "sparse_tall": lambda s, d: support.opsaw_case(s, d, E=700, K=40, L=24, n_nodes=60, allow_empty=True),
         "pooling": lambda s, d: support.opsaw_case(s, d, E=5000, K=13, L=32, n_nodes=7),
         "pooling_mixed_lengths": lambda s, d: _with_lengths(
@@ -81,6 +82,7 @@ CASES = {
             support.sasaw_case(s, d, E=6000, nA=4, L=8, n_nodes=300, n2=3, n3=5, N=40, allow_empty=True),
             "indices_W_1", SENDER_COUNTS
         ),
+        "forty_five_per_sender": lambda s, d: support.sasaw_case(s, d, E=2250, nA=4, L=16, n_nodes=50, n2=4, n3=3, N=30),
         "many_columns": lambda s, d: support.sasaw_case(s, d, E=500, nA=9, L=128, n_nodes=21, n2=9, n3=9, N=120, allow_empty=True),
         "ragged_columns": lambda s, d: support.sasaw_case(s, d, E=400, nA=4, L=70, n_nodes=17, n2=6, n3=11, N=80, allow_empty=True),
         "three_blocks": lambda s, d: support.sasaw_case(s, d, E=300, nA=16, L=164, n_nodes=40, n2=16, n3=16, N=300, allow_empty=True),
