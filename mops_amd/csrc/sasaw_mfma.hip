@@ -155,8 +155,8 @@ __global__ __launch_bounds__(DENSE_THREADS) void dense_coupling_kernel(
         );
         return;
     }
-    __shared__ int32_t keys[TABLE_TILE];
-    __shared__ T coefficients[TABLE_TILE];
+    __shared__ __align__(16) int32_t keys[TABLE_TILE];
+    __shared__ __align__(16) T coefficients[TABLE_TILE];
 
     const int tid = threadIdx.x;
     const int32_t slot = blockIdx.x * DENSE_THREADS + tid;
@@ -201,12 +201,26 @@ __global__ __launch_bounds__(DENSE_THREADS) void dense_coupling_kernel(
         // entries beyond N hold key -1 and match nothing
         const int32_t count = (min(TABLE_TILE, N - base) + 7) & ~7;
         for (int32_t i0 = 0; i0 < count; i0 += 8) {
+            // (all lanes read the same addresses: 16 bytes per LDS read)
             int32_t entry_key[8];
             T coefficient[8];
+            constexpr int PER_READ = 16 / sizeof(T);
+            typedef T Wide __attribute__((ext_vector_type(PER_READ)));
 #pragma unroll
-            for (int u = 0; u < 8; u++) {
-                entry_key[u] = keys[i0 + u];
-                coefficient[u] = coefficients[i0 + u];
+            for (int u = 0; u < 8; u += 4) {
+                const int4 four = *reinterpret_cast<const int4*>(&keys[i0 + u]);
+                entry_key[u] = four.x;
+                entry_key[u + 1] = four.y;
+                entry_key[u + 2] = four.z;
+                entry_key[u + 3] = four.w;
+            }
+#pragma unroll
+            for (int u = 0; u < 8; u += PER_READ) {
+                const Wide some = *reinterpret_cast<const Wide*>(&coefficients[i0 + u]);
+#pragma unroll
+                for (int c = 0; c < PER_READ; c++) {
+                    coefficient[u + c] = some[c];
+                }
             }
 #pragma unroll
             for (int u = 0; u < 8; u++) {
