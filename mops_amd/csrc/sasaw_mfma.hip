@@ -824,8 +824,10 @@ template <typename T> struct EdgeGradArgs {
 constexpr int EDGE_BATCH = 2; // edges whose W blocks are in LDS together (4: more LDS and registers
                               // per wavefront, 98 instead of 89 us for the whole vjp; 1: 112 us)
 
-/// grad_W in the same launch (WITH_WEIGHTS): the first `n_senders` workgroups
-/// are one sender each (weight_gradient_of_sender), the others 16 edges each.
+/// grad_W in the same launch (WITH_WEIGHTS): the workgroups after those of the
+/// edges (16 edges each) are one sender each (weight_gradient_of_sender): the
+/// short jobs last, where they fill the places the long ones leave as they end
+/// (the other order: 74 instead of 70 us in f32, 132 instead of 122 in f64).
 /// The two halves of a vjp do not depend on each other and both wait for
 /// memory most of the time; as one launch they share the device without a
 /// second stream (forking and joining streams costs about 10 us per call,
@@ -853,10 +855,11 @@ __global__ __launch_bounds__(WAVE) void edge_gradients_kernel(const EdgeGradArgs
     const int lane = threadIdx.x;
     if constexpr (WITH_WEIGHTS) {
         // (M2S steps of four cover n3 as well as n2 here: the host sees to it)
-        if (static_cast<int32_t>(blockIdx.x) < w.n_senders) {
+        const int32_t edge_blocks = (p.n_edges + STAGE - 1) / STAGE;
+        if (static_cast<int32_t>(blockIdx.x) >= edge_blocks) {
             weight_gradient_of_sender<T, NT, M2S>(
                 w.grad_W, p.senders, p.n_edges, w.contraction, w.slot_edges, w.slot_counts,
-                static_cast<int32_t>(blockIdx.x), t_area, lane
+                static_cast<int32_t>(blockIdx.x) - edge_blocks, t_area, lane
             );
             return;
         }
@@ -866,7 +869,7 @@ __global__ __launch_bounds__(WAVE) void edge_gradients_kernel(const EdgeGradArgs
     const bool want_A = p.grad_A != nullptr;
     const bool want_B = p.grad_B != nullptr;
 
-    const int32_t chunk_begin = (static_cast<int32_t>(blockIdx.x) - (WITH_WEIGHTS ? w.n_senders : 0)) * STAGE;
+    const int32_t chunk_begin = static_cast<int32_t>(blockIdx.x) * STAGE;
     const int32_t n = min(STAGE, p.n_edges - chunk_begin);
     const int32_t my_edge = i < n ? chunk_begin + i : -1;
     const int32_t my_source = my_edge >= 0 ? p.senders[my_edge] : -1;
