@@ -78,6 +78,22 @@ MOPS_EXPORT int mops_amd_kernel_time(double* total_milliseconds, int64_t* launch
  * than 0). Returns the previous setting. */
 MOPS_EXPORT int mops_amd_accept_unsorted_indices(int accept);
 
+/* Scratch memory and HIP graphs.
+ *
+ * Some calls need temporary device memory (lists of the edges of every
+ * sender, partial sums of very long segments). Each calling thread keeps one
+ * block for it, which grows when a call needs more. Growing allocates, which
+ * is not possible while the thread's stream is being captured into a graph: a
+ * mops_cuda_* call that would have to grow the block during a capture fails
+ * with status 1 and a message that says so. Before capturing, either make one
+ * eager call with the largest shapes, or reserve the memory here.
+ * mops_amd_reserve_scratch makes the calling thread's block at least `bytes`
+ * large (0 / 1 / 2); mops_amd_scratch_capacity returns its present size.
+ * A block that was used during a capture is never freed (a graph that was
+ * captured may replay kernels that name it). */
+MOPS_EXPORT int mops_amd_reserve_scratch(int64_t bytes);
+MOPS_EXPORT int64_t mops_amd_scratch_capacity(void);
+
 #ifdef __cplusplus
 }
 #endif

@@ -146,3 +146,14 @@ extern "C" int mops_amd_kernel_time(double* total_milliseconds, int64_t* launche
     mops::amd::collect_kernel_time(total_milliseconds, launches);
     MOPS_CATCH_EXCEPTIONS_END
 }
+
+extern "C" int mops_amd_reserve_scratch(int64_t bytes) {
+    MOPS_CATCH_EXCEPTIONS_BEGIN
+    (void)mops::amd::scratch(extent(bytes));
+    mops::amd::finish_call("reserve_scratch");
+    MOPS_CATCH_EXCEPTIONS_END
+}
+
+extern "C" int64_t mops_amd_scratch_capacity(void) {
+    return static_cast<int64_t>(mops::amd::scratch_capacity());
+}

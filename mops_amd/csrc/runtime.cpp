@@ -2,6 +2,7 @@
 
 #include <cstdlib>
 #include <limits>
+#include <mutex>
 #include <utility>
 #include <vector>
 
@@ -17,15 +18,21 @@ void check_hip(hipError_t status, const char* what) {
 
 namespace {
 
-struct ThreadState {
-    hipStream_t stream = nullptr;
-    bool synchronous = true;
-
+// Device objects of one calling thread. They outlive the thread: when it ends
+// they go to a process-wide pool (no HIP call is made from a thread's exit
+// path, where the HIP runtime may already be gone) and the next new thread
+// takes them over, so short-lived worker threads do not leak device memory.
+struct Resources {
     // scratch cache
     void* block = nullptr;
     size_t capacity = 0;
     int device = -1;
-    hipStream_t block_stream = nullptr;
+    hipStream_t block_stream = nullptr; // stream of the block's latest user
+    bool block_in_graph = false;        // handed out while a stream was being captured
+    hipEvent_t last_use = nullptr;      // recorded behind the latest eager call that used the block
+    bool last_use_recorded = false;
+    // blocks a captured graph may still name: kept until the process ends
+    std::vector<void*> retired;
 
     // side stream and its two events, per device
     struct Side {
@@ -36,16 +43,67 @@ struct ThreadState {
     };
     std::vector<Side> sides;
 
-    // kernel timing
-    bool timing = false;
-    std::vector<std::pair<hipEvent_t, hipEvent_t>> recorded;
+    // timing events
     std::vector<hipEvent_t> spare;
 };
 
+struct Pool {
+    std::mutex mutex;
+    std::vector<Resources*> idle;
+};
+
+Pool& pool() {
+    static Pool* instance = new Pool(); // never destroyed: threads may end after main returns
+    return *instance;
+}
+
+struct ThreadState {
+    hipStream_t stream = nullptr;
+    bool synchronous = true;
+    Resources* resources = nullptr;
+
+    // this call
+    bool used_scratch = false;
+    bool capturing = false;
+
+    // kernel timing
+    bool timing = false;
+    std::vector<std::pair<hipEvent_t, hipEvent_t>> recorded;
+
+    Resources& res() {
+        if (resources == nullptr) {
+            Pool& p = pool();
+            std::lock_guard<std::mutex> lock(p.mutex);
+            if (!p.idle.empty()) {
+                resources = p.idle.back();
+                p.idle.pop_back();
+            }
+        }
+        if (resources == nullptr) {
+            resources = new Resources();
+        }
+        return *resources;
+    }
+
+    ~ThreadState() {
+        if (resources == nullptr) {
+            return;
+        }
+        for (auto& pair : recorded) {
+            resources->spare.push_back(pair.first);
+            resources->spare.push_back(pair.second);
+        }
+        Pool& p = pool();
+        std::lock_guard<std::mutex> lock(p.mutex);
+        p.idle.push_back(resources);
+    }
+};
+
 hipEvent_t take_event(ThreadState& st) {
-    if (!st.spare.empty()) {
-        hipEvent_t event = st.spare.back();
-        st.spare.pop_back();
+    auto& spare = st.res().spare;
+    if (!spare.empty()) {
+        hipEvent_t event = spare.back();
+        spare.pop_back();
         return event;
     }
     hipEvent_t event = nullptr;
@@ -54,10 +112,14 @@ hipEvent_t take_event(ThreadState& st) {
 }
 
 ThreadState& state() {
-    // Deliberately never destroyed: at thread or process exit the HIP runtime
-    // may already be gone, and freeing device memory then would fault.
-    static thread_local ThreadState* instance = new ThreadState();
-    return *instance;
+    static thread_local ThreadState instance;
+    return instance;
+}
+
+bool is_capturing(hipStream_t stream) {
+    hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+    MOPS_HIP_CHECK(hipStreamIsCapturing(stream, &capture));
+    return capture != hipStreamCaptureStatusNone;
 }
 
 } // namespace
@@ -77,6 +139,19 @@ bool set_synchronous(bool value) {
 void finish_call(const char* operation) {
     check_hip(hipGetLastError(), operation);
     auto& st = state();
+    if (st.used_scratch) {
+        // so that another stream (of this thread later, or of the thread that
+        // inherits the block) can wait for this call without the host waiting
+        st.used_scratch = false;
+        Resources& res = st.res();
+        if (!st.capturing) {
+            if (res.last_use == nullptr) {
+                check_hip(hipEventCreateWithFlags(&res.last_use, hipEventDisableTiming), operation);
+            }
+            check_hip(hipEventRecord(res.last_use, st.stream), operation);
+            res.last_use_recorded = true;
+        }
+    }
     if (st.synchronous) {
         check_hip(hipStreamSynchronize(st.stream), operation);
     }
@@ -86,19 +161,20 @@ SideStream::SideStream(hipStream_t main) : main_(main) {
     auto& st = state();
     int device = 0;
     MOPS_HIP_CHECK(hipGetDevice(&device));
-    ThreadState::Side* side = nullptr;
-    for (auto& candidate : st.sides) {
+    Resources::Side* side = nullptr;
+    auto& sides = st.res().sides;
+    for (auto& candidate : sides) {
         if (candidate.device == device) {
             side = &candidate;
         }
     }
     if (side == nullptr) {
-        ThreadState::Side created{device, nullptr, nullptr, nullptr};
+        Resources::Side created{device, nullptr, nullptr, nullptr};
         MOPS_HIP_CHECK(hipStreamCreateWithFlags(&created.stream, hipStreamNonBlocking));
         MOPS_HIP_CHECK(hipEventCreateWithFlags(&created.forked, hipEventDisableTiming));
         MOPS_HIP_CHECK(hipEventCreateWithFlags(&created.joined, hipEventDisableTiming));
-        st.sides.push_back(created);
-        side = &st.sides.back();
+        sides.push_back(created);
+        side = &sides.back();
     }
     side_ = side->stream;
     joined_ = side->joined;
@@ -117,9 +193,7 @@ MainKernelTimer::MainKernelTimer(hipStream_t stream) : stream_(stream) {
     if (!st.timing) {
         return;
     }
-    hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
-    MOPS_HIP_CHECK(hipStreamIsCapturing(stream, &capture));
-    if (capture != hipStreamCaptureStatusNone) {
+    if (is_capturing(stream)) {
         return;
     }
     hipEvent_t start = take_event(st);
@@ -140,9 +214,7 @@ LaunchEvents launch_events(hipStream_t stream) {
     if (!st.timing) {
         return events;
     }
-    hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
-    MOPS_HIP_CHECK(hipStreamIsCapturing(stream, &capture));
-    if (capture != hipStreamCaptureStatusNone) {
+    if (is_capturing(stream)) {
         return events;
     }
     events.start = take_event(st);
@@ -165,8 +237,8 @@ void collect_kernel_time(double* milliseconds, int64_t* launches) {
         float elapsed = 0.0f;
         MOPS_HIP_CHECK(hipEventElapsedTime(&elapsed, pair.first, pair.second));
         total += elapsed;
-        st.spare.push_back(pair.first);
-        st.spare.push_back(pair.second);
+        st.res().spare.push_back(pair.first);
+        st.res().spare.push_back(pair.second);
     }
     *milliseconds = total;
     *launches = static_cast<int64_t>(st.recorded.size());
@@ -175,49 +247,70 @@ void collect_kernel_time(double* milliseconds, int64_t* launches) {
 
 void* scratch(size_t bytes) {
     auto& st = state();
+    Resources& res = st.res();
     int device = 0;
     MOPS_HIP_CHECK(hipGetDevice(&device));
+    // st.stream is the stream of this call: the caller named it and keeps it alive
+    st.capturing = is_capturing(st.stream);
 
-    if (st.block != nullptr && (device != st.device || bytes > st.capacity)) {
-        // hipFree waits for the device, so nothing can still be using the block
-        int restore = device;
-        MOPS_HIP_CHECK(hipSetDevice(st.device));
-        MOPS_HIP_CHECK(hipFree(st.block));
-        MOPS_HIP_CHECK(hipSetDevice(restore));
-        st.block = nullptr;
-        st.capacity = 0;
+    if (res.block != nullptr && (device != res.device || bytes > res.capacity)) {
+        if (st.capturing) {
+            // Allocating would end the capture, and the graph would keep the
+            // address of a block that the next growth frees.
+            throw std::runtime_error(
+                "mops: this call needs " + std::to_string(bytes) + " bytes of scratch memory but the calling "
+                "thread holds " + std::to_string(res.capacity) + " and its stream is being captured into a graph; "
+                "make one call with the largest shapes on this thread before capturing"
+            );
+        }
+        if (res.block_in_graph) {
+            // a captured graph may replay kernels that name this block
+            res.retired.push_back(res.block);
+        } else {
+            // hipFree waits for the device, so nothing can still be using the block
+            int restore = device;
+            MOPS_HIP_CHECK(hipSetDevice(res.device));
+            MOPS_HIP_CHECK(hipFree(res.block));
+            MOPS_HIP_CHECK(hipSetDevice(restore));
+        }
+        res.block = nullptr;
+        res.capacity = 0;
+        res.block_in_graph = false;
+        res.last_use_recorded = false;
     }
 
-    if (st.block == nullptr) {
+    if (res.block == nullptr) {
+        if (st.capturing) {
+            throw std::runtime_error(
+                "mops: this call needs scratch memory and the calling thread has none yet, but its stream is being "
+                "captured into a graph; make one call with the largest shapes on this thread before capturing"
+            );
+        }
         size_t capacity = bytes + bytes / 2;
         if (capacity < (size_t(1) << 20)) {
             capacity = size_t(1) << 20;
         }
-        MOPS_HIP_CHECK(hipMalloc(&st.block, capacity));
-        st.capacity = capacity;
-        st.device = device;
-        st.block_stream = st.stream;
-    } else if (st.block_stream != st.stream) {
-        // The previous user of the block ran on another stream: let it finish
-        // before this stream overwrites the block. Streams that are being
-        // captured into a graph cannot be waited for (and their work does not
-        // run now anyway); ordering graph replays is the caller's business.
-        hipStreamCaptureStatus previous = hipStreamCaptureStatusNone;
-        hipStreamCaptureStatus next = hipStreamCaptureStatusNone;
-        // the previous stream may have been destroyed by its owner meanwhile:
-        // then there is nothing left to wait for
-        bool previous_alive = hipStreamIsCapturing(st.block_stream, &previous) == hipSuccess;
-        if (!previous_alive) {
-            (void)hipGetLastError();
-        }
-        MOPS_HIP_CHECK(hipStreamIsCapturing(st.stream, &next));
-        if (previous_alive && previous == hipStreamCaptureStatusNone &&
-            next == hipStreamCaptureStatusNone) {
-            MOPS_HIP_CHECK(hipStreamSynchronize(st.block_stream));
-        }
-        st.block_stream = st.stream;
+        MOPS_HIP_CHECK(hipMalloc(&res.block, capacity));
+        res.capacity = capacity;
+        res.device = device;
+    } else if (res.block_stream != st.stream && res.last_use_recorded && !st.capturing) {
+        // The previous user of the block ran on another stream: this stream
+        // waits (on the device, not the host) for the event recorded behind
+        // it. The previous stream itself is not touched: its owner may have
+        // destroyed it. A stream that is being captured cannot wait for an
+        // event outside its graph, and its work does not run now anyway;
+        // ordering graph replays against eager calls is the caller's business.
+        MOPS_HIP_CHECK(hipStreamWaitEvent(st.stream, res.last_use, 0));
     }
-    return st.block;
+    res.block_stream = st.stream;
+    res.block_in_graph = res.block_in_graph || st.capturing;
+    st.used_scratch = true;
+    return res.block;
+}
+
+size_t scratch_capacity() {
+    auto& st = state();
+    return st.resources == nullptr ? 0 : st.resources->capacity;
 }
 
 int32_t narrow_i32(size_t value, const char* what) {

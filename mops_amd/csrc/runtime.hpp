@@ -37,10 +37,16 @@ void finish_call(const char* operation);
 /// Scratch device memory of at least `bytes` bytes, 256-byte aligned, valid
 /// until the next call of this function on the same thread. The block is
 /// cached per thread and grows on demand (growing frees the old block, which
-/// waits for the device); when the calling thread switches to another stream
-/// the previous stream is drained first, so two streams never share the
-/// block at the same time.
+/// waits for the device; a block that was handed out while a stream was being
+/// captured is kept until the process ends instead, because the graph names
+/// it). Growing while the thread's stream is being captured throws. When the
+/// calling thread switches to another stream, the new stream waits on the
+/// device for the previous call that used the block, so two streams never
+/// share the block at the same time. A thread that ends leaves its block to
+/// the next new thread.
 void* scratch(size_t bytes);
+/// Bytes of the calling thread's scratch block (0: none yet).
+size_t scratch_capacity();
 
 /// A second stream of the calling thread, for a kernel of a call that does not
 /// depend on the call's other kernels and leaves room on the device beside

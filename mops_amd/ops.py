@@ -11,15 +11,32 @@ Device tensors go to the ``mops_cuda_*`` entry points, which run on the
 current PyTorch stream of the tensors' device without blocking the host.
 """
 from . import _dispatch
+from ._c_api import SIGNATURES
 from ._c_lib import device_library, host_library
 from .checks import check_arguments, check_scalar
 
 
 def _call(function, reference, tensors):
     """Invoke ``function`` with ``tensors`` in ABI order on the right device."""
+    names = [name for _, name in SIGNATURES[function]]
     if _dispatch.on_device(reference):
         import torch
 
+        # A host pointer handed to a device kernel is a memory fault, not an
+        # exception: refuse anything that does not live where `reference` does.
+        for name, tensor in zip(names, tensors):
+            if tensor is None:
+                continue
+            if not _dispatch.is_torch(tensor):
+                raise TypeError(
+                    f"`{name}` must be a torch tensor on {reference.device} in {function} "
+                    f"(the first tensor is there), got {type(tensor)}"
+                )
+            if tensor.device != reference.device:
+                raise ValueError(
+                    f"`{name}` is on {tensor.device} but the first tensor is on "
+                    f"{reference.device} in {function}: all tensors must be on the same device"
+                )
         library = device_library()
         with torch.cuda.device(reference.device):
             stream = torch.cuda.current_stream(reference.device)
@@ -27,6 +44,12 @@ def _call(function, reference, tensors):
             library.cdll.mops_amd_set_synchronous(0)
             library.call(function, *tensors)
     else:
+        for name, tensor in zip(names, tensors):
+            if tensor is not None and _dispatch.on_device(tensor):
+                raise ValueError(
+                    f"`{name}` is on {tensor.device} but the first tensor is in host memory "
+                    f"in {function}: all tensors must be on the same device"
+                )
         host_library().call(function, *tensors)
 
 

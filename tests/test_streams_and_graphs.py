@@ -5,6 +5,7 @@ thread) and, in asynchronous mode, neither allocates nor synchronises once its
 scratch block has its size, so a call can be captured; SASAW's vjp forks to a
 side stream and joins again inside the call, which a capture has to follow.
 """
+import ctypes
 import threading
 
 import numpy as np
@@ -80,23 +81,29 @@ def test_graph_replays_match_eager_calls(device, op):
             assert torch.equal(again, want), (op, replay)
 
 
-def test_two_host_threads_on_their_own_streams(device):
-    """The per-thread state (stream, scratch block, error message) keeps two callers apart."""
+def test_two_host_threads_on_their_own_streams(oracle, device):
+    """Two host threads, each on a stream of its own, call different operations at the same time:
+    the per-thread state (stream, scratch block, error message) keeps them apart, and both get
+    the oracle's results."""
     results = {}
     errors = []
+    ready = threading.Barrier(2)
 
     def worker(op):
         try:
-            case = support.to_device(CASES[op](np.float32), device)
+            host_case = CASES[op](np.float32)
+            case = support.to_device(host_case, device)
             stream = torch.cuda.Stream(device=device)
+            ready.wait()
             with torch.cuda.stream(stream):
                 first = [t.clone() for t in _call(op, case)]
                 for _ in range(20):
                     again = _call(op, case)
                 stream.synchronize()
-                results[op] = all(torch.equal(a, b) for a, b in zip(first, again))
+            results[op] = (host_case, first, all(torch.equal(a, b) for a, b in zip(first, again)))
         except Exception as error:  # pragma: no cover - reported below
             errors.append((op, repr(error)))
+            ready.abort()
 
     threads = [threading.Thread(target=worker, args=(op,)) for op in ("opsaw", "sasaw")]
     for thread in threads:
@@ -104,4 +111,108 @@ def test_two_host_threads_on_their_own_streams(device):
     for thread in threads:
         thread.join()
     assert not errors, errors
-    assert results == {"opsaw": True, "sasaw": True}
+    for op in ("opsaw", "sasaw"):
+        host_case, first, repeatable = results[op]
+        assert repeatable, op
+        spec = OPS[op]
+        support.assert_close(first[0].cpu().numpy(), support.cpu_forward(oracle, op, host_case), np.float32, op)
+        expected = support.cpu_vjp(oracle, op, host_case)
+        for name, got in zip(spec.differentiable, first[1:]):
+            support.assert_close(got.cpu().numpy(), expected[name], np.float32, f"{op} grad_{name}")
+
+
+def test_threads_that_end_hand_their_scratch_block_on(device):
+    """A thread's scratch block goes to the next new thread instead of being lost."""
+    from mops_amd._c_lib import device_library
+
+    library = device_library()
+    library.cdll.mops_amd_scratch_capacity.restype = ctypes.c_int64
+    library.cdll.mops_amd_reserve_scratch.argtypes = [ctypes.c_int64]
+    seen = []
+
+    def worker(reserve):
+        torch.cuda.set_device(device)
+        if reserve:
+            assert library.cdll.mops_amd_reserve_scratch(3 << 20) == 0
+        else:
+            # the first use of the state takes over what an ended thread left
+            assert library.cdll.mops_amd_reserve_scratch(1) == 0
+        seen.append(library.cdll.mops_amd_scratch_capacity())
+
+    for reserve in (True, False):
+        thread = threading.Thread(target=worker, args=(reserve,))
+        thread.start()
+        thread.join()
+    assert seen[0] >= 3 << 20
+    assert seen[1] == seen[0]
+
+
+def test_growing_the_scratch_block_during_a_capture_is_refused(device):
+    """No allocation can happen while a stream is being captured: the call fails with a message
+    instead (a host-side check; nothing is launched)."""
+    from mops_amd._c_lib import device_library
+
+    library = device_library()
+    library.cdll.mops_amd_scratch_capacity.restype = ctypes.c_int64
+    library.cdll.mops_amd_reserve_scratch.argtypes = [ctypes.c_int64]
+    torch.cuda.set_device(device)
+    library.cdll.mops_amd_set_stream(torch.cuda.current_stream(device).cuda_stream)
+    assert library.cdll.mops_amd_reserve_scratch(1) == 0
+    capacity = library.cdll.mops_amd_scratch_capacity()
+    assert capacity >= 1 << 20
+
+    marker = torch.zeros(16, device=device)
+    stream = torch.cuda.Stream(device=device)
+    stream.wait_stream(torch.cuda.current_stream(device))
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(stream):
+        with torch.cuda.graph(graph, stream=stream):
+            library.cdll.mops_amd_set_stream(stream.cuda_stream)
+            library.cdll.mops_amd_set_synchronous(0)
+            marker.add_(1.0)
+            within = library.cdll.mops_amd_reserve_scratch(capacity)  # fits: fine during a capture
+            status = library.cdll.mops_amd_reserve_scratch(4 * capacity)
+            message = library.last_error()
+    library.cdll.mops_amd_set_stream(torch.cuda.current_stream(device).cuda_stream)
+    assert within == 0
+    assert status == 1
+    assert "being captured" in message and "before capturing" in message
+    assert library.cdll.mops_amd_scratch_capacity() == capacity  # untouched
+    graph.replay()
+    torch.cuda.synchronize()
+    assert float(marker[0]) == 1.0
+
+
+def test_a_block_that_a_graph_names_outlives_a_later_growth(device):
+    """Eager calls with larger shapes after a capture must not free the block the graph uses."""
+    from mops_amd._c_lib import device_library
+
+    library = device_library()
+    library.cdll.mops_amd_scratch_capacity.restype = ctypes.c_int64
+    library.cdll.mops_amd_reserve_scratch.argtypes = [ctypes.c_int64]
+    op = "opsa_pooling"  # pieces of long segments meet in scratch memory
+    case = support.to_device(CASES[op](np.float32), device)
+    eager = [t.clone() for t in _call(op, case)]
+    torch.cuda.synchronize()
+    stream = torch.cuda.Stream(device=device)
+    stream.wait_stream(torch.cuda.current_stream(device))
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(stream):
+        _call(op, case)
+        torch.cuda.synchronize()
+        with torch.cuda.graph(graph, stream=stream):
+            captured = _call(op, case)
+    torch.cuda.synchronize()
+    library.cdll.mops_amd_set_stream(torch.cuda.current_stream(device).cuda_stream)
+    before = library.cdll.mops_amd_scratch_capacity()
+    assert library.cdll.mops_amd_reserve_scratch(8 * before) == 0  # grows: the old block is kept
+    assert library.cdll.mops_amd_scratch_capacity() >= 8 * before
+    filler = torch.full((before // 4,), float("nan"), device=device)  # would land in a freed block
+    for tensor in captured:
+        tensor.fill_(float("nan"))
+    torch.cuda.synchronize()
+    graph.replay()
+    torch.cuda.synchronize()
+    for got, want in zip(captured, eager):
+        assert torch.equal(got, want)
+    del filler

@@ -133,24 +133,67 @@ def test_operator_second_derivatives(oracle, device, op):
     assert torch.autograd.gradgradcheck(operator, arguments(op, on_device), fast_mode=True)
 
 
+class ScriptedHpe(torch.nn.Module):
+    def forward(self, A, C, indices_A):
+        return torch.ops.mops.homogeneous_polynomial_evaluation(A, C, indices_A)
+
+
+class ScriptedSap(torch.nn.Module):
+    def forward(self, A, B, C, indices_A, indices_B, indices_output, output_size: int):
+        return torch.ops.mops.sparse_accumulation_of_products(
+            A, B, C, indices_A, indices_B, indices_output, output_size
+        )
+
+
+class ScriptedOpsa(torch.nn.Module):
+    def forward(self, A, B, indices_output, output_size: int):
+        return torch.ops.mops.outer_product_scatter_add(A, B, indices_output, output_size)
+
+
+class ScriptedOpsaw(torch.nn.Module):
+    def forward(self, A, B, W, indices_W, indices_output):
+        return torch.ops.mops.outer_product_scatter_add_with_weights(A, B, W, indices_W, indices_output)
+
+
+class ScriptedSasaw(torch.nn.Module):
+    def forward(
+        self, A, B, C, W, indices_A, indices_W_1, indices_W_2, indices_output_1, indices_output_2, output_size: int
+    ):
+        return torch.ops.mops.sparse_accumulation_scatter_add_with_weights(
+            A, B, C, W, indices_A, indices_W_1, indices_W_2, indices_output_1, indices_output_2, output_size
+        )
+
+
+SCRIPTED = {"hpe": ScriptedHpe, "sap": ScriptedSap, "opsa": ScriptedOpsa, "opsaw": ScriptedOpsaw, "sasaw": ScriptedSasaw}
+
+
+@pytest.mark.parametrize("op", list(SCRIPTED))
+def test_modules_can_be_scripted(op):
+    """Scripting resolves the operator against its schema (no GPU needed), as
+    python/mops-torch/tests/torchscript.py:7-260 of the reference does for every operation."""
+    scripted = torch.jit.script(SCRIPTED[op]())
+    assert "mops::" + support.OPS[op].function in str(scripted.graph)
+
+
 @pytest.mark.gpu
-def test_torchscript_save_and_load(oracle, device, tmp_path):
-    """A scripted module that calls the operators survives save / load, as in the reference's
-    python/mops-torch/tests/torchscript.py."""
-
-    class Model(torch.nn.Module):
-        def forward(self, A, B, indices_output, output_size: int):
-            return torch.ops.mops.outer_product_scatter_add(A, B, indices_output, output_size)
-
-    case = SMALL["opsa"](np.float64)
+@pytest.mark.parametrize("op", list(SCRIPTED))
+def test_torchscript_save_and_load(oracle, device, tmp_path, op):
+    """A scripted module of every operation survives save / load and gives the oracle's values
+    and gradients."""
+    case = SMALL[op](np.float64)
     on_device = support.to_device(case, device)
-    scripted = torch.jit.script(Model())
-    path = str(tmp_path / "model.pt")
+    spec = support.OPS[op]
+    scripted = torch.jit.script(SCRIPTED[op]())
+    path = str(tmp_path / f"{op}.pt")
     scripted.save(path)
     loaded = torch.jit.load(path)
-    actual = loaded(*arguments("opsa", on_device))
-    support.assert_close(actual.cpu().numpy(), support.cpu_forward(oracle, "opsa", case), np.float64, "scripted opsa")
-    on_device["A"].requires_grad_(True)
-    loaded(*arguments("opsa", on_device)).backward(on_device["grad_output"])
-    expected = support.cpu_vjp(oracle, "opsa", case, wanted=["A"])["A"]
-    support.assert_close(on_device["A"].grad.cpu().numpy(), expected, np.float64, "scripted opsa grad_A")
+    actual = loaded(*arguments(op, on_device))
+    support.assert_close(actual.cpu().numpy(), support.cpu_forward(oracle, op, case), np.float64, f"scripted {op}")
+    for name in spec.differentiable:
+        on_device[name].requires_grad_(True)
+    loaded(*arguments(op, on_device)).backward(on_device["grad_output"])
+    expected = support.cpu_vjp(oracle, op, case)
+    for name in spec.differentiable:
+        support.assert_close(
+            on_device[name].grad.cpu().numpy(), expected[name], np.float64, f"scripted {op} grad_{name}"
+        )
