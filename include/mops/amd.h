@@ -15,6 +15,7 @@
 #include <stdint.h>
 
 #include "mops/exports.h"
+#include "mops/tensor.h"
 
 #ifdef __cplusplus
 extern "C" {
@@ -93,6 +94,41 @@ MOPS_EXPORT int mops_amd_accept_unsorted_indices(int accept);
  * captured may replay kernels that name it). */
 MOPS_EXPORT int mops_amd_reserve_scratch(int64_t bytes);
 MOPS_EXPORT int64_t mops_amd_scratch_capacity(void);
+
+/* The entry point that allocates nothing.
+ *
+ * No counterpart in lab-cosmo/mops. It is for callers that cannot allocate
+ * device memory: code under HIP graph capture, tight serving loops, harnesses
+ * that forbid hipMalloc. Same arguments, checks, results (bit for bit) and
+ * return convention as
+ * mops_cuda_sparse_accumulation_scatter_add_with_weights_vjp_f32, but the
+ * temporaries of its kernels (the dense coupling table and the list of every
+ * sender's edges) live in an array of 4 MiB that is part of the library's
+ * device code, one copy per GPU, held until the process ends; the call makes
+ * no hipMalloc / hipFree and creates no stream or event. Limits, reported as
+ * status 1 with a message: A.shape[1], W.shape[1], output.shape[1] in 1..16;
+ * temporaries within 4 MiB (about 7800 nodes); when grad_W is asked for
+ * together with grad_A or grad_B, at most 48 edges per node on average and
+ * W.shape[1], output.shape[1] in the same multiple of four; indices_output_1
+ * sorted (mops_amd_accept_unsorted_indices does not apply). All calls on one
+ * GPU share the array: calls that overlap on one GPU (two streams, two
+ * threads) race; the caller serialises them. Nothing in the array needs to be
+ * zero at entry. Runs on the calling thread's stream (mops_amd_set_stream). */
+MOPS_EXPORT int mops_amd_sparse_accumulation_scatter_add_with_weights_vjp_no_alloc_f32(
+    mops_tensor_2d_f32_t grad_A,
+    mops_tensor_2d_f32_t grad_B,
+    mops_tensor_3d_f32_t grad_W,
+    mops_tensor_3d_f32_t grad_output,
+    mops_tensor_2d_f32_t A,
+    mops_tensor_2d_f32_t B,
+    mops_tensor_1d_f32_t C,
+    mops_tensor_3d_f32_t W,
+    mops_tensor_1d_i32_t indices_A,
+    mops_tensor_1d_i32_t indices_W_1,
+    mops_tensor_1d_i32_t indices_W_2,
+    mops_tensor_1d_i32_t indices_output_1,
+    mops_tensor_1d_i32_t indices_output_2
+);
 
 #ifdef __cplusplus
 }

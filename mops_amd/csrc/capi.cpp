@@ -13,6 +13,7 @@
 #include "mops.hpp"
 
 #include "first_occurrences.hpp"
+#include "no_alloc.hpp"
 #include "edge_order.hpp"
 #include "runtime.hpp"
 
@@ -156,4 +157,12 @@ extern "C" int mops_amd_reserve_scratch(int64_t bytes) {
 
 extern "C" int64_t mops_amd_scratch_capacity(void) {
     return static_cast<int64_t>(mops::amd::scratch_capacity());
+}
+
+extern "C" int mops_amd_sparse_accumulation_scatter_add_with_weights_vjp_no_alloc_f32(
+    MOPS_SASAW_VJP_PARAMS(MOPS_C_FIRST_f32, MOPS_C_NEXT_f32)
+) {
+    MOPS_CATCH_EXCEPTIONS_BEGIN
+    mops::amd::sasaw_vjp_no_alloc(MOPS_SASAW_VJP_PARAMS(MOPS_FORWARD_FIRST, MOPS_FORWARD_NEXT));
+    MOPS_CATCH_EXCEPTIONS_END
 }

@@ -37,6 +37,9 @@
 // The reference has no device implementation of this operation
 // (mops/src/sasaw/sasaw.cu:1, mops/src/sasaw/cuda.tpp:18).
 #include <algorithm>
+#include <atomic>
+#include <stdexcept>
+#include <string>
 
 #include "mops/sasaw.hpp"
 
@@ -44,6 +47,7 @@
 #include "device_common.hpp"
 #include "first_occurrences.hpp"
 #include "index_validation.hpp"
+#include "no_alloc.hpp"
 #include "edge_order.hpp"
 #include "runtime.hpp"
 #include "sasaw_mfma.hpp"
@@ -802,3 +806,106 @@ MOPS_CXX_INSTANTIATE(sparse_accumulation_scatter_add_with_weights_vjp, MOPS_SASA
 MOPS_CXX_INSTANTIATE(sparse_accumulation_scatter_add_with_weights_vjp_vjp, MOPS_SASAW_VJP_VJP_PARAMS)
 
 } // namespace mops::cuda
+
+// ---------------------------------------------------------------------------
+// the entry point that allocates nothing
+
+namespace mops::amd {
+namespace {
+
+// Temporary memory of the no-allocation entry point: part of the code object,
+// so every GPU the library runs on holds its own copy from the moment the
+// code object is loaded there until the process ends. In host code this name
+// is only a handle for hipGetSymbolAddress, never an address.
+static __device__ __align__(256) unsigned char no_alloc_scratch[NO_ALLOC_SCRATCH_BYTES];
+
+constexpr int MAX_DEVICES = 64;
+std::atomic<void*> no_alloc_scratch_address[MAX_DEVICES];
+
+/// Address of the array on the current device (asked for once per device).
+void* no_alloc_scratch_of_current_device() {
+    int device = 0;
+    MOPS_HIP_CHECK(hipGetDevice(&device));
+    if (device < 0 || device >= MAX_DEVICES) {
+        throw std::runtime_error("mops: device number " + std::to_string(device) + " is beyond the no-allocation entry point's table");
+    }
+    void* address = no_alloc_scratch_address[device].load(std::memory_order_acquire);
+    if (address == nullptr) {
+        MOPS_HIP_CHECK(hipGetSymbolAddress(&address, HIP_SYMBOL(no_alloc_scratch)));
+        if (address == nullptr) {
+            throw std::runtime_error("mops: hipGetSymbolAddress gave no address for the no-allocation scratch array");
+        }
+        // (two threads may both ask: they get the same answer)
+        no_alloc_scratch_address[device].store(address, std::memory_order_release);
+    }
+    return address;
+}
+
+} // namespace
+
+void sasaw_vjp_no_alloc(
+    Tensor<float, 2> grad_A,
+    Tensor<float, 2> grad_B,
+    Tensor<float, 3> grad_W,
+    Tensor<float, 3> grad_output,
+    Tensor<float, 2> A,
+    Tensor<float, 2> B,
+    Tensor<float, 1> C,
+    Tensor<float, 3> W,
+    Tensor<int32_t, 1> indices_A,
+    Tensor<int32_t, 1> indices_W_1,
+    Tensor<int32_t, 1> indices_W_2,
+    Tensor<int32_t, 1> indices_output_1,
+    Tensor<int32_t, 1> indices_output_2
+) {
+    const char* operation = "cuda_sparse_accumulation_scatter_add_with_weights_vjp";
+    checks::Validator validator(operation);
+    checks::sasaw_vjp(
+        validator, grad_A, grad_B, grad_W, grad_output, A, B, C, W, indices_A, indices_W_1, indices_W_2,
+        indices_output_1, indices_output_2
+    );
+    const bool want_edges = grad_A.data != nullptr || grad_B.data != nullptr;
+    const bool want_W = grad_W.data != nullptr;
+    if (!want_edges && !want_W) {
+        return;
+    }
+    const Sizes s = sizes_of(grad_output, A, B, C, W);
+    const sasaw_mfma::Shape shape{s.n_nodes, s.n_edges, s.nA, s.L, s.N, s.n2, s.n3};
+    const char* who = "mops_amd_sparse_accumulation_scatter_add_with_weights_vjp_no_alloc_f32: ";
+    if (!sasaw_mfma::supports(shape, sizeof(float))) {
+        throw std::runtime_error(
+            std::string(who) + "only the shapes of the matrix-core kernels are served without allocation (at least "
+            "one node, edge and table entry; A.shape[1], W.shape[1] and output.shape[1] between 1 and 16); use "
+            "mops_cuda_sparse_accumulation_scatter_add_with_weights_vjp_f32"
+        );
+    }
+    if (!sasaw_mfma::vjp_allocates_nothing(shape, sizeof(float), want_edges, want_W)) {
+        throw std::runtime_error(
+            std::string(who) + "for this graph (more than 48 edges per node on average, or W.shape[1] and "
+            "output.shape[1] in different multiples of four) grad_W is computed beside the other gradients on a "
+            "second stream, which this entry point cannot create; use "
+            "mops_cuda_sparse_accumulation_scatter_add_with_weights_vjp_f32, or ask for grad_W in a call of its own"
+        );
+    }
+    const size_t needed = sasaw_mfma::workspace_bytes(shape, sizeof(float));
+    if (needed > NO_ALLOC_SCRATCH_BYTES) {
+        throw std::runtime_error(
+            std::string(who) + "these shapes need " + std::to_string(needed) + " bytes of temporary memory, the "
+            "built-in array holds " + std::to_string(NO_ALLOC_SCRATCH_BYTES) + " (about " +
+            std::to_string(NO_ALLOC_SCRATCH_BYTES / 528 - 64) + " nodes); use "
+            "mops_cuda_sparse_accumulation_scatter_add_with_weights_vjp_f32"
+        );
+    }
+    void* workspace = no_alloc_scratch_of_current_device();
+    const sasaw_mfma::Indices indices{
+        indices_A.data, indices_W_1.data, indices_W_2.data, indices_output_1.data, indices_output_2.data
+    };
+    sasaw_mfma::vjp<float>(
+        grad_A.data, grad_B.data, grad_W.data, grad_output.data, A.data, B.data, C.data, W.data, indices, shape,
+        workspace, current_stream()
+    );
+    finish_call(operation);
+}
+
+} // namespace mops::amd
+

@@ -1357,6 +1357,20 @@ size_t workspace_bytes(const Shape& s, size_t element_size) {
                                                     : 0);
 }
 
+bool vjp_allocates_nothing(const Shape& s, size_t element_size, bool want_edge_gradients, bool want_grad_W) {
+    if (!want_grad_W) {
+        return true; // the edge-gradient launch alone
+    }
+    if (orders_edges_by_sender(s, element_size)) {
+        return false; // the counting sort of a large graph
+    }
+    if (want_edge_gradients) {
+        // one launch for all three gradients; otherwise grad_W runs beside the others on a second stream
+        return lists_edges_in_slots(s) && (s.n2 + 3) / 4 == (s.n3 + 3) / 4;
+    }
+    return true;
+}
+
 template <typename T>
 void forward(
     T* output, const T* A, const T* B, const T* C, const T* W, const Indices& indices,

@@ -42,6 +42,11 @@ void forward(
     const Shape& shape, void* workspace, hipStream_t stream
 );
 
+/// Whether vjp() for this shape and these wanted gradients only launches
+/// kernels on `stream` with `workspace` as their temporary memory: no second
+/// stream, no events, no allocation.
+bool vjp_allocates_nothing(const Shape& shape, size_t element_size, bool want_edge_gradients, bool want_grad_W);
+
 /// Any of grad_A, grad_B, grad_W may be null.
 template <typename T>
 void vjp(
