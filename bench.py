@@ -1,31 +1,39 @@
 """Benchmark of the mops device path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--all/--no-all]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--extra-shapes] [--no-per-op]
 
-Prints ONE JSON line. The headline workload is BASELINE configuration 1
-(sparse accumulation of products, float32: A[32000,13], B[32000,7], 900
-products, 20 outputs); one "step" is its forward followed by its vjp with
-respect to A and B. ``value`` is algorithmic bytes of a step (every input read
-once, every output written once) divided by the wall time per step, inputs
-resident in HBM, inputs rotated through more than 256 MB of distinct buffers so
-that the 256 MB Infinity Cache cannot serve them.
+Prints ONE JSON line. One "step" is the forward pass followed by the vjp of
+ALL eight operation x dtype combinations of the BASELINE configurations
+(configs[0] HPE f64; configs[1] SAP f32, f64; configs[2] OPSA f32, f64;
+configs[3] OPSAW f32; configs[4] SASAW f32, f64): sixteen calls. ``value`` is
+the algorithmic bytes of a step (every input read once, every output written
+once, index tensors included) divided by the wall time per step, inputs
+resident in HBM and rotated over buffer sets of more than 256 MB per operation
+so that the Infinity Cache cannot serve them. The timed region is an integer
+number of replays of one HIP graph that holds a divisor of K steps, so the
+figure does not depend on K.
 
-Per-kernel figures (``roofline`` for the dominant kernel of the headline, and
-``per_op`` for every BASELINE configuration, forward and vjp separately) are
-device times: the launches of one function over the rotating buffers are
-captured into a HIP graph and the replay is timed with HIP events on the
-stream the kernels run on, which removes the Python / ctypes launch overhead
-from the measurement. The time is per call of the function, i.e. it contains
-every kernel the call launches (first_occurrences, the sender regrouping, the
-table regrouping), not only the main one.
+``per_op`` has one entry per function: the device time of a call (every kernel
+the call launches; HIP-graph replays between HIP events), the same with the
+same buffers every call (``device_us_same_buffers``), the time a plain copy
+kernel takes to read and write exactly the tensors the call reads and writes
+(``copy_us``: the yardstick; ``frac_of_copy`` = copy_us / device_us), and the
+CPU oracle on the host cores. ``roofline`` is the kernel with the most time in
+a step; ``roofline_per_op`` lists the main kernel of every call. Their
+durations come from pairs of HIP events that the library puts around that
+kernel on the stream it launches it on (mops_amd_kernel_timing in
+include/mops/amd.h); ``traffic`` is read from the rocprofv3 counter summary in
+profiles/ (kernels are matched by name).
 
 ``cpu_baseline`` times the CPU oracle (a port of the reference's OpenMP
-algorithm, oracle/oracle.cpp) on the same headline workload on this machine's
-host cores for about ten seconds.
+algorithm, oracle/oracle.cpp) on the same step on this machine's host cores,
+with all threads and with one.
 """
 import argparse
+import ctypes
 import json
 import os
+import re
 import sys
 import time
 
@@ -37,11 +45,23 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0  # MI355X, published
 ROTATE_BYTES = 320 * 1024 * 1024  # > 256 MB Infinity Cache
-# HBM bytes per launch of the main SAP f32 kernels from two rocprofv3 --pmc
-# runs (profiles/all_ops_baseline_shapes_hbm_traffic.txt): FETCH_SIZE x 1.9993
-# (the factor a 64 MiB element-wise pass gives) + WRITE_SIZE x 1.0, in KiB.
-# forward: 1742.5 and 2500.0; vjp: 3099.8 and 2500.0.
-MEASURED_TRAFFIC_BYTES = {"forward": 6094000, "vjp": 8888000}
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "all_ops_baseline_shapes_hbm_traffic.txt")
+
+# The kernel that does the arithmetic of each call at the BASELINE shapes, as
+# rocprofv3 prints it (a prefix; {T} = float / double). Used to label the
+# per-kernel figures and to find the kernel in the counter summary.
+MAIN_KERNELS = {
+    ("hpe", "forward"): "forward_ordered_kernel<{T}, 4>",
+    ("hpe", "vjp"): "vjp_ordered_kernel<{T}, 4>",
+    ("sap", "forward"): "sap_mfma::forward_kernel<{T}, 2, 2>",
+    ("sap", "vjp"): "sap_mfma::vjp_kernel<{T}, 5>",
+    ("opsa", "forward"): "forward_kernel<{T}, 2, false>",
+    ("opsa", "vjp"): "edge_rows_vjp_kernel<{T}, 1, 2, false, true, false, false>",
+    ("opsaw", "forward"): "forward_kernel<{T}, 2, true>",
+    ("opsaw", "vjp"): "edge_rows_vjp_kernel<{T}, 1, 2, true, true, false, true>",
+    ("sasaw", "forward"): "sasaw_mfma::forward_kernel<{T}, 2, 3, 64, false>",
+    ("sasaw", "vjp"): "sasaw_mfma::edge_gradients_kernel<{T}, 2, 3, true>",
+}
 
 
 def nbytes(arrays):
@@ -61,10 +81,10 @@ def algorithmic_bytes(op, case, kind):
     return nbytes(inputs) + case["grad_output"].nbytes + nbytes(grads)
 
 
-def build_configs():
+def build_configs(extra):
     from tests import support
 
-    return [
+    configs = [
         ("c0", "hpe", np.float64, support.hpe_case(0, np.float64)),
         ("c1", "sap", np.float32, support.sap_case(1, np.float32)),
         ("c1", "sap", np.float64, support.sap_case(1, np.float64)),
@@ -73,16 +93,24 @@ def build_configs():
         ("c3", "opsaw", np.float32, support.opsaw_case(3, np.float32)),
         ("c4", "sasaw", np.float32, support.sasaw_case(4, np.float32)),
         ("c4", "sasaw", np.float64, support.sasaw_case(4, np.float64)),
-        # beyond the BASELINE shapes: feature counts that fill whole 16-wide matrix tiles
-        ("wide", "opsa", np.float32, support.opsa_case(5, np.float32, K=32, L=64)),
-        ("wide", "opsaw", np.float32, support.opsaw_case(6, np.float32, K=32, L=64)),
-        # many rows: HPE with a lane per row (forward) and by feature (vjp)
-        ("many_rows", "hpe", np.float64, support.hpe_case(10, np.float64, I=20000, nA=50, J=4000, K=3)),
-        # 128 feature channels: the kernels take them in blocks of 64 columns
-        ("wide128", "opsa", np.float32, support.opsa_case(7, np.float32, K=16, L=128)),
-        ("wide128", "opsaw", np.float32, support.opsaw_case(8, np.float32, K=16, L=128)),
-        ("wide128", "sasaw", np.float32, support.sasaw_case(9, np.float32, L=128)),
     ]
+    if extra:
+        configs += [
+            # beyond the BASELINE shapes: feature counts that fill whole 16-wide matrix tiles
+            ("wide", "opsa", np.float32, support.opsa_case(5, np.float32, K=32, L=64)),
+            ("wide", "opsaw", np.float32, support.opsaw_case(6, np.float32, K=32, L=64)),
+            # many rows: HPE with a lane per row (forward) and by feature (vjp)
+            ("many_rows", "hpe", np.float64, support.hpe_case(10, np.float64, I=20000, nA=50, J=4000, K=3)),
+            # 128 feature channels
+            ("wide128", "opsa", np.float32, support.opsa_case(7, np.float32, K=16, L=128)),
+            ("wide128", "opsaw", np.float32, support.opsaw_case(8, np.float32, K=16, L=128)),
+            ("wide128", "sasaw", np.float32, support.sasaw_case(9, np.float32, L=128)),
+        ]
+    return configs
+
+
+class Span(ctypes.Structure):
+    _fields_ = [("data", ctypes.c_void_p), ("bytes", ctypes.c_int64)]
 
 
 class DeviceWorkload:
@@ -136,6 +164,23 @@ class DeviceWorkload:
         self.forward()
         self.vjp()
 
+    # the copy yardstick on the tensors the call reads and writes
+    def _copy(self, read_names, write_names):
+        t = self._next()
+        reads = (Span * len(read_names))(*[Span(t[n].data_ptr(), t[n].numel() * t[n].element_size()) for n in read_names])
+        writes = (Span * len(write_names))(
+            *[Span(t[n].data_ptr(), t[n].numel() * t[n].element_size()) for n in write_names]
+        )
+        status = self.library.cdll.mops_amd_copy_yardstick(reads, len(read_names), writes, len(write_names))
+        if status != 0:
+            raise RuntimeError(self.library.last_error())
+
+    def copy_forward(self):
+        self._copy(list(self.spec.inputs), ["output"])
+
+    def copy_vjp(self):
+        self._copy(["grad_output", *self.spec.inputs], ["grad_" + n for n in self.spec.differentiable])
+
 
 def bind_library_to_torch_stream(device):
     import torch
@@ -144,28 +189,21 @@ def bind_library_to_torch_stream(device):
 
     library = device_library()
     torch.cuda.set_device(device)
-    library.cdll.mops_amd_set_stream(torch.cuda.current_stream(device).cuda_stream)
+    library.cdll.mops_amd_set_stream(ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream))
     library.cdll.mops_amd_set_synchronous(0)
     return library
 
 
-def device_time_per_call(function, calls, replays, device):
-    """Average device time (seconds) of one call of ``function``.
-
-    ``calls`` consecutive calls are captured into a HIP graph; the graph is
-    replayed ``replays`` times between two HIP events on the capture stream's
-    parent (torch's current) stream.
-    """
+def capture(function, calls, device):
+    """A HIP graph of ``calls`` consecutive calls of ``function`` (None if the capture fails)."""
     import torch
 
     for _ in range(3):
-        function()  # warm up: allocates the library's scratch block outside the capture
+        function()  # warm up: the library's scratch block takes its size outside the capture
     torch.cuda.synchronize()
-
     graph = torch.cuda.CUDAGraph()
     stream = torch.cuda.Stream(device=device)
     stream.wait_stream(torch.cuda.current_stream(device))
-    captured = True
     try:
         with torch.cuda.stream(stream):
             bind_library_to_torch_stream(device)
@@ -176,14 +214,22 @@ def device_time_per_call(function, calls, replays, device):
                 for _ in range(calls):
                     function()
     except Exception as error:  # pragma: no cover - depends on the runtime
-        captured = False
         sys.stderr.write(f"graph capture failed ({error}); timing eager launches instead\n")
+        graph = None
     bind_library_to_torch_stream(device)
     torch.cuda.synchronize()
+    return graph
 
+
+def device_time_per_call(function, calls, replays, device):
+    """Average device time (seconds) of one call of ``function``: replays of a graph of ``calls``
+    calls between two HIP events on the stream the replays are launched on."""
+    import torch
+
+    graph = capture(function, calls, device)
     start = torch.cuda.Event(enable_timing=True)
     stop = torch.cuda.Event(enable_timing=True)
-    if captured:
+    if graph is not None:
         graph.replay()
         torch.cuda.synchronize()
         start.record()
@@ -196,44 +242,12 @@ def device_time_per_call(function, calls, replays, device):
             function()
         stop.record()
     torch.cuda.synchronize()
-    return start.elapsed_time(stop) * 1e-3 / (replays * calls), captured
-
-
-def capture_steps(workload, steps, device):
-    """A HIP graph holding ``steps`` consecutive steps of ``workload`` (None if capture fails)."""
-    import torch
-
-    for _ in range(3):
-        workload.step()
-    torch.cuda.synchronize()
-    graph = torch.cuda.CUDAGraph()
-    stream = torch.cuda.Stream(device=device)
-    stream.wait_stream(torch.cuda.current_stream(device))
-    try:
-        with torch.cuda.stream(stream):
-            bind_library_to_torch_stream(device)
-            workload.step()
-            torch.cuda.synchronize()
-            with torch.cuda.graph(graph, stream=stream):
-                bind_library_to_torch_stream(device)
-                for _ in range(steps):
-                    workload.step()
-    except Exception as error:  # pragma: no cover - depends on the runtime
-        sys.stderr.write(f"graph capture failed ({error}); timing eager launches instead\n")
-        graph = None
-    bind_library_to_torch_stream(device)
-    torch.cuda.synchronize()
-    return graph
+    return start.elapsed_time(stop) * 1e-3 / (replays * calls), graph is not None
 
 
 def main_kernel_time(library, function, calls):
-    """Average duration (seconds) of the main kernel of ``function`` over ``calls`` eager calls.
-
-    The library attaches a pair of HIP events to that kernel's launch on the
-    stream it launches it on (mops_amd_kernel_timing in include/mops/amd.h).
-    """
-    import ctypes
-
+    """Average duration (seconds) of the main kernel of ``function`` over ``calls`` eager calls,
+    from the pairs of HIP events the library records around it on its launch stream."""
     import torch
 
     function()
@@ -254,29 +268,63 @@ def main_kernel_time(library, function, calls):
 
 def cpu_time(function, seconds, max_calls):
     function()
-    function()
     times = []
     begin = time.perf_counter()
-    while len(times) < max_calls and (time.perf_counter() - begin < seconds or len(times) < 3):
+    while len(times) < max_calls and (time.perf_counter() - begin < seconds or len(times) < 2):
         t0 = time.perf_counter()
         function()
         times.append(time.perf_counter() - t0)
     return times
 
 
+def cpu_model():
+    try:
+        with open("/proc/cpuinfo") as handle:
+            for line in handle:
+                if line.startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+def measured_traffic(kernel_prefix):
+    """HBM bytes per launch of the kernel whose name starts with ``kernel_prefix``, from the
+    rocprofv3 counter summary under profiles/ (last column of its table: total MB), or None."""
+    try:
+        with open(TRAFFIC_FILE) as handle:
+            lines = handle.read().split("\n")
+    except OSError:
+        return None
+    for line in lines:
+        if line.startswith(kernel_prefix[:95]):
+            columns = re.findall(r"[-+]?\d+\.\d+", line[len(kernel_prefix[:95]):])
+            if len(columns) >= 5:
+                return int(round(float(columns[-1]) * 1e6))
+    return None
+
+
+def largest_divisor(n, limit):
+    for candidate in range(min(n, limit), 0, -1):
+        if n % candidate == 0:
+            return candidate
+    return 1
+
+
 def main():
     parser = argparse.ArgumentParser()
     parser.add_argument("--gpus", type=int, default=1)
-    parser.add_argument("--steps", type=int, default=2000)
-    parser.add_argument("--warmup", type=int, default=100)
+    parser.add_argument("--steps", type=int, default=200)
+    parser.add_argument("--warmup", type=int, default=20)
     parser.add_argument("--cpu-seconds", type=float, default=10.0)
-    parser.add_argument("--no-per-op", action="store_true", help="only the headline workload")
+    parser.add_argument("--no-per-op", action="store_true", help="only the headline step")
+    parser.add_argument("--extra-shapes", action="store_true", help="per_op also for shapes beyond the BASELINE ones")
     parser.add_argument(
         "--profile",
         choices=["hpe", "sap", "opsa", "opsaw", "sasaw", "all"],
         help="for rocprofv3: run 50 eager forward+vjp calls of the operation(s) at the BASELINE "
-        "shapes (all their dtypes) and 20 element-wise passes over 64 MiB (read 64 MiB, write 64 MiB) as a yardstick for the HBM "
-        "counters, print nothing, exit",
+        "shapes (all their dtypes), each followed by the copy yardstick on the same tensors, and 20 element-wise "
+        "passes over 64 MiB (read 64 MiB, write 64 MiB) as a yardstick for the HBM counters, print nothing, exit",
     )
     args = parser.parse_args()
 
@@ -297,16 +345,21 @@ def main():
         sys.stderr.write("bench.py needs a GPU (the device library has no CPU fallback)\n")
         sys.exit(2)
     device = torch.device("cuda:0")
-    bind_library_to_torch_stream(device)
+    library = bind_library_to_torch_stream(device)
+    library.cdll.mops_amd_copy_yardstick.argtypes = [ctypes.c_void_p, ctypes.c_int32, ctypes.c_void_p, ctypes.c_int32]
     oracle = support.oracle_library()
-    configs = build_configs()
+    configs = build_configs(args.extra_shapes)
+    baseline = [c for c in configs if c[0].startswith("c")]
 
     if args.profile:
-        for config, op_name, _, op_case in configs:
-            if config.startswith("c") and args.profile in (op_name, "all"):
+        for config, op_name, _, op_case in baseline:
+            if args.profile in (op_name, "all"):
                 w = DeviceWorkload(op_name, op_case, device)
                 for _ in range(50):
-                    w.step()
+                    w.forward()
+                    w.copy_forward()
+                    w.vjp()
+                    w.copy_vjp()
                 torch.cuda.synchronize()
                 del w
                 torch.cuda.empty_cache()
@@ -317,40 +370,47 @@ def main():
         torch.cuda.synchronize()
         return
 
-    # ---------------- headline: c1 SAP f32, forward + vjp -------------------
-    # The K timed steps are replays of HIP graphs that hold `steps_per_graph`
-    # steps each (the launch-bound loop is what graphs are for); what does not
-    # fill a whole graph is launched eagerly inside the same timed region.
-    _, op, dtype, case = configs[1]
-    workload = DeviceWorkload(op, case, device)
-    step_bytes = algorithmic_bytes(op, case, "forward") + algorithmic_bytes(op, case, "vjp")
-    steps_per_graph = max(1, min(workload.n_sets // 2, args.steps))
-    graph = capture_steps(workload, steps_per_graph, device)
+    # ---------------- headline: one step = forward + vjp of all eight combinations ----------
+    workloads = {}
+    for config, op_name, op_dtype, op_case in baseline:
+        workloads[(config, op_name, np.dtype(op_dtype).name)] = DeviceWorkload(op_name, op_case, device)
+    step_bytes = sum(
+        algorithmic_bytes(w.op, w.case, "forward") + algorithmic_bytes(w.op, w.case, "vjp") for w in workloads.values()
+    )
+
+    def step():
+        for w in workloads.values():
+            w.step()
+
+    steps_per_graph = largest_divisor(args.steps, 8)
+    graph = capture(step, steps_per_graph, device)
     for _ in range(args.warmup):
-        workload.step()
+        step()
     torch.cuda.synchronize()
     begin = time.perf_counter()
-    done = 0
     if graph is not None:
-        while done + steps_per_graph <= args.steps:
+        for _ in range(args.steps // steps_per_graph):
             graph.replay()
-            done += steps_per_graph
-    while done < args.steps:
-        workload.step()
-        done += 1
+    else:
+        for _ in range(args.steps):
+            step()
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - begin
-    ms_per_step = elapsed / args.steps * 1e3
-    value = step_bytes / (elapsed / args.steps) / 1e9
+    seconds_per_step = elapsed / args.steps
+    value = step_bytes / seconds_per_step / 1e9
 
-    # ---------------- device time per function ------------------------------
+    # ---------------- per function: call, copy yardstick, main kernel, CPU ------------------
     per_op = []
-    selected = configs if not args.no_per_op else [configs[1]]
+    roofline_per_op = []
+    selected = [] if args.no_per_op else configs
     for config, op_name, op_dtype, op_case in selected:
-        w = workload if (op_name, op_dtype) == (op, dtype) else DeviceWorkload(op_name, op_case, device)
-        for kind, function in (("forward", w.forward), ("vjp", w.vjp)):
+        key = (config, op_name, np.dtype(op_dtype).name)
+        w = workloads.get(key) or DeviceWorkload(op_name, op_case, device)
+        type_name = "float" if op_dtype == np.float32 else "double"
+        for kind, function, copy in (("forward", w.forward, w.copy_forward), ("vjp", w.vjp, w.copy_vjp)):
             calls = min(w.n_sets, 64)
             seconds, captured = device_time_per_call(function, calls, 20, device)
+            copy_seconds, _ = device_time_per_call(copy, calls, 20, device)
             abytes = algorithmic_bytes(op_name, op_case, kind)
             entry = {
                 "config": config,
@@ -361,82 +421,114 @@ def main():
                 "algorithmic_bytes": abytes,
                 "GBps": round(abytes / seconds / 1e9, 1),
                 "hbm_frac": round(abytes / seconds / 1e9 / HBM_PEAK_GBS, 4),
+                "copy_us": round(copy_seconds * 1e6, 3),
+                "frac_of_copy": round(copy_seconds / seconds, 3),
                 "timed": "hip-graph replay, HIP events" if captured else "eager launches, HIP events",
             }
             w.rotate = False
             warm_seconds, _ = device_time_per_call(function, calls, 20, device)
             w.rotate = True
             entry["device_us_same_buffers"] = round(warm_seconds * 1e6, 3)
-            if not args.no_per_op:
-                cpu_function = (
-                    (lambda c=op_case, o=op_name: support.cpu_forward(oracle, o, c))
-                    if kind == "forward"
-                    else (lambda c=op_case, o=op_name: support.cpu_vjp(oracle, o, c))
-                )
-                times = cpu_time(cpu_function, 0.5, 20)
-                entry["cpu_ms"] = round(float(np.median(times)) * 1e3, 3)
-                entry["cpu_GBps"] = round(abytes / float(np.median(times)) / 1e9, 3)
+            cpu_function = (
+                (lambda c=op_case, o=op_name: support.cpu_forward(oracle, o, c))
+                if kind == "forward"
+                else (lambda c=op_case, o=op_name: support.cpu_vjp(oracle, o, c))
+            )
+            times = cpu_time(cpu_function, 0.4, 20)
+            entry["cpu_ms"] = round(float(np.median(times)) * 1e3, 3)
+            entry["cpu_GBps"] = round(abytes / float(np.median(times)) / 1e9, 3)
             per_op.append(entry)
-        if w is not workload:
+
+            if config.startswith("c"):
+                kernel_seconds, launches = main_kernel_time(library, function, 200)
+                name = MAIN_KERNELS.get((op_name, kind), "?").format(T=type_name)
+                timed_by = "HIP events around the kernel on its launch stream, eager calls, rotating inputs"
+                if kernel_seconds is None:
+                    # this call's kernels carry no events: the whole call as one interval
+                    kernel_seconds, launches = seconds, calls * 20
+                    timed_by = "whole call (all its kernels) as HIP-graph replays between HIP events"
+                roofline_per_op.append(
+                    {
+                        "config": config,
+                        "op": op_name,
+                        "dtype": np.dtype(op_dtype).name,
+                        "function": kind,
+                        "kernel": name,
+                        "avg_us": round(kernel_seconds * 1e6, 3),
+                        "launches_timed": launches,
+                        "algorithmic_bytes_per_launch": abytes,
+                        "achieved_GBps": round(abytes / kernel_seconds / 1e9, 1),
+                        "frac": round(abytes / kernel_seconds / 1e9 / HBM_PEAK_GBS, 4),
+                        "traffic": measured_traffic(name),
+                        "timed": timed_by,
+                    }
+                )
+        if key not in workloads:
             del w
             torch.cuda.empty_cache()
 
-    # ---------------- roofline of the dominant kernel -----------------------
-    # At this shape each call is one kernel (mops_amd/csrc/sap_mfma.hip), timed
-    # with a pair of HIP events that the library hands to the launch itself
-    # (hipExtLaunchKernelGGL stamps them with the begin and the end of that
-    # kernel on the stream it runs on). Consecutive eager calls from Python
-    # cannot be used instead: the interpreter needs longer per call than the
-    # kernel runs.
-    library = bind_library_to_torch_stream(device)
-    kernels = {}
-    for kind, function, name in (
-        ("forward", workload.forward, "mops::amd::sap_mfma::(anonymous namespace)::forward_kernel<float, 2, 2>"),
-        ("vjp", workload.vjp, "mops::amd::sap_mfma::(anonymous namespace)::vjp_kernel<float, 5>"),
-    ):
-        seconds, launches = main_kernel_time(library, function, 400)
-        kernels[kind] = (seconds, launches, name)
-    dominant_kind = max(kernels, key=lambda k: kernels[k][0] or 0.0)
-    kernel_seconds, kernel_launches, kernel_name = kernels[dominant_kind]
-    kernel_bytes = algorithmic_bytes(op, case, dominant_kind)
-    if kernel_seconds is None:
-        headline_entries = [e for e in per_op if e["op"] == op and e["dtype"] == np.dtype(dtype).name]
-        entry = max(headline_entries, key=lambda e: e["device_us"])
-        kernel_seconds = entry["device_us"] * 1e-6
-    achieved = kernel_bytes / kernel_seconds / 1e9
+    # ---------------- roofline of the kernel with the most time in a step -------------------
+    if roofline_per_op:
+        dominant = max(roofline_per_op, key=lambda e: e["avg_us"])
+    else:
+        # --no-per-op: only the kernel that dominated the last full run is timed
+        w = workloads[("c4", "sasaw", "float64")]
+        kernel_seconds, launches = main_kernel_time(library, w.vjp, 200)
+        abytes = algorithmic_bytes("sasaw", w.case, "vjp")
+        if kernel_seconds is None:
+            kernel_seconds, _ = device_time_per_call(w.vjp, w.n_sets, 20, device)
+            launches = w.n_sets * 20
+        name = MAIN_KERNELS[("sasaw", "vjp")].format(T="double")
+        dominant = {
+            "config": "c4", "op": "sasaw", "dtype": "float64", "function": "vjp", "kernel": name,
+            "avg_us": round(kernel_seconds * 1e6, 3), "launches_timed": launches,
+            "algorithmic_bytes_per_launch": abytes, "achieved_GBps": round(abytes / kernel_seconds / 1e9, 1),
+            "frac": round(abytes / kernel_seconds / 1e9 / HBM_PEAK_GBS, 4), "traffic": measured_traffic(name),
+            "timed": "HIP events around the kernel on its launch stream",
+        }  # fmt: skip
     roofline = {
         "bound": "hbm",
-        "kernel": kernel_name,
-        "achieved": round(achieved, 1),
+        "kernel": dominant["kernel"],
+        "of": f"{dominant['config']} {dominant['op']} {dominant['dtype']} {dominant['function']}",
+        "achieved": dominant["achieved_GBps"],
         "peak": HBM_PEAK_GBS,
         "unit": "GB/s",
-        "frac": round(achieved / HBM_PEAK_GBS, 4),
-        "traffic": MEASURED_TRAFFIC_BYTES.get(dominant_kind),
-        "algorithmic_bytes_per_launch": kernel_bytes,
-        "avg_launch_us": round(kernel_seconds * 1e6, 3),
-        "launches_timed": kernel_launches,
-        "timed": "HIP events attached to the kernel launch (start/stop of that kernel on its launch stream), "
-        "eager launches, rotating inputs",
-        "other_kernel_us": {
-            kind: None if kernels[kind][0] is None else round(kernels[kind][0] * 1e6, 3) for kind in kernels
-        },
+        "frac": dominant["frac"],
+        "traffic": dominant["traffic"],
+        "traffic_from": os.path.relpath(TRAFFIC_FILE, ROOT),
+        "algorithmic_bytes_per_launch": dominant["algorithmic_bytes_per_launch"],
+        "avg_launch_us": dominant["avg_us"],
+        "launches_timed": dominant["launches_timed"],
+        "timed": dominant["timed"],
     }
 
-    # ---------------- CPU baseline on the headline workload -----------------
+    # ---------------- CPU baseline on the same step ------------------------------------------
     def cpu_step():
-        support.cpu_forward(oracle, op, case)
-        support.cpu_vjp(oracle, op, case)
+        for w in workloads.values():
+            support.cpu_forward(oracle, w.op, w.case)
+            support.cpu_vjp(oracle, w.op, w.case)
 
+    threads = int(oracle.cdll.mops_oracle_num_threads())
     times = cpu_time(cpu_step, args.cpu_seconds, 100000)
     cpu_seconds = float(np.median(times))
-    threads = int(oracle.cdll.mops_oracle_num_threads())
+    oracle.cdll.mops_oracle_set_num_threads(1)
+    single = cpu_time(cpu_step, args.cpu_seconds, 100000)
+    oracle.cdll.mops_oracle_set_num_threads(threads)
+    single_seconds = float(np.median(single))
     cpu_baseline = {
         "value": round(step_bytes / cpu_seconds / 1e9, 3),
         "unit": "GB/s",
         "cores": threads,
         "kind": "port",
-        "sample": f"{len(times)} steps of the same workload (median {cpu_seconds * 1e3:.2f} ms/step) "
-        f"in {sum(times):.1f} s, OpenMP threads = {threads}",
+        "cpu_model": cpu_model(),
+        "sample": f"{len(times)} steps of the same workload (all eight combinations, forward + vjp; median "
+        f"{cpu_seconds * 1e3:.1f} ms/step) in {sum(times):.1f} s, OpenMP threads = {threads}",
+        "one_thread": {
+            "value": round(step_bytes / single_seconds / 1e9, 3),
+            "unit": "GB/s",
+            "cores": 1,
+            "sample": f"{len(single)} steps (median {single_seconds * 1e3:.1f} ms/step) in {sum(single):.1f} s",
+        },
     }
 
     result = {
@@ -446,22 +538,23 @@ def main():
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
-        "ms_per_step": round(ms_per_step, 5),
+        "ms_per_step": round(seconds_per_step * 1e3, 5),
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "f32",
+        "dtype": "f32+f64",
         "data": "synthetic",
         "config": {
-            "workload": "BASELINE configs[1]: sparse_accumulation_of_products f32, A[32000,13] "
-            "B[32000,7] C[900] sorted indices_output in [0,20); one step = forward + vjp(A, B); "
-            f"inputs rotated over {workload.n_sets} buffer sets; timed as replays of HIP graphs of "
-            f"{steps_per_graph} steps",
+            "workload": "BASELINE configs[0..4], every operation x dtype they name: HPE f64 (c0), SAP f32 + f64 (c1), "
+            "OPSA f32 + f64 (c2), OPSAW f32 (c3), SASAW f32 + f64 (c4); one step = forward + vjp of all eight "
+            f"(sixteen calls); inputs rotated over > 320 MB of buffer sets per operation; timed as "
+            f"{args.steps // steps_per_graph} replays of one HIP graph of {steps_per_graph} steps",
             "algorithmic_bytes_per_step": step_bytes,
             "value_is": "algorithmic bytes per step / wall time per step",
         },
         "roofline": roofline,
         "cpu_baseline": cpu_baseline,
+        "roofline_per_op": roofline_per_op,
         "per_op": per_op,
         "device": torch.cuda.get_device_name(0),
     }

@@ -1041,6 +1041,7 @@ void homogeneous_polynomial_evaluation(MOPS_HPE_PARAMS(MOPS_CXX_FIRST, MOPS_CXX_
     if (R > 0) {
         size_t lds = (static_cast<size_t>(nA) * R + THREADS) * sizeof(scalar_t);
         unsigned blocks = static_cast<unsigned>(ceil_div(static_cast<size_t>(n_rows), R));
+        MainKernelTimer timer(stream);
 #define MOPS_LAUNCH_ORDERED(ORDER)                                                                  \
     forward_ordered_kernel<scalar_t, ORDER><<<blocks, THREADS, lds, stream>>>(                     \
         output.data, A.data, C.data, indices_A.data, n_rows, nA, n_monomials, R                    \
@@ -1208,6 +1209,7 @@ void homogeneous_polynomial_evaluation_vjp(MOPS_HPE_VJP_PARAMS(MOPS_CXX_FIRST, M
             static_cast<unsigned>(ceil_div(static_cast<size_t>(n_rows), R)),
             static_cast<unsigned>(ceil_div(static_cast<size_t>(nA), span))
         );
+        MainKernelTimer timer(stream);
 #define MOPS_LAUNCH_ORDERED(ORDER)                                                                  \
     vjp_ordered_kernel<scalar_t, ORDER><<<blocks, WAVE, lds, stream>>>(                            \
         grad_A.data, grad_output.data, A.data, C.data, indices_A.data, n_rows, nA, n_monomials, R, \

@@ -1352,6 +1352,8 @@ void launch_forward(
         finish_call(operation);
         return;
     }
+    {
+    MainKernelTimer timer(stream);
 #define MOPS_LAUNCH_FORWARD(NT)                                                                    \
     forward_kernel<T, NT, WEIGHTED><<<blocks, BLOCK, 0, stream>>>(                                 \
         output.data, A.data, B.data, W, indices_W, indices_output.data, n_edges, n_output, K, L    \
@@ -1362,6 +1364,7 @@ void launch_forward(
         MOPS_LAUNCH_FORWARD(2);
     } else {
         MOPS_LAUNCH_FORWARD(4);
+    }
     }
 #undef MOPS_LAUNCH_FORWARD
     finish_call(operation);

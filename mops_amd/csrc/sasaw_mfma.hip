@@ -1389,6 +1389,7 @@ void forward(
         );
         const size_t lds = forward_lds(block, sizeof(T));
         T* target = output + first;
+        MainKernelTimer timer(stream);
         with_shape_constants(tiles_for(block.L), (s.n2 + 3) / 4, [&](auto tiles, auto steps) {
             if (short_chunks) {
                 auto kernel = forward_kernel<T, decltype(tiles)::value, decltype(steps)::value, SHORT_CHUNK, false>;
@@ -1506,6 +1507,7 @@ void vjp(
         const int32_t grid = (s.n_edges + STAGE - 1) / STAGE + weights.n_senders;
         const size_t lds =
             std::max(edge_gradients_lds(block, sizeof(T)), with_weights ? t_area_bytes(block, sizeof(T)) : 0);
+        MainKernelTimer timer(stream);
         with_shape_constants(tiles_for(block.L), (s.n2 + 3) / 4, [&](auto tiles_constant, auto steps) {
             if (with_weights) {
                 auto kernel = edge_gradients_kernel<T, decltype(tiles_constant)::value, decltype(steps)::value, true>;

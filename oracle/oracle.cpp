@@ -840,6 +840,8 @@ ORACLE_EXPORT int mops_oracle_first_occurrences(
 #ifdef _OPENMP
 #include <omp.h>
 ORACLE_EXPORT int mops_oracle_num_threads(void) { return omp_get_max_threads(); }
+ORACLE_EXPORT void mops_oracle_set_num_threads(int threads) { omp_set_num_threads(threads < 1 ? 1 : threads); }
 #else
 ORACLE_EXPORT int mops_oracle_num_threads(void) { return 1; }
+ORACLE_EXPORT void mops_oracle_set_num_threads(int) {}
 #endif
