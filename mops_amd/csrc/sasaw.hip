@@ -51,6 +51,7 @@
 #include "edge_order.hpp"
 #include "runtime.hpp"
 #include "sasaw_mfma.hpp"
+#include "sasaw_segments.hpp"
 #include "sender_buckets.hpp"
 
 namespace mops::amd {
@@ -626,6 +627,14 @@ void sparse_accumulation_scatter_add_with_weights(MOPS_SASAW_PARAMS(MOPS_CXX_FIR
     hipStream_t stream = current_stream();
 
     const sasaw_mfma::Shape shape{s.n_nodes, s.n_edges, s.nA, s.L, s.N, s.n2, s.n3};
+    if (sasaw_segments::supports(shape, sizeof(scalar_t))) {
+        const sasaw_mfma::Indices indices{
+            indices_A.data, indices_W_1.data, indices_W_2.data, indices_output_1.data, indices_output_2.data
+        };
+        sasaw_segments::forward<scalar_t>(output.data, A.data, B.data, C.data, W.data, indices, shape, stream);
+        finish_call(operation);
+        return;
+    }
     if (sasaw_mfma::supports(shape, sizeof(scalar_t))) {
         const sasaw_mfma::Indices indices{
             indices_A.data, indices_W_1.data, indices_W_2.data, indices_output_1.data, indices_output_2.data

@@ -1,0 +1,38 @@
+// SASAW for coupling tables whose component indices have at most 16 values
+// each (equivariant message passing), any number of feature channels, as
+// per-node sums of rank-one updates on the matrix cores. sasaw.hip calls these
+// when `supports()` says so and keeps its general kernels for everything else.
+#ifndef MOPS_AMD_SASAW_SEGMENTS_HPP
+#define MOPS_AMD_SASAW_SEGMENTS_HPP
+
+#include <cstddef>
+#include <cstdint>
+
+#include <hip/hip_runtime.h>
+
+#include "sasaw_mfma.hpp"
+
+namespace mops::amd::sasaw_segments {
+
+using sasaw_mfma::Indices;
+using sasaw_mfma::Shape;
+
+/// Whether these kernels cover the shape for elements of `element_size` bytes.
+bool supports(const Shape& shape, size_t element_size);
+
+template <typename T>
+void forward(
+    T* output, const T* A, const T* B, const T* C, const T* W, const Indices& indices,
+    const Shape& shape, hipStream_t stream
+);
+
+/// grad_W from the lists of every sender's edges (sender_buckets.hpp).
+template <typename T>
+void grad_W_from_slots(
+    T* grad_W, const T* grad_output, const T* A, const T* B, const T* C, const Indices& indices,
+    const Shape& shape, const SenderSlots& slots, hipStream_t stream
+);
+
+} // namespace mops::amd::sasaw_segments
+
+#endif

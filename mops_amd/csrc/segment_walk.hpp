@@ -31,8 +31,37 @@
 
 namespace mops::amd {
 
+/// What a wavefront looks at of the sorted index: asked for as early as a
+/// kernel likes (the loads do not depend on anything), used by walk_pieces.
+struct ChunkIndex {
+    int32_t mine;   // value at the lane's position of the chunk
+    int32_t before; // value at the position before it (-1 in front of position 0)
+    int32_t ahead;  // value at the lane's position of the 64 positions after the chunk
+};
+
+template <int CHUNK>
+__device__ __forceinline__ ChunkIndex load_chunk_index(
+    const int32_t* __restrict__ sorted_index, int32_t n_input, int32_t wave_index
+) {
+    static_assert(CHUNK >= 1 && CHUNK <= WAVE, "one index value per lane");
+    const int lane = threadIdx.x & (WAVE - 1);
+    const int32_t chunk_begin = wave_index * CHUNK;
+    const int32_t position = chunk_begin + lane;
+    const bool inside = lane < CHUNK && position < n_input;
+    ChunkIndex index;
+    index.mine = load_or_zero(sorted_index, static_cast<size_t>(position), inside);
+    index.before = (inside && position > 0) ? sorted_index[position - 1] : -1;
+    // the 64 positions after the chunk, asked for now: the last segment of the
+    // chunk almost always ends there, and its end is then known without
+    // another round trip to memory
+    const int32_t ahead_position = chunk_begin + CHUNK + lane;
+    index.ahead = load_or_zero(sorted_index, static_cast<size_t>(ahead_position), ahead_position < n_input);
+    return index;
+}
+
 /// Called by all lanes of a wavefront. `wave_index` is the global number of
-/// the wavefront (uniform). CHUNK <= 64.
+/// the wavefront (uniform). CHUNK <= 64. `index`: load_chunk_index of the
+/// same arguments.
 ///   on_segment(row, first, last)  all lanes, uniform arguments, 0 <= row < n_rows
 ///   on_empty_rows(begin, end)     all lanes, rows in [begin, end) receive nothing
 ///   on_piece(row, first, last, from_start, to_end)   (walk_split_segments)
@@ -42,6 +71,7 @@ __device__ __forceinline__ void walk_pieces(
     int32_t n_input,
     int32_t n_rows,
     int32_t wave_index,
+    const ChunkIndex& index,
     PieceFn&& on_piece,
     EmptyRowsFn&& on_empty_rows
 ) {
@@ -54,13 +84,9 @@ __device__ __forceinline__ void walk_pieces(
     }
     const int32_t position = chunk_begin + lane;
     const bool inside = lane < CHUNK && position < n_input;
-    const int32_t mine = inside ? sorted_index[position] : 0;
-    const int32_t before = (inside && position > 0) ? sorted_index[position - 1] : -1;
-    // the 64 positions after the chunk, asked for now: the last segment of the
-    // chunk almost always ends there, and its end is then known without
-    // another round trip to memory
-    const int32_t ahead_position = chunk_begin + CHUNK + lane;
-    const int32_t ahead = load_or_zero(sorted_index, static_cast<size_t>(ahead_position), ahead_position < n_input);
+    const int32_t mine = index.mine;
+    const int32_t before = index.before;
+    const int32_t ahead = index.ahead;
     const bool segment_starts_here = inside && (position == 0 || mine != before);
     const bool starts_here = segment_starts_here || (SPLIT > 0 && inside && position % (SPLIT > 0 ? SPLIT : 1) == 0);
 
@@ -138,8 +164,29 @@ __device__ __forceinline__ void walk_owned_segments(
     SegmentFn&& on_segment,
     EmptyRowsFn&& on_empty_rows
 ) {
+    if (wave_index * CHUNK >= n_input) {
+        return;
+    }
+    const ChunkIndex index = load_chunk_index<CHUNK>(sorted_index, n_input, wave_index);
     walk_pieces<CHUNK, 0>(
-        sorted_index, n_input, n_rows, wave_index,
+        sorted_index, n_input, n_rows, wave_index, index,
+        [&](int32_t row, int32_t first, int32_t last, bool, bool) { on_segment(row, first, last); }, on_empty_rows
+    );
+}
+
+/// The same with the index values asked for beforehand (load_chunk_index).
+template <int CHUNK, typename SegmentFn, typename EmptyRowsFn>
+__device__ __forceinline__ void walk_owned_segments(
+    const int32_t* __restrict__ sorted_index,
+    int32_t n_input,
+    int32_t n_rows,
+    int32_t wave_index,
+    const ChunkIndex& index,
+    SegmentFn&& on_segment,
+    EmptyRowsFn&& on_empty_rows
+) {
+    walk_pieces<CHUNK, 0>(
+        sorted_index, n_input, n_rows, wave_index, index,
         [&](int32_t row, int32_t first, int32_t last, bool, bool) { on_segment(row, first, last); }, on_empty_rows
     );
 }
@@ -154,7 +201,11 @@ __device__ __forceinline__ void walk_split_segments(
     EmptyRowsFn&& on_empty_rows
 ) {
     static_assert(SPLIT > 0, "distance between cuts");
-    walk_pieces<CHUNK, SPLIT>(sorted_index, n_input, n_rows, wave_index, on_piece, on_empty_rows);
+    if (wave_index * CHUNK >= n_input) {
+        return;
+    }
+    const ChunkIndex index = load_chunk_index<CHUNK>(sorted_index, n_input, wave_index);
+    walk_pieces<CHUNK, SPLIT>(sorted_index, n_input, n_rows, wave_index, index, on_piece, on_empty_rows);
 }
 
 } // namespace mops::amd
