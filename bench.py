@@ -60,7 +60,7 @@ MAIN_KERNELS = {
     ("opsaw", "forward"): "forward_kernel<{T}, 2, true>",
     ("opsaw", "vjp"): "edge_rows_vjp_kernel<{T}, 1, 2, true, true, false, true>",
     ("sasaw", "forward"): "sasaw_segments::contract_kernel<{T}, 9, true, (sasaw_segments::(anonymous namespace)::Source)0",
-    ("sasaw", "vjp"): "sasaw_mfma::edge_gradients_kernel<{T}, 2, 3, true>",
+    ("sasaw", "vjp"): "sasaw_segments::(anonymous namespace)::gradients_kernel<{T}, 9, true>",
 }
 
 

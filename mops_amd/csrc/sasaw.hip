@@ -742,6 +742,19 @@ void sparse_accumulation_scatter_add_with_weights_vjp(MOPS_SASAW_VJP_PARAMS(MOPS
     hipStream_t stream = current_stream();
 
     const sasaw_mfma::Shape shape{s.n_nodes, s.n_edges, s.nA, s.L, s.N, s.n2, s.n3};
+    if (s.L > 0 && sasaw_segments::vjp_supported(shape, sizeof(scalar_t), want_W)) {
+        const sasaw_mfma::Indices indices{
+            indices_A.data, indices_W_1.data, indices_W_2.data, indices_output_1.data, indices_output_2.data
+        };
+        const size_t bytes = sasaw_segments::vjp_workspace_bytes(shape, want_W);
+        void* workspace = bytes > 0 ? scratch(bytes) : nullptr;
+        sasaw_segments::vjp<scalar_t>(
+            grad_A.data, grad_B.data, grad_W.data, grad_output.data, A.data, B.data, C.data, W.data, indices,
+            shape, workspace, stream
+        );
+        finish_call(operation);
+        return;
+    }
     if (sasaw_mfma::supports(shape, sizeof(scalar_t))) {
         const sasaw_mfma::Indices indices{
             indices_A.data, indices_W_1.data, indices_W_2.data, indices_output_1.data, indices_output_2.data
@@ -881,6 +894,27 @@ void sasaw_vjp_no_alloc(
     const Sizes s = sizes_of(grad_output, A, B, C, W);
     const sasaw_mfma::Shape shape{s.n_nodes, s.n_edges, s.nA, s.L, s.N, s.n2, s.n3};
     const char* who = "mops_amd_sparse_accumulation_scatter_add_with_weights_vjp_no_alloc_f32: ";
+    const sasaw_mfma::Indices indices{
+        indices_A.data, indices_W_1.data, indices_W_2.data, indices_output_1.data, indices_output_2.data
+    };
+    if (s.L > 0 && sasaw_segments::vjp_supported(shape, sizeof(float), want_W)) {
+        // (the same kernels as the existing entry point takes for these shapes)
+        const size_t needed = sasaw_segments::vjp_workspace_bytes(shape, want_W);
+        if (needed > NO_ALLOC_SCRATCH_BYTES) {
+            throw std::runtime_error(
+                std::string(who) + "these shapes need " + std::to_string(needed) + " bytes of temporary memory, the "
+                "built-in array holds " + std::to_string(NO_ALLOC_SCRATCH_BYTES) + " (about " +
+                std::to_string(NO_ALLOC_SCRATCH_BYTES / 528 - 64) + " nodes); use "
+                "mops_cuda_sparse_accumulation_scatter_add_with_weights_vjp_f32"
+            );
+        }
+        sasaw_segments::vjp<float>(
+            grad_A.data, grad_B.data, grad_W.data, grad_output.data, A.data, B.data, C.data, W.data, indices, shape,
+            no_alloc_scratch_of_current_device(), current_stream()
+        );
+        finish_call(operation);
+        return;
+    }
     if (!sasaw_mfma::supports(shape, sizeof(float))) {
         throw std::runtime_error(
             std::string(who) + "only the shapes of the matrix-core kernels are served without allocation (at least "
@@ -890,9 +924,8 @@ void sasaw_vjp_no_alloc(
     }
     if (!sasaw_mfma::vjp_allocates_nothing(shape, sizeof(float), want_edges, want_W)) {
         throw std::runtime_error(
-            std::string(who) + "for this graph (more than 48 edges per node on average, or W.shape[1] and "
-            "output.shape[1] in different multiples of four) grad_W is computed beside the other gradients on a "
-            "second stream, which this entry point cannot create; use "
+            std::string(who) + "for this graph (more than 48 edges per node on average) grad_W is computed beside "
+            "the other gradients on a second stream, which this entry point cannot create; use "
             "mops_cuda_sparse_accumulation_scatter_add_with_weights_vjp_f32, or ask for grad_W in a call of its own"
         );
     }
@@ -906,9 +939,6 @@ void sasaw_vjp_no_alloc(
         );
     }
     void* workspace = no_alloc_scratch_of_current_device();
-    const sasaw_mfma::Indices indices{
-        indices_A.data, indices_W_1.data, indices_W_2.data, indices_output_1.data, indices_output_2.data
-    };
     sasaw_mfma::vjp<float>(
         grad_A.data, grad_B.data, grad_W.data, grad_output.data, A.data, B.data, C.data, W.data, indices, shape,
         workspace, current_stream()

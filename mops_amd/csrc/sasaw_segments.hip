@@ -32,6 +32,7 @@
 
 #include <algorithm>
 #include <atomic>
+#include <cstdlib>
 #include <stdexcept>
 #include <type_traits>
 
@@ -84,15 +85,64 @@ template <typename T> __device__ __forceinline__ void place_of_component(int32_t
     }
 }
 
+/// The layouts the dense table is needed in. All are "what one lane of a
+/// wavefront holds as an operand of one matrix instruction, instruction after
+/// instruction", so that reading it is one conflict-free LDS access.
+enum class Layout : int32_t {
+    // result = D * sums (contract_kernel, and grad_W): see above
+    RESULT,
+    // grad_A: right operand of (grad_output of a node)^T * D[:, m2, :], per
+    // block row m2 and step s3 over the rows of the result:
+    //   table[((m2 * steps3 + s3) * 64 + 16 * k + m1] = D[4 * s3 + k, m2, m1]
+    ALPHA,
+    // grad_B: left operand of D' * (grad_output of a node), whose rows are
+    // pairs (component of A, block row) in the order the accumulators of the
+    // next product want them: pair p = s * bucket + m2 (s = m1 / 4) lies in
+    // tile p / 4, register p % 4, of the lanes q = m1 % 4:
+    //   table[((p / 4) * steps3 + s3) * 64 + 16 * k + row(q, p % 4)] = D[4 * s3 + k, m2, m1]
+    BETA
+};
+
 struct Table {
     const int32_t* PA;   // [N]
     const int32_t* Pred; // [N] index of the block row that is summed over (forward: PW2)
     const int32_t* Pout; // [N] index of the row of the result (forward: PO2)
     int32_t N, nA, n_red, n_out;
     int32_t registers; // ceil(nA / 4)
+    Layout layout;
+    int32_t bucket; // BETA: accumulator tiles of the kernel (>= n_red)
 
-    __host__ __device__ int32_t slots() const { return registers * n_red * WAVE; }
+    __host__ __device__ int32_t steps3() const { return (n_out + 3) / 4; }
+    __host__ __device__ int32_t slots() const {
+        switch (layout) {
+        case Layout::ALPHA:
+            return n_red * steps3() * WAVE;
+        case Layout::BETA:
+            return (registers * bucket + 3) / 4 * steps3() * WAVE;
+        default:
+            return registers * n_red * WAVE;
+        }
+    }
 };
+
+/// Where D[o, c, m1] goes (all three inside their ranges).
+template <typename T> __device__ __forceinline__ int32_t slot_in(const Table& t, int32_t m1, int32_t c, int32_t o) {
+    switch (t.layout) {
+    case Layout::ALPHA:
+        return (c * t.steps3() + (o >> 2)) * WAVE + 16 * (o & 3) + m1;
+    case Layout::BETA: {
+        const int32_t pair = (m1 >> 2) * t.bucket + c;
+        const int q = m1 & 3, r = pair & 3;
+        const int row = sizeof(T) == 4 ? 4 * q + r : 4 * r + q;
+        return ((pair >> 2) * t.steps3() + (o >> 2)) * WAVE + 16 * (o & 3) + row;
+    }
+    default: {
+        int q, r;
+        place_of_component<T>(m1, t.registers, q, r);
+        return (r * t.n_red + c) * WAVE + 16 * q + o;
+    }
+    }
+}
 
 constexpr int32_t NOBODY = 0x7fffffff;
 
@@ -152,9 +202,7 @@ __device__ __forceinline__ void build_table(
             const int32_t n = first + lane + k * WAVE;
             const bool inside = n < t.N && in_bounds(mine.m1[k], t.nA) && in_bounds(mine.c[k], t.n_red) &&
                                 in_bounds(mine.o[k], t.n_out);
-            int q, r;
-            place_of_component<T>(inside ? mine.m1[k] : 0, t.registers, q, r);
-            slot[k] = inside ? (r * t.n_red + mine.c[k]) * WAVE + 16 * q + mine.o[k] : -1;
+            slot[k] = inside ? slot_in<T>(t, mine.m1[k], mine.c[k], mine.o[k]) : -1;
             pending |= inside ? 1u << k : 0u;
         }
         // Every round the smallest pending entry of each slot is added to it: the
@@ -205,22 +253,7 @@ template <typename T> struct Contraction {
 /// Edges whose operands a wavefront asks for together: STEPS steps of four.
 /// (Two sets of operands are in registers at a time: one being multiplied,
 /// one on its way.)
-#ifndef MOPS_SEG_STEPS_F32
-#define MOPS_SEG_STEPS_F32 1
-#endif
-#ifndef MOPS_SEG_STEPS_F64
-#define MOPS_SEG_STEPS_F64 1
-#endif
-#ifndef MOPS_SEG_DOUBLE_BUFFER
-#define MOPS_SEG_DOUBLE_BUFFER 1
-#endif
-#ifndef MOPS_SEG_INNER_BARRIER
-#define MOPS_SEG_INNER_BARRIER 0
-#endif
-#ifndef MOPS_SEG_AHEAD
-#define MOPS_SEG_AHEAD 2
-#endif
-template <typename T> constexpr int steps_in_flight() { return sizeof(T) == 4 ? MOPS_SEG_STEPS_F32 : MOPS_SEG_STEPS_F64; }
+template <typename T> constexpr int steps_in_flight() { return 1; }
 
 /// A tensor as a buffer: loads are a uniform descriptor, a 32-bit byte offset
 /// per lane and a uniform byte offset (the hardware adds the three), and an
@@ -244,13 +277,62 @@ template <typename T> struct BufferOf {
 };
 constexpr uint32_t BEYOND = 0xffffffffu; // a byte offset no tensor reaches (the host sends larger ones elsewhere)
 
+/// The value, in a way the compiler cannot see through. What a kernel with
+/// several roles derives from the lane number for ONE role would otherwise be
+/// computed once in front of the loop over the units of work and kept in
+/// registers through all roles: dozens of registers per role, and spills.
+__device__ __forceinline__ int opaque(int value) {
+    asm volatile("" : "+v"(value));
+    return value;
+}
+
+/// All ones unless `wanted`: OR-ed into a byte offset it makes the load read
+/// zero. (Arithmetic instead of a choice between an offset and a constant: the
+/// compiler turns such a choice in front of a load into two branches.)
+__device__ __forceinline__ uint32_t unless(bool wanted) { return static_cast<uint32_t>(wanted) - 1u; }
+
+/// Four consecutive elements. VECTORS: as 16-byte loads (the tensor's rows must
+/// then be a multiple of four elements long and start on 16-byte boundaries,
+/// so that the four are inside or outside a row together); otherwise one by
+/// one, each with its own limit `inside` (elements from which on there is nothing).
+template <typename T, bool VECTORS>
+__device__ __forceinline__ void load_four(
+    T (&to)[4], const BufferOf<T>& buffer, uint32_t lane_bytes, uint32_t uniform_bytes, int32_t inside, uint32_t mask
+) {
+    if constexpr (VECTORS) {
+        const uint32_t at = lane_bytes | mask | unless(inside > 0);
+        if constexpr (sizeof(T) == 4) {
+            const auto raw = __builtin_amdgcn_raw_buffer_load_b128(buffer.descriptor, at, uniform_bytes, 0);
+            to[0] = __builtin_bit_cast(T, static_cast<uint32_t>(raw[0]));
+            to[1] = __builtin_bit_cast(T, static_cast<uint32_t>(raw[1]));
+            to[2] = __builtin_bit_cast(T, static_cast<uint32_t>(raw[2]));
+            to[3] = __builtin_bit_cast(T, static_cast<uint32_t>(raw[3]));
+        } else {
+#pragma unroll
+            for (int half = 0; half < 2; half++) {
+                const auto raw =
+                    __builtin_amdgcn_raw_buffer_load_b128(buffer.descriptor, at, uniform_bytes + 16 * half, 0);
+                typedef uint32_t Two __attribute__((ext_vector_type(2)));
+                to[2 * half] = __builtin_bit_cast(T, Two{raw[0], raw[1]});
+                to[2 * half + 1] = __builtin_bit_cast(T, Two{raw[2], raw[3]});
+            }
+        }
+    } else {
+#pragma unroll
+        for (int v = 0; v < 4; v++) {
+            to[v] = buffer.load((lane_bytes + v * static_cast<uint32_t>(sizeof(T))) | mask | unless(v < inside), uniform_bytes);
+        }
+    }
+}
+
 /// What a wavefront keeps for one node. NB = accumulator tiles: the block rows
 /// n_red, or (EXACT false) a bucket above them.
-template <typename T, int NB, bool EXACT> struct NodeSum {
+template <typename T, int NB, bool EXACT, bool COMPACT = false> struct NodeSum {
     using M = Mfma<T>;
     static constexpr int STEPS = steps_in_flight<T>();
 
     const Contraction<T>& p;
+    int32_t registers_of_A; // ceil(nA / 4)
     int lane, i, q;
     int32_t column;       // of the feature axis, this lane's
     bool column_inside;
@@ -269,14 +351,9 @@ template <typename T, int NB, bool EXACT> struct NodeSum {
         T w[STEPS][NB];
     };
 
-    __device__ __forceinline__ NodeSum(const Contraction<T>& contraction, int32_t registers) : p(contraction) {
-        lane = threadIdx.x & (WAVE - 1);
-        i = lane & 15;
-        q = lane >> 4;
+    __device__ __forceinline__ NodeSum(const Contraction<T>& contraction, int32_t registers)
+        : p(contraction), registers_of_A(registers) {
         set_column_tile(0);
-        const int32_t component = component_of_row<T>(i, registers);
-        component_bytes = static_cast<uint32_t>(component < p.nA ? component : 0) * sizeof(T);
-        component_mask = component < p.nA ? 0u : BEYOND;
         row_bytes = static_cast<uint32_t>(p.ld) * sizeof(T);
         block_bytes = static_cast<uint32_t>(p.n_red) * row_bytes;
         a_row_bytes = static_cast<uint32_t>(p.nA) * sizeof(T);
@@ -287,6 +364,12 @@ template <typename T, int NB, bool EXACT> struct NodeSum {
 
     /// The 16 columns of the feature axis this wavefront works on next.
     __device__ __forceinline__ void set_column_tile(int32_t column_tile) {
+        lane = opaque(static_cast<int>(threadIdx.x & (WAVE - 1)));
+        i = lane & 15;
+        q = lane >> 4;
+        const int32_t component = component_of_row<T>(i, registers_of_A);
+        component_bytes = static_cast<uint32_t>(component < p.nA ? component : 0) * sizeof(T);
+        component_mask = component < p.nA ? 0u : BEYOND;
         column = 16 * column_tile + i;
         column_inside = column < p.L;
         column_bytes = static_cast<uint32_t>(min(column, p.L - 1)) * sizeof(T);
@@ -341,9 +424,6 @@ template <typename T, int NB, bool EXACT> struct NodeSum {
             for (int c = 0; c < NB; c++) {
                 right[c] = from.w[u][c] * from.b[u];
             }
-#if MOPS_SEG_INNER_BARRIER
-            __builtin_amdgcn_sched_barrier(0);
-#endif
 #pragma unroll
             for (int c = 0; c < NB; c++) {
                 if (has_row(c)) { // (uniform)
@@ -360,14 +440,6 @@ template <typename T, int NB, bool EXACT> struct NodeSum {
     /// condition makes every later wait a wait for all loads.
     __device__ __forceinline__ void add(int32_t edges, int32_t sources, int32_t n) {
         constexpr int BATCH = 4 * STEPS;
-#if !MOPS_SEG_DOUBLE_BUFFER
-        for (int32_t done = 0; done < n; done += BATCH) {
-            Operands operands;
-            load(operands, edges, sources, done);
-            multiply(operands);
-        }
-        return;
-#endif
         // Unrolled over all batches a list of 64 can have, with an early way out:
         // in straight-line code the compiler counts the loads in flight exactly
         // (around a loop it waits for the oldest ones at the top of every round,
@@ -376,8 +448,33 @@ template <typename T, int NB, bool EXACT> struct NodeSum {
         // instructions of this one. AHEAD batches are on their way while one is
         // multiplied: a round trip to memory lasts several times as long as the
         // matrix instructions of a batch.
-        constexpr int AHEAD = MOPS_SEG_AHEAD;
+        constexpr int AHEAD = 2;
         constexpr int BATCHES = WAVE / BATCH;
+        if constexpr (COMPACT) {
+            // (a kernel with other roles beside this one: the same in rounds of
+            // four batches, a quarter of the code)
+            constexpr int ROUND = 4;
+            for (int32_t done = 0; done < n; done += ROUND * BATCH) {
+                Operands ring[AHEAD + 1];
+#pragma unroll
+                for (int b = 0; b < AHEAD; b++) {
+                    load(ring[b], edges, sources, done + b * BATCH);
+                }
+#pragma unroll
+                for (int b = 0; b < ROUND; b++) {
+                    if (b + AHEAD < ROUND) {
+                        load(ring[(b + AHEAD) % (AHEAD + 1)], edges, sources, done + (b + AHEAD) * BATCH);
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                    multiply(ring[b % (AHEAD + 1)]);
+                    __builtin_amdgcn_sched_barrier(0);
+                    if (done + (b + 1) * BATCH >= n) {
+                        break;
+                    }
+                }
+            }
+            return;
+        }
         Operands ring[AHEAD + 1];
 #pragma unroll
         for (int b = 0; b < AHEAD; b++) {
@@ -435,14 +532,68 @@ template <typename T, int NB, bool EXACT> struct NodeSum {
     }
 };
 
-#ifdef MOPS_SEG_TRACE
-__device__ long long seg_trace[8192 * 8];
-#define MOPS_TRACE_SET(k, v) do { if (lane == 0) seg_trace[(group * 16 + wave) * 8 + (k)] = (v); } while (0)
-#define MOPS_TRACE_CODE(...) __VA_ARGS__
-#else
-#define MOPS_TRACE_SET(k, v)
-#define MOPS_TRACE_CODE(...)
-#endif
+/// The sums of NODE `node` from its slots (sender_buckets.hpp): `first_half` and
+/// `second_half` are the node's 128 places (lane k: places k and k + 64),
+/// `part_counts` the numbers of edges in its four parts; `listed_index` the
+/// index the slots were listed from, read in full by a node whose slots
+/// overflowed. Returns whether the node has edges at all.
+template <typename Sum>
+__device__ __forceinline__ bool sum_over_slots(
+    Sum& sum, int32_t first_half, int32_t second_half, int4 part_counts, const int32_t* __restrict__ listed_index,
+    int32_t node, int lane
+) {
+    const auto& p = sum.p;
+    sum.clear();
+    bool any = false;
+    // lane k of `edges` holds edge k of n <= 64
+    auto hand_on = [&](int32_t edges, int32_t n) {
+        const int32_t mine = lane < n ? edges : -1;
+        const int32_t sources = load_or_zero(p.gather_index, static_cast<size_t>(max(mine, 0)), mine >= 0);
+        sum.add(mine, mine >= 0 ? sources : -1, n);
+        any = true;
+    };
+    static_assert(SLOT_PARTS == 4 && SLOT_CAPACITY == 2 * WAVE, "the four parts of a node's places in two registers");
+    const int32_t c0 = __builtin_amdgcn_readfirstlane(part_counts.x);
+    const int32_t c1 = __builtin_amdgcn_readfirstlane(part_counts.y);
+    const int32_t c2 = __builtin_amdgcn_readfirstlane(part_counts.z);
+    const int32_t c3 = __builtin_amdgcn_readfirstlane(part_counts.w);
+    const int32_t count = c0 + c1 + c2 + c3;
+    if (max(max(c0, c1), max(c2, c3)) <= SLOT_PART_CAPACITY) {
+        // the parts moved together: position k of the list is in part `part`, place k - before
+        auto edge_at = [&](int32_t position) {
+            const int32_t part =
+                (position >= c0 ? 1 : 0) + (position >= c0 + c1 ? 1 : 0) + (position >= c0 + c1 + c2 ? 1 : 0);
+            const int32_t before = part == 0 ? 0 : part == 1 ? c0 : part == 2 ? c0 + c1 : c0 + c1 + c2;
+            const int32_t place = part * SLOT_PART_CAPACITY + position - before;
+            const int32_t low = __shfl(first_half, place & (WAVE - 1));
+            const int32_t high = __shfl(second_half, place & (WAVE - 1));
+            return place < WAVE ? low : high;
+        };
+        if (count > 0) {
+            hand_on(edge_at(lane), min(count, WAVE));
+        }
+        if (count > WAVE) {
+            hand_on(edge_at(lane + WAVE), count - WAVE);
+        }
+    } else {
+        // more edges in a part than places (a hub of a sparse graph): this
+        // wavefront reads the whole index itself
+        const unsigned long long below = (1ull << lane) - 1ull;
+        for (int32_t base = 0; base < p.n_edges; base += WAVE) {
+            const int32_t e = base + lane;
+            const bool named = e < p.n_edges && listed_index[min(e, p.n_edges - 1)] == node;
+            const unsigned long long mask = __ballot(named);
+            if (mask != 0) {
+                // the matches moved to the first lanes, in edge order
+                const int32_t n = __popcll(mask);
+                const int32_t named_below = __popcll(mask & below);
+                const int32_t place = named ? named_below : n + lane - named_below;
+                hand_on(__builtin_amdgcn_ds_permute(place << 2, e), n);
+            }
+        }
+    }
+    return any;
+}
 
 /// Where the edges of a node come from.
 enum class Source {
@@ -509,8 +660,6 @@ __global__ __launch_bounds__((group_threads<T, NB>())) void contract_kernel(cons
     const int32_t group = static_cast<int32_t>(blockIdx.x);
     const int32_t n_groups = static_cast<int32_t>(gridDim.x);
     NodeSum<T, NB, EXACT> sum(p, registers);
-    MOPS_TRACE_CODE(long long t_start = clock64(); long long t_add = 0, t_finish = 0, t_turn = 0, t_mark = 0; int n_units_done = 0, n_edges_done = 0;)
-
     // turn k of this workgroup is unit group + k * n_groups
     auto unit_of_turn = [&](int32_t turn) { return group + turn * n_groups; };
     auto take_turn = [&]() {
@@ -575,73 +724,21 @@ __global__ __launch_bounds__((group_threads<T, NB>())) void contract_kernel(cons
             table_seen = true;
         }
     };
-    MOPS_TRACE_CODE(long long t_built = clock64();)
 
     while (unit < args.n_units) {
-        MOPS_TRACE_CODE(n_units_done++; t_mark = clock64();)
         const int32_t next_unit = unit_of_turn(take_turn());
         UnitAhead<SOURCE> next;
         look_ahead(next, next_unit);
-        MOPS_TRACE_CODE(t_turn += clock64() - t_mark;)
-
         const int32_t item = unit / p.column_tiles;
         sum.set_column_tile(unit - item * p.column_tiles);
         if constexpr (SOURCE == Source::SLOTS) {
-            const int32_t node = item;
-            sum.clear();
-            bool any = false;
-            // lane k of `edges` holds edge k of n <= 64
-            auto hand_on = [&](int32_t edges, int32_t n) {
-                const int32_t mine = lane < n ? edges : -1;
-                const int32_t sources = load_or_zero(p.gather_index, static_cast<size_t>(max(mine, 0)), mine >= 0);
-                sum.add(mine, mine >= 0 ? sources : -1, n);
-                any = true;
-            };
-            static_assert(SLOT_PARTS == 4 && SLOT_CAPACITY == 2 * WAVE, "the four parts of a node's places in two registers");
-            const int32_t c0 = __builtin_amdgcn_readfirstlane(current.part_counts.x);
-            const int32_t c1 = __builtin_amdgcn_readfirstlane(current.part_counts.y);
-            const int32_t c2 = __builtin_amdgcn_readfirstlane(current.part_counts.z);
-            const int32_t c3 = __builtin_amdgcn_readfirstlane(current.part_counts.w);
-            const int32_t count = c0 + c1 + c2 + c3;
-            if (max(max(c0, c1), max(c2, c3)) <= SLOT_PART_CAPACITY) {
-                // the parts moved together: position k of the list is in part `part`, place k - before
-                auto edge_at = [&](int32_t position) {
-                    const int32_t part = (position >= c0 ? 1 : 0) + (position >= c0 + c1 ? 1 : 0) +
-                                         (position >= c0 + c1 + c2 ? 1 : 0);
-                    const int32_t before = part == 0 ? 0 : part == 1 ? c0 : part == 2 ? c0 + c1 : c0 + c1 + c2;
-                    const int32_t place = part * SLOT_PART_CAPACITY + position - before;
-                    const int32_t low = __shfl(current.first_half, place & (WAVE - 1));
-                    const int32_t high = __shfl(current.second_half, place & (WAVE - 1));
-                    return place < WAVE ? low : high;
-                };
-                if (count > 0) {
-                    hand_on(edge_at(lane), min(count, WAVE));
-                }
-                if (count > WAVE) {
-                    hand_on(edge_at(lane + WAVE), count - WAVE);
-                }
-            } else {
-                // more edges in a part than places (a hub of a sparse graph): this
-                // wavefront reads the whole index itself
-                const unsigned long long below = (1ull << lane) - 1ull;
-                for (int32_t base = 0; base < p.n_edges; base += WAVE) {
-                    const int32_t e = base + lane;
-                    const bool named = e < p.n_edges && args.listed_index[min(e, p.n_edges - 1)] == node;
-                    const unsigned long long mask = __ballot(named);
-                    if (mask != 0) {
-                        // the matches moved to the first lanes, in edge order
-                        const int32_t n = __popcll(mask);
-                        const int32_t named_below = __popcll(mask & below);
-                        const int32_t place = named ? named_below : n + lane - named_below;
-                        hand_on(__builtin_amdgcn_ds_permute(place << 2, e), n);
-                    }
-                }
-            }
-            if (any) {
+            if (sum_over_slots(
+                    sum, current.first_half, current.second_half, current.part_counts, args.listed_index, item, lane
+                )) {
                 wait_for_table();
-                sum.finish(table, registers, node);
+                sum.finish(table, registers, item);
             } else {
-                sum.clear_rows(node, node + 1);
+                sum.clear_rows(item, item + 1);
             }
         } else {
             const int32_t chunk_begin = item * CHUNK;
@@ -649,7 +746,6 @@ __global__ __launch_bounds__((group_threads<T, NB>())) void contract_kernel(cons
                 args.sorted_index, p.n_edges, p.n_blocks, item, current.index,
                 [&](int32_t node, int32_t first, int32_t last) {
                     sum.clear();
-                    MOPS_TRACE_CODE(long long t0 = clock64(); n_edges_done += last - first;)
                     for (int32_t base = first; base < last; base += WAVE) {
                         const int32_t n = min(WAVE, last - base);
                         const int32_t offset = base - chunk_begin; // >= 0: owned segments start in the chunk
@@ -665,10 +761,8 @@ __global__ __launch_bounds__((group_threads<T, NB>())) void contract_kernel(cons
                         }
                         sum.add(edges, edges >= 0 ? sources : -1, n);
                     }
-                    MOPS_TRACE_CODE(long long t1 = clock64(); t_add += t1 - t0;)
                     wait_for_table();
                     sum.finish(table, registers, node);
-                    MOPS_TRACE_CODE(t_finish += clock64() - t1;)
                 },
                 [&](int32_t begin, int32_t end) { sum.clear_rows(begin, end); }
             );
@@ -676,14 +770,480 @@ __global__ __launch_bounds__((group_threads<T, NB>())) void contract_kernel(cons
         unit = next_unit;
         current = next;
     }
-    MOPS_TRACE_SET(0, t_start);
-    MOPS_TRACE_SET(1, t_built);
-    MOPS_TRACE_SET(2, clock64());
-    MOPS_TRACE_SET(3, n_units_done);
-    MOPS_TRACE_SET(4, t_add);
-    MOPS_TRACE_SET(5, t_finish);
-    MOPS_TRACE_SET(6, t_turn);
-    MOPS_TRACE_SET(7, n_edges_done);
+}
+
+// ---------------------------------------------------------------------------
+// grad_A and grad_B
+//
+// With G = grad_output, i the receiver of edge e and j its sender:
+//
+//   Z'_i[m1, m2, l] = sum_m3 D[m3, m2, m1] * G[i, m3, l]          once per node i (segment of the sorted index)
+//   grad_A[e, m1]   = sum_{m2, l} Z'_i[m1, m2, l] * (B[e, l] * W[j, m2, l])
+//   grad_B[e, l]    = sum_m2 W[j, m2, l] * sum_m1 A[e, m1] * Z'_i[m1, m2, l]
+//
+// Both are matrix products with 16 edges of the segment as one dimension and
+// Z'_i, which all edges of the segment share, as one operand. Z'_i is itself a
+// product of the dense table with G[i] and comes out of the matrix cores in
+// exactly the register layout the next product wants it in (that is what the
+// layouts ALPHA and BETA of the table are for), so nothing goes through LDS.
+//   grad_B of a tile of 16 columns l:   Z' as 16 columns x pairs (m1, m2): 27 steps per 16 edges (nA = n2 = 9)
+//   grad_A, 16 columns l at a time:     Z' as m1 x (m2, l):                36 steps per 16 edges and 16 columns
+// A wavefront does one of these for all segments that start in a chunk of 16
+// positions: the roles are units of work of the same kind as in contract_kernel.
+
+template <typename T> struct GradientArgs {
+    const T* A;  // [n_edges][nA]
+    const T* B;  // [n_edges][L]
+    const T* W;  // [n_nodes][n2][L]
+    const T* G;  // [n_nodes][n3][L]  grad_output
+    const T* C;  // [N]
+    T* grad_A;   // null: not wanted
+    T* grad_B;
+    T* grad_W;
+    const int32_t* receivers; // sorted
+    const int32_t* senders;
+    int32_t n_edges, n_nodes, nA, L, n2, n3, column_tiles;
+    Table table_W, table_alpha, table_beta;
+    int32_t edge_roles;   // units per chunk: (grad_A ? 1 : 0) + (grad_B ? column_tiles : 0)
+    int32_t edge_chunk;   // positions of the sorted index per unit of the per-edge gradients: 16, 32 or 64
+    int32_t n_edge_units; // chunks * edge_roles
+    int32_t n_W_units;    // n_nodes * column_tiles when grad_W is wanted; these units come last (measured: 6 to 10 us
+                          // slower at 60 000 edges when they come first)
+    int32_t n_units;      // the sum
+    const int32_t* slot_edges;
+    const int32_t* slot_counts;
+};
+
+template <typename T, int NB, bool EXACT, bool VECTORS> struct EdgeGradients {
+    using M = Mfma<T>;
+    static constexpr uint32_t ELEMENT = sizeof(T);
+
+    const GradientArgs<T>& p;
+    int lane, i, q;
+    int32_t steps1, steps3; // ceil(nA / 4), ceil(n3 / 4)
+    uint32_t row_bytes, w_block_bytes, g_block_bytes, a_row_bytes;
+    BufferOf<T> A, B, W, G;
+
+    __device__ __forceinline__ EdgeGradients(const GradientArgs<T>& args) : p(args) {
+        lane = threadIdx.x & (WAVE - 1);
+        i = lane & 15;
+        q = lane >> 4;
+        steps1 = (p.nA + 3) / 4;
+        steps3 = (p.n3 + 3) / 4;
+        row_bytes = static_cast<uint32_t>(p.L) * ELEMENT;
+        w_block_bytes = static_cast<uint32_t>(p.n2) * row_bytes;
+        g_block_bytes = static_cast<uint32_t>(p.n3) * row_bytes;
+        a_row_bytes = static_cast<uint32_t>(p.nA) * ELEMENT;
+        A.set(p.A, static_cast<uint32_t>(p.n_edges) * a_row_bytes);
+        B.set(p.B, static_cast<uint32_t>(p.n_edges) * row_bytes);
+        W.set(p.W, static_cast<uint32_t>(p.n_nodes) * w_block_bytes);
+        G.set(p.G, static_cast<uint32_t>(p.n_nodes) * g_block_bytes);
+    }
+
+    __device__ __forceinline__ bool has_row(int c) const { return EXACT || c < p.n2; }
+
+    /// grad_B[e, 16 tile .. 16 tile + 16] for the edges first .. last of `node`.
+    /// `near_source`: senders of the 128 positions from `near_begin`.
+    __device__ __forceinline__ void grad_B_of_segment(
+        const T* __restrict__ table, int32_t node, int32_t first, int32_t last, int32_t tile,
+        const int32_t (&near_source)[2], int32_t near_begin
+    ) const {
+        const int lane = opaque(this->lane);
+        const int i = lane & 15, q = lane >> 4;
+        const int32_t column = 16 * tile + i;
+        const bool column_inside = column < p.L;
+        const uint32_t column_bytes = static_cast<uint32_t>(min(column, p.L - 1)) * ELEMENT;
+        // Z'_i as right operand: lane (column, q) holds, for pair (s, m2), Z'[4 s + q, m2, column]
+        T g_rows[4];
+#pragma unroll
+        for (int s3 = 0; s3 < 4; s3++) {
+            const int32_t m3 = 4 * s3 + q;
+            g_rows[s3] = G.load(
+                (static_cast<uint32_t>(node) * g_block_bytes + static_cast<uint32_t>(min(m3, p.n3 - 1)) * row_bytes +
+                 column_bytes) |
+                    unless(m3 < p.n3 && column_inside),
+                0
+            );
+        }
+        const int32_t pair_tiles = (steps1 * NB + 3) / 4;
+        typename M::Acc pairs[NB]; // (4 * NB pairs at most)
+#pragma unroll
+        for (int t = 0; t < NB; t++) {
+            pairs[t] = M::zero();
+            if (t < pair_tiles) { // (uniform)
+#pragma unroll
+                for (int s3 = 0; s3 < 4; s3++) {
+                    if (s3 < steps3) {
+                        pairs[t] = M::mma(table[(t * steps3 + s3) * WAVE + lane], g_rows[s3], pairs[t]);
+                    }
+                }
+            }
+        }
+        for (int32_t base = first; base < last; base += 16) {
+            const int32_t n = min(16, last - base);
+            // the edge of row `row` of the tile, and its sender
+            auto edge_of_row = [&](int row, int32_t& edge, int32_t& sender) {
+                const int32_t position = base + row;
+                edge = row < n ? position : -1;
+                const int32_t offset = position - near_begin;
+                if (base + 15 - near_begin < 2 * WAVE) { // (uniform: the whole tile is at hand)
+                    const int32_t s0 = __shfl(near_source[0], offset & (WAVE - 1));
+                    const int32_t s1 = __shfl(near_source[1], offset & (WAVE - 1));
+                    sender = offset < WAVE ? s0 : s1;
+                } else {
+                    sender = load_or_zero(p.senders, static_cast<size_t>(max(edge, 0)), edge >= 0);
+                }
+            };
+            // left operand: lane (edge i, q) holds A[edge, 4 s + q]
+            int32_t my_edge, my_sender;
+            edge_of_row(i, my_edge, my_sender);
+            T a_rows[4];
+#pragma unroll
+            for (int s = 0; s < 4; s++) {
+                const int32_t m1 = 4 * s + q;
+                a_rows[s] = A.load(
+                    (static_cast<uint32_t>(max(my_edge, 0)) * a_row_bytes + static_cast<uint32_t>(min(m1, p.nA - 1)) * ELEMENT) |
+                        unless(my_edge >= 0 && m1 < p.nA),
+                    0
+                );
+            }
+            // the rows of W of the four edges this lane holds results for
+            int32_t row_edge[4];
+            T w[4][NB];
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                int32_t sender;
+                edge_of_row(M::row(lane, r), row_edge[r], sender);
+                const bool usable = row_edge[r] >= 0 && in_bounds(sender, p.n_nodes) && column_inside;
+                const uint32_t from =
+                    (static_cast<uint32_t>(usable ? sender : 0) * w_block_bytes + column_bytes) | unless(usable);
+#pragma unroll
+                for (int c = 0; c < NB; c++) {
+                    w[r][c] = W.load(from, static_cast<uint32_t>(EXACT ? c : min(c, p.n2 - 1)) * row_bytes);
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            // Y'[edge, m2, column] = sum_m1 A[edge, m1] Z'[m1, m2, column]
+            T result[4] = {T(0), T(0), T(0), T(0)};
+#pragma unroll
+            for (int c = 0; c < NB; c++) {
+                if (has_row(c)) {
+                    typename M::Acc y = M::zero();
+#pragma unroll
+                    for (int s = 0; s < 4; s++) {
+                        if (s < steps1) {
+                            y = M::mma(a_rows[s], pairs[(s * NB + c) >> 2][(s * NB + c) & 3], y);
+                        }
+                    }
+#pragma unroll
+                    for (int r = 0; r < 4; r++) {
+                        result[r] += y[r] * w[r][c];
+                    }
+                }
+            }
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                if (row_edge[r] >= 0 && column_inside) {
+                    p.grad_B[static_cast<size_t>(row_edge[r]) * p.L + column] = result[r];
+                }
+            }
+        }
+    }
+
+    /// grad_A[e, :] for the edges first .. last of `node`.
+    __device__ __forceinline__ void grad_A_of_segment(
+        const T* __restrict__ table, int32_t node, int32_t first, int32_t last, const int32_t (&near_source)[2],
+        int32_t near_begin
+    ) const {
+        constexpr int TILES = 4; // tiles of 16 edges whose sums over the columns are in registers together
+        const int lane = opaque(this->lane);
+        const int i = lane & 15, q = lane >> 4;
+        // row `row` of a tile of Z' stands for column 4 q + r of the 16 (the lane
+        // that holds it, and the register): consecutive columns in one lane
+        const int local_column = sizeof(T) == 4 ? i : 4 * (i & 3) + (i >> 2);
+        for (int32_t base = first; base < last; base += 16 * TILES) {
+            const int32_t n = min(16 * TILES, last - base);
+            const int32_t n_tiles = (n + 15) / 16;
+            // the edge of this lane's column of tile t, and its sender
+            int32_t my_edge[TILES], my_sender[TILES];
+#pragma unroll
+            for (int t = 0; t < TILES; t++) {
+                const int32_t position = base + 16 * t + i;
+                my_edge[t] = 16 * t + i < n ? position : -1;
+                const int32_t offset = position - near_begin;
+                if (base + 16 * t + 15 - near_begin < 2 * WAVE) { // (uniform: the whole tile is at hand)
+                    const int32_t s0 = __shfl(near_source[0], offset & (WAVE - 1));
+                    const int32_t s1 = __shfl(near_source[1], offset & (WAVE - 1));
+                    my_sender[t] = offset < WAVE ? s0 : s1;
+                } else {
+                    my_sender[t] = load_or_zero(p.senders, static_cast<size_t>(max(my_edge[t], 0)), my_edge[t] >= 0);
+                }
+            }
+            typename M::Acc sums[TILES];
+#pragma unroll
+            for (int t = 0; t < TILES; t++) {
+                sums[t] = M::zero();
+            }
+            for (int32_t tile = 0; tile < p.column_tiles; tile++) {
+                // Z'_i of these 16 columns as left operand: lane (m1, q), register r of
+                // tile m2: Z'[m1, m2, 16 tile + 4 q + r]
+                T g_columns[4];
+                const int32_t column = 16 * tile + local_column;
+#pragma unroll
+                for (int s3 = 0; s3 < 4; s3++) {
+                    const int32_t m3 = 4 * s3 + q;
+                    g_columns[s3] = G.load(
+                        (static_cast<uint32_t>(node) * g_block_bytes +
+                         static_cast<uint32_t>(min(m3, p.n3 - 1)) * row_bytes +
+                         static_cast<uint32_t>(min(column, p.L - 1)) * ELEMENT) |
+                            unless(m3 < p.n3 && column < p.L),
+                        0
+                    );
+                }
+                typename M::Acc z[NB];
+#pragma unroll
+                for (int c = 0; c < NB; c++) {
+                    z[c] = M::zero();
+                    if (has_row(c)) {
+#pragma unroll
+                        for (int s3 = 0; s3 < 4; s3++) {
+                            if (s3 < steps3) {
+                                z[c] = M::mma(g_columns[s3], table[(c * steps3 + s3) * WAVE + lane], z[c]);
+                            }
+                        }
+                    }
+                }
+                const int32_t first_column = 16 * tile + 4 * q; // of this lane's four
+                const int32_t inside = p.L - first_column;      // columns from there on that exist
+#pragma unroll
+                for (int t = 0; t < TILES; t++) {
+                    if (t < n_tiles) { // (uniform)
+                        const bool usable = my_edge[t] >= 0 && in_bounds(my_sender[t], p.n_nodes);
+                        T b[4];
+                        load_four<T, VECTORS>(
+                            b, B,
+                            static_cast<uint32_t>(max(my_edge[t], 0)) * row_bytes +
+                                static_cast<uint32_t>(min(first_column, p.L - 1)) * ELEMENT,
+                            0, inside, unless(usable)
+                        );
+                        const uint32_t from = static_cast<uint32_t>(usable ? my_sender[t] : 0) * w_block_bytes +
+                                              static_cast<uint32_t>(min(first_column, p.L - 1)) * ELEMENT;
+                        T w[NB][4];
+#pragma unroll
+                        for (int c = 0; c < NB; c++) {
+                            load_four<T, VECTORS>(
+                                w[c], W, from, static_cast<uint32_t>(EXACT ? c : min(c, p.n2 - 1)) * row_bytes, inside,
+                                unless(usable)
+                            );
+                        }
+                        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                        for (int c = 0; c < NB; c++) {
+                            if (has_row(c)) {
+#pragma unroll
+                                for (int r = 0; r < 4; r++) {
+                                    sums[t] = M::mma(z[c][r], w[c][r] * b[r], sums[t]);
+                                }
+                            }
+                        }
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+                }
+            }
+#pragma unroll
+            for (int t = 0; t < TILES; t++) {
+                if (t < n_tiles && my_edge[t] >= 0) {
+#pragma unroll
+                    for (int r = 0; r < 4; r++) {
+                        const int32_t m1 = M::row(lane, r);
+                        if (m1 < p.nA) {
+                            p.grad_A[static_cast<size_t>(my_edge[t]) * p.nA + m1] = sums[t][r];
+                        }
+                    }
+                }
+            }
+        }
+    }
+};
+
+/// grad_A, grad_B and grad_W in one persistent launch (see contract_kernel for
+/// how the units of work are dealt out): the per-edge gradients of the segments
+/// that start in a chunk of 16, 32 or 64 positions, one unit for grad_A and one for
+/// every 16 columns of grad_B, then grad_W of a node from its slots, one unit for
+/// every 16 columns. Three wavefronts build the three layouts of the table side
+/// by side.
+/// Wavefronts per SIMD of the gradient kernel (it needs more registers than
+/// contract_kernel: Z' of a node, the rows of W of 16 edges and the sums).
+template <typename T, int NB> constexpr int gradient_waves_per_simd() { return sizeof(T) == 4 && NB <= 9 ? 3 : 2; }
+template <typename T, int NB> constexpr int gradient_group_threads() {
+    return 4 * gradient_waves_per_simd<T, NB>() * WAVE;
+}
+
+template <typename T, int NB, bool VECTORS>
+__global__ __launch_bounds__((gradient_group_threads<T, NB>())) void gradients_kernel(const GradientArgs<T> args) {
+    constexpr bool EXACT = false; // (the block rows are compared with n2 / n3 as the loops go)
+    constexpr int THREADS = gradient_group_threads<T, NB>();
+    constexpr int GROUP_WAVES = THREADS / WAVE;
+    static_assert(GROUP_WAVES >= 3, "a wavefront per layout of the table");
+    extern __shared__ __align__(16) char lds_raw[];
+    // the three layouts of the table, then an array of owners for each (build_table)
+    T* const table_W = reinterpret_cast<T*>(lds_raw);
+    T* const table_alpha = table_W + args.table_W.slots();
+    T* const table_beta = table_alpha + args.table_alpha.slots();
+    int32_t* const owner_W = reinterpret_cast<int32_t*>(table_beta + args.table_beta.slots());
+    int32_t* const owner_alpha = owner_W + args.table_W.slots();
+    int32_t* const owner_beta = owner_alpha + args.table_alpha.slots();
+    int32_t* next_turn = owner_beta + args.table_beta.slots();
+    int32_t* table_ready = next_turn + 1; // [3]: W, alpha, beta
+
+    const int lane = threadIdx.x & (WAVE - 1);
+    const int32_t wave = threadIdx.x >> 6;
+    const int32_t group = static_cast<int32_t>(blockIdx.x);
+    const int32_t n_groups = static_cast<int32_t>(gridDim.x);
+    const bool want_W = args.grad_W != nullptr, want_A = args.grad_A != nullptr, want_B = args.grad_B != nullptr;
+
+    Contraction<T> contraction;
+    contraction.A = args.A;
+    contraction.B = args.B;
+    contraction.rows = args.G;
+    contraction.gather_index = args.receivers;
+    contraction.result = args.grad_W;
+    contraction.n_edges = args.n_edges;
+    contraction.n_blocks = args.n_nodes;
+    contraction.nA = args.nA;
+    contraction.L = args.L;
+    contraction.ld = args.L;
+    contraction.n_red = args.n3;
+    contraction.n_out = args.n2;
+    contraction.column_tiles = args.column_tiles;
+    NodeSum<T, NB, EXACT, true> sum(contraction, args.table_W.registers);
+    EdgeGradients<T, NB, EXACT, VECTORS> edges(args);
+
+    auto unit_of_turn = [&](int32_t turn) { return group + turn * n_groups; };
+    auto take_turn = [&]() {
+        int32_t turn = 0;
+        if (lane == 0) {
+            turn = atomicAdd(next_turn, 1);
+        }
+        return __builtin_amdgcn_readfirstlane(turn);
+    };
+    // what is asked for ahead of a unit: of a chunk, the index values around
+    // it and the senders of the 128 positions from its first; of a node, its slots
+    struct Ahead {
+        int32_t v[6];
+    };
+    auto look_ahead = [&](Ahead& ahead, int32_t unit) {
+        const bool exists = unit < args.n_units;
+        if (!exists || unit < args.n_edge_units) {
+            const int32_t chunk = exists ? unit / args.edge_roles : 0;
+            const ChunkIndex index = load_chunk_index_of(args.receivers, args.n_edges, chunk, args.edge_chunk);
+            ahead.v[0] = index.mine;
+            ahead.v[1] = index.before;
+            ahead.v[2] = index.ahead;
+#pragma unroll
+            for (int h = 0; h < 2; h++) {
+                const int32_t position = chunk * args.edge_chunk + h * WAVE + lane;
+                const int32_t sender =
+                    load_or_zero(args.senders, static_cast<size_t>(position), position < args.n_edges);
+                ahead.v[3 + h] = position < args.n_edges ? sender : -1;
+            }
+            ahead.v[5] = 0;
+        } else {
+            const int32_t node = (unit - args.n_edge_units) / args.column_tiles;
+            const int32_t* mine = args.slot_edges + static_cast<size_t>(node) * SLOT_CAPACITY;
+            ahead.v[0] = mine[lane];
+            ahead.v[1] = mine[lane + WAVE];
+            const int4 counts = reinterpret_cast<const int4*>(args.slot_counts)[node];
+            ahead.v[2] = counts.x;
+            ahead.v[3] = counts.y;
+            ahead.v[4] = counts.z;
+            ahead.v[5] = counts.w;
+        }
+    };
+
+    int32_t unit = unit_of_turn(wave);
+    Ahead current;
+    MyEntries<T> entries;
+    // wavefront 0 builds the table of grad_W, 1 that of grad_A, 2 that of grad_B
+    const bool builder = (wave == 0 && want_W) || (wave == 1 && want_A) || (wave == 2 && want_B);
+    const Table& my_layout = wave == 0 ? args.table_W : wave == 1 ? args.table_alpha : args.table_beta;
+    if (builder) {
+        load_entries<T>(entries, args.C, my_layout, 0, lane);
+    }
+    look_ahead(current, unit);
+    if (threadIdx.x == 0) {
+        *next_turn = GROUP_WAVES;
+        table_ready[0] = 0;
+        table_ready[1] = 0;
+        table_ready[2] = 0;
+    }
+    __syncthreads(); // (everybody is here at once: nothing has been waited for yet)
+    bool seen_W = false, seen_alpha = false, seen_beta = false;
+    if (builder) {
+        T* my_table = wave == 0 ? table_W : wave == 1 ? table_alpha : table_beta;
+        int32_t* my_owner = wave == 0 ? owner_W : wave == 1 ? owner_alpha : owner_beta;
+        build_table<T>(my_table, my_owner, entries, args.C, my_layout, lane);
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+        if (lane == 0) {
+            __hip_atomic_store(&table_ready[wave], 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
+        }
+        seen_W = wave == 0;
+        seen_alpha = wave == 1;
+        seen_beta = wave == 2;
+    }
+    // (a builder depends on nobody, so the wait ends)
+    auto wait_for = [&](bool& seen, int which) {
+        if (!seen) {
+            while (__hip_atomic_load(&table_ready[which], __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP) == 0) {
+                __builtin_amdgcn_s_sleep(4);
+            }
+            seen = true;
+        }
+    };
+
+    while (unit < args.n_units) {
+        const int32_t next_unit = unit_of_turn(take_turn());
+        Ahead next;
+        look_ahead(next, next_unit);
+
+        if (unit < args.n_edge_units) {
+            const int32_t chunk = unit / args.edge_roles;
+            const int32_t role = unit - chunk * args.edge_roles;
+            const bool for_A = want_A && role == 0;
+            const int32_t tile = role - (want_A ? 1 : 0);
+            const ChunkIndex index{current.v[0], current.v[1], current.v[2]};
+            const int32_t near_source[2] = {current.v[3], current.v[4]};
+            if (for_A) {
+                wait_for(seen_alpha, 1);
+            } else {
+                wait_for(seen_beta, 2);
+            }
+            walk_pieces_of<0>(
+                args.receivers, args.n_edges, args.n_nodes, chunk, args.edge_chunk, index,
+                [&](int32_t node, int32_t first, int32_t last, bool, bool) {
+                    if (for_A) {
+                        edges.grad_A_of_segment(table_alpha, node, first, last, near_source, chunk * args.edge_chunk);
+                    } else {
+                        edges.grad_B_of_segment(table_beta, node, first, last, tile, near_source, chunk * args.edge_chunk);
+                    }
+                },
+                [&](int32_t, int32_t) {}
+            );
+        } else {
+            const int32_t item = unit - args.n_edge_units;
+            const int32_t node = item / args.column_tiles;
+            sum.set_column_tile(item - node * args.column_tiles);
+            const int4 counts = make_int4(current.v[2], current.v[3], current.v[4], current.v[5]);
+            if (sum_over_slots(sum, current.v[0], current.v[1], counts, args.senders, node, lane)) {
+                wait_for(seen_W, 0);
+                sum.finish(table_W, args.table_W.registers, node);
+            } else {
+                sum.clear_rows(node, node + 1);
+            }
+        }
+        unit = next_unit;
+        current = next;
+    }
 }
 
 // ---------------------------------------------------------------------------
@@ -703,6 +1263,8 @@ Table table_of(const Shape& s, const int32_t* PA, const int32_t* Pred, const int
     t.n_red = n_red;
     t.n_out = n_out;
     t.registers = (s.nA + 3) / 4;
+    t.layout = Layout::RESULT;
+    t.bucket = n_red;
     return t;
 }
 
@@ -710,6 +1272,9 @@ Table table_of(const Shape& s, const int32_t* PA, const int32_t* Pred, const int
 /// numbers of components of spherical harmonics up to some degree), otherwise
 /// rounded up to one of those.
 template <typename Launch> void with_block_rows(int32_t n_red, Launch&& launch) {
+#ifdef MOPS_SEG_DEV
+    launch(std::integral_constant<int, 9>{}, std::true_type{}); // (development builds: one size only)
+#else
     if (n_red == 1) {
         launch(std::integral_constant<int, 1>{}, std::true_type{});
     } else if (n_red == 4) {
@@ -725,6 +1290,7 @@ template <typename Launch> void with_block_rows(int32_t n_red, Launch&& launch) 
     } else {
         launch(std::integral_constant<int, 16>{}, std::false_type{});
     }
+#endif
 }
 
 template <typename Kernel> void allow_lds(Kernel kernel, size_t lds) {
@@ -832,16 +1398,6 @@ Contraction<T> contraction_of(
 
 } // namespace
 
-#ifdef MOPS_SEG_TRACE
-extern "C" __attribute__((visibility("default"))) int mops_seg_trace_read(long long* host, int count) {
-    return static_cast<int>(hipMemcpyFromSymbol(host, HIP_SYMBOL(seg_trace), count * sizeof(long long)));
-}
-extern "C" __attribute__((visibility("default"))) int mops_seg_trace_clear() {
-    static long long zeros[8192 * 8];
-    return static_cast<int>(hipMemcpyToSymbol(HIP_SYMBOL(seg_trace), zeros, sizeof(zeros)));
-}
-#endif
-
 bool supports(const Shape& s, size_t element_size) {
     if (s.n_nodes < 1 || s.n_edges < 1 || s.N < 1 || s.N > MAX_TABLE || s.L < 1) {
         return false;
@@ -870,6 +1426,106 @@ void forward(
     launch_contract<T, Source::SORTED>(args, stream);
 }
 
+/// Whether the persistent gradient kernel serves this vjp: the senders' edges
+/// fit the slots on average (sparse graphs), which grad_W needs.
+bool vjp_supported(const Shape& s, size_t element_size, bool want_grad_W) {
+    if (!sasaw_segments::supports(s, element_size)) {
+        return false;
+    }
+    return !want_grad_W || static_cast<size_t>(s.n_edges) <= static_cast<size_t>(s.n_nodes) * 48;
+}
+
+size_t vjp_workspace_bytes(const Shape& s, bool want_grad_W) {
+    return want_grad_W ? sender_slots_bytes(s.n_nodes) : 0;
+}
+
+/// Positions of the sorted index per unit of the per-edge gradients: the most
+/// of 64, 32, 16 that leave about one unit or more for each of `wanted_units`
+/// (the resident wavefronts, twice as many for double, whose units take longer
+/// and so even out worse). Measured at 60 000 edges, all three gradients,
+/// with 16 / 32 / 64: float 71 / 70 / 66 us, double 111 / 105 / 113 us; grad_A
+/// alone: float 34 / 36 / 54 us.
+int32_t edge_chunk_for(int32_t n_edges, int32_t edge_roles, int64_t wanted_units) {
+    for (int32_t chunk : {64, 32}) {
+        const int64_t units = (static_cast<int64_t>(n_edges) + chunk - 1) / chunk * edge_roles;
+        if (units * 10 >= wanted_units * 9) {
+            return chunk;
+        }
+    }
+    return 16;
+}
+
+template <typename T>
+void vjp(
+    T* grad_A, T* grad_B, T* grad_W, const T* grad_output, const T* A, const T* B, const T* C, const T* W,
+    const Indices& indices, const Shape& s, void* workspace, hipStream_t stream
+) {
+    GradientArgs<T> args{};
+    args.A = A;
+    args.B = B;
+    args.W = W;
+    args.G = grad_output;
+    args.C = C;
+    args.grad_A = grad_A;
+    args.grad_B = grad_B;
+    args.grad_W = grad_W;
+    args.receivers = indices.output_1;
+    args.senders = indices.W_1;
+    args.n_edges = s.n_edges;
+    args.n_nodes = s.n_nodes;
+    args.nA = s.nA;
+    args.L = s.L;
+    args.n2 = s.n2;
+    args.n3 = s.n3;
+    args.column_tiles = (s.L + 15) / 16;
+    if (grad_W != nullptr) {
+        // the edges of every sender, listed by a launch of its own in front
+        const SenderSlots slots = list_edges_in_slots(indices.W_1, s.n_edges, s.n_nodes, workspace, stream);
+        args.slot_edges = slots.edges;
+        args.slot_counts = slots.counts;
+    }
+    args.edge_roles = (grad_A != nullptr ? 1 : 0) + (grad_B != nullptr ? args.column_tiles : 0);
+    const int64_t W_units = grad_W != nullptr ? static_cast<int64_t>(s.n_nodes) * args.column_tiles : 0;
+    args.n_W_units = narrow_i32(static_cast<size_t>(W_units), "units of work");
+    // (rows of B and W are read 16 bytes at a time where their alignment allows)
+    const bool vectors =
+        s.L % 4 == 0 && reinterpret_cast<uintptr_t>(B) % 16 == 0 && reinterpret_cast<uintptr_t>(W) % 16 == 0;
+    MainKernelTimer timer(stream);
+
+    with_block_rows(std::max(s.n2, s.n3), [&](auto block_rows, auto fits) {
+        constexpr int NB = decltype(block_rows)::value;
+        // grad_W sums over the rows of grad_output (n3 of them), the others over those of W (n2)
+        args.table_W = table_of(s, indices.A, indices.output_2, indices.W_2, s.n3, s.n2);
+        args.table_alpha = table_of(s, indices.A, indices.W_2, indices.output_2, s.n2, s.n3);
+        args.table_alpha.layout = Layout::ALPHA;
+        args.table_beta = args.table_alpha;
+        args.table_beta.layout = Layout::BETA;
+        args.table_beta.bucket = NB;
+        const size_t slots = static_cast<size_t>(args.table_W.slots()) + args.table_alpha.slots() + args.table_beta.slots();
+        const size_t lds = slots * (sizeof(T) + sizeof(int32_t)) + 32;
+        constexpr int GROUP_WAVES = gradient_group_threads<T, NB>() / WAVE;
+        const int64_t resident_waves = static_cast<int64_t>(GROUP_WAVES) * compute_units();
+        args.edge_chunk = edge_chunk_for(s.n_edges, args.edge_roles, resident_waves * sizeof(T) / 4);
+        const int64_t chunks = (static_cast<int64_t>(s.n_edges) + args.edge_chunk - 1) / args.edge_chunk;
+        args.n_edge_units = narrow_i32(static_cast<size_t>(chunks * args.edge_roles), "units of work");
+        const int64_t units = W_units + chunks * args.edge_roles;
+        args.n_units = narrow_i32(static_cast<size_t>(units), "units of work");
+        const unsigned grid =
+            static_cast<unsigned>(std::min<int64_t>(compute_units(), (units + GROUP_WAVES - 1) / GROUP_WAVES));
+        (void)fits;
+        if (vectors) {
+            auto kernel = gradients_kernel<T, NB, true>;
+            allow_lds(kernel, lds);
+            kernel<<<grid, gradient_group_threads<T, NB>(), lds, stream>>>(args);
+        } else {
+            auto kernel = gradients_kernel<T, NB, false>;
+            allow_lds(kernel, lds);
+            kernel<<<grid, gradient_group_threads<T, NB>(), lds, stream>>>(args);
+        }
+    });
+    MOPS_HIP_CHECK(hipGetLastError());
+}
+
 template <typename T>
 void grad_W_from_slots(
     T* grad_W, const T* grad_output, const T* A, const T* B, const T* C, const Indices& indices, const Shape& s,
@@ -891,6 +1547,14 @@ template void forward<float>(
 );
 template void forward<double>(
     double*, const double*, const double*, const double*, const double*, const Indices&, const Shape&, hipStream_t
+);
+template void vjp<float>(
+    float*, float*, float*, const float*, const float*, const float*, const float*, const float*, const Indices&,
+    const Shape&, void*, hipStream_t
+);
+template void vjp<double>(
+    double*, double*, double*, const double*, const double*, const double*, const double*, const double*,
+    const Indices&, const Shape&, void*, hipStream_t
 );
 template void grad_W_from_slots<float>(
     float*, const float*, const float*, const float*, const float*, const Indices&, const Shape&, const SenderSlots&,

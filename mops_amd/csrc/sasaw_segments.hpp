@@ -26,6 +26,19 @@ void forward(
     const Shape& shape, hipStream_t stream
 );
 
+/// Whether vjp() serves the shape (grad_W needs a sparse graph: at most 48
+/// edges per node on average), and the device scratch it needs. vjp() makes no
+/// allocation and uses no second stream.
+bool vjp_supported(const Shape& shape, size_t element_size, bool want_grad_W);
+size_t vjp_workspace_bytes(const Shape& shape, bool want_grad_W);
+
+/// Any of grad_A, grad_B, grad_W may be null (not all).
+template <typename T>
+void vjp(
+    T* grad_A, T* grad_B, T* grad_W, const T* grad_output, const T* A, const T* B, const T* C,
+    const T* W, const Indices& indices, const Shape& shape, void* workspace, hipStream_t stream
+);
+
 /// grad_W from the lists of every sender's edges (sender_buckets.hpp).
 template <typename T>
 void grad_W_from_slots(

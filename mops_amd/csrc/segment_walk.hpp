@@ -39,51 +39,58 @@ struct ChunkIndex {
     int32_t ahead;  // value at the lane's position of the 64 positions after the chunk
 };
 
-template <int CHUNK>
-__device__ __forceinline__ ChunkIndex load_chunk_index(
-    const int32_t* __restrict__ sorted_index, int32_t n_input, int32_t wave_index
+/// `chunk`: positions per wavefront, 1..64 (uniform).
+__device__ __forceinline__ ChunkIndex load_chunk_index_of(
+    const int32_t* __restrict__ sorted_index, int32_t n_input, int32_t wave_index, const int32_t chunk
 ) {
-    static_assert(CHUNK >= 1 && CHUNK <= WAVE, "one index value per lane");
     const int lane = threadIdx.x & (WAVE - 1);
-    const int32_t chunk_begin = wave_index * CHUNK;
+    const int32_t chunk_begin = wave_index * chunk;
     const int32_t position = chunk_begin + lane;
-    const bool inside = lane < CHUNK && position < n_input;
+    const bool inside = lane < chunk && position < n_input;
     ChunkIndex index;
     index.mine = load_or_zero(sorted_index, static_cast<size_t>(position), inside);
     index.before = (inside && position > 0) ? sorted_index[position - 1] : -1;
     // the 64 positions after the chunk, asked for now: the last segment of the
     // chunk almost always ends there, and its end is then known without
     // another round trip to memory
-    const int32_t ahead_position = chunk_begin + CHUNK + lane;
+    const int32_t ahead_position = chunk_begin + chunk + lane;
     index.ahead = load_or_zero(sorted_index, static_cast<size_t>(ahead_position), ahead_position < n_input);
     return index;
 }
 
+template <int CHUNK>
+__device__ __forceinline__ ChunkIndex load_chunk_index(
+    const int32_t* __restrict__ sorted_index, int32_t n_input, int32_t wave_index
+) {
+    static_assert(CHUNK >= 1 && CHUNK <= WAVE, "one index value per lane");
+    return load_chunk_index_of(sorted_index, n_input, wave_index, CHUNK);
+}
+
 /// Called by all lanes of a wavefront. `wave_index` is the global number of
-/// the wavefront (uniform). CHUNK <= 64. `index`: load_chunk_index of the
-/// same arguments.
+/// the wavefront (uniform). CHUNK <= 64 (a template argument of the wrappers
+/// below, or a uniform run-time value of walk_pieces_of). `index`:
+/// load_chunk_index of the same arguments.
 ///   on_segment(row, first, last)  all lanes, uniform arguments, 0 <= row < n_rows
 ///   on_empty_rows(begin, end)     all lanes, rows in [begin, end) receive nothing
 ///   on_piece(row, first, last, from_start, to_end)   (walk_split_segments)
-template <int CHUNK, int SPLIT, typename PieceFn, typename EmptyRowsFn>
-__device__ __forceinline__ void walk_pieces(
+template <int SPLIT, typename PieceFn, typename EmptyRowsFn>
+__device__ __forceinline__ void walk_pieces_of(
     const int32_t* __restrict__ sorted_index,
     int32_t n_input,
     int32_t n_rows,
     int32_t wave_index,
+    const int32_t chunk,
     const ChunkIndex& index,
     PieceFn&& on_piece,
     EmptyRowsFn&& on_empty_rows
 ) {
-    static_assert(CHUNK >= 1 && CHUNK <= WAVE, "one index value per lane");
-    static_assert(SPLIT == 0 || SPLIT % CHUNK == 0, "cuts fall on chunk boundaries");
     const int lane = threadIdx.x & (WAVE - 1);
-    const int32_t chunk_begin = wave_index * CHUNK;
+    const int32_t chunk_begin = wave_index * chunk;
     if (chunk_begin >= n_input) {
         return;
     }
     const int32_t position = chunk_begin + lane;
-    const bool inside = lane < CHUNK && position < n_input;
+    const bool inside = lane < chunk && position < n_input;
     const int32_t mine = index.mine;
     const int32_t before = index.before;
     const int32_t ahead = index.ahead;
@@ -114,9 +121,9 @@ __device__ __forceinline__ void walk_pieces(
             }
             last = limit;
             bool found_end = false;
-            for (int32_t probe = chunk_begin + CHUNK; probe < limit; probe += WAVE) {
+            for (int32_t probe = chunk_begin + chunk; probe < limit; probe += WAVE) {
                 const int32_t at = probe + lane;
-                const bool first_look = probe == chunk_begin + CHUNK; // uniform
+                const bool first_look = probe == chunk_begin + chunk; // uniform
                 const int32_t value = first_look ? ahead : load_or_zero(sorted_index, static_cast<size_t>(at), at < n_input);
                 const bool differs = at >= n_input || value != row;
                 const unsigned long long mask = __ballot(differs);
@@ -147,12 +154,27 @@ __device__ __forceinline__ void walk_pieces(
     }
 
     // rows after the last value
-    if (n_input - 1 >= chunk_begin && n_input - 1 < chunk_begin + CHUNK) {
+    if (n_input - 1 >= chunk_begin && n_input - 1 < chunk_begin + chunk) {
         const int32_t tail_begin = max(sorted_index[n_input - 1] + 1, 0);
         if (tail_begin < n_rows) {
             on_empty_rows(tail_begin, n_rows);
         }
     }
+}
+
+template <int CHUNK, int SPLIT, typename PieceFn, typename EmptyRowsFn>
+__device__ __forceinline__ void walk_pieces(
+    const int32_t* __restrict__ sorted_index,
+    int32_t n_input,
+    int32_t n_rows,
+    int32_t wave_index,
+    const ChunkIndex& index,
+    PieceFn&& on_piece,
+    EmptyRowsFn&& on_empty_rows
+) {
+    static_assert(CHUNK >= 1 && CHUNK <= WAVE, "one index value per lane");
+    static_assert(SPLIT == 0 || SPLIT % CHUNK == 0, "cuts fall on chunk boundaries");
+    walk_pieces_of<SPLIT>(sorted_index, n_input, n_rows, wave_index, CHUNK, index, on_piece, on_empty_rows);
 }
 
 template <int CHUNK, typename SegmentFn, typename EmptyRowsFn>
