@@ -22,6 +22,7 @@
 // are reproducible from run to run. The reference's CUDA vjp accumulates
 // with shared-memory float atomics (mops/src/hpe/hpe.cu:288) and is not.
 #include <algorithm>
+#include <type_traits>
 
 #include "mops/hpe.hpp"
 
@@ -36,7 +37,7 @@ namespace mops::amd {
 namespace {
 
 constexpr size_t LDS_BUDGET = 60 * 1024;
-constexpr int32_t MANY_ROWS = 4096;                     // from here on the vjp goes by feature (at 1000 rows: 31.6 us against 27.5)
+constexpr int32_t MANY_ROWS = 4096;                     // from here on the vjp goes by feature (at 1000 rows it is the slower way)
 constexpr int32_t FORWARD_MANY_ROWS = 200 * 64;            // from here on the forward pass has a lane per row
 constexpr size_t BY_FEATURE_LDS_BUDGET = 140 * 1024;    // its two tiles, of the 160 KB of a compute unit
 
@@ -272,7 +273,7 @@ __global__ __launch_bounds__(WAVE) void vjp_kernel(
 // (prefix * suffix, 3 K multiplications instead of K^2) live in registers, and
 // the factors of the next monomial are fetched while the current one is used.
 // ---------------------------------------------------------------------------
-template <typename T, int ORDER>
+template <typename T, int ORDER, bool ALL_FEATURES>
 __global__ __launch_bounds__(WAVE) void vjp_ordered_kernel(
     T* __restrict__ grad_A,
     const T* __restrict__ grad_output,
@@ -282,111 +283,198 @@ __global__ __launch_bounds__(WAVE) void vjp_ordered_kernel(
     int32_t n_rows,
     int32_t nA,
     int32_t n_monomials,
-    int32_t R,
+    int32_t log2_R,
     int32_t span
 ) {
+    // LDS: a[nA + 1][R] accumulator[G][feature_count + 1][R]. The extra row of
+    // `a` stays zero and the extra accumulator row is never read: a factor
+    // outside [0, nA) reads the one, a term that is not to be kept (a feature
+    // of another range, a monomial beyond the last) goes to the other, and
+    // the loop over the monomials has no branch in it.
+    // ALL_FEATURES: span == nA, the workgroup keeps the terms of all features.
     extern __shared__ __align__(16) unsigned char lds_bytes[];
+    const int32_t R = 1 << log2_R;
     T* a_stage = reinterpret_cast<T*>(lds_bytes);
-    T* accumulator = a_stage + static_cast<size_t>(nA) * R;
-    const int32_t feature_begin = blockIdx.y * span;
-    const int32_t feature_count = min(span, nA - feature_begin);
+    T* accumulator = a_stage + static_cast<size_t>(nA + 1) * R;
+    const int32_t feature_begin = ALL_FEATURES ? 0 : blockIdx.y * span;
+    const int32_t feature_count = ALL_FEATURES ? nA : min(span, nA - feature_begin);
 
     const int tid = threadIdx.x;
-    const int G = WAVE / R;
-    const int r = tid % R;
-    const int g = tid / R;
+    const int G = WAVE >> log2_R;
+    const int r = tid & (R - 1);
+    const int g = tid >> log2_R;
     const int32_t row0 = blockIdx.x * R;
     const int32_t rows = min(R, n_rows - row0);
 
-    const T* a_src = A + static_cast<size_t>(row0) * nA;
-    for (int32_t i = tid; i < rows * nA; i += WAVE) {
-        int32_t row = i / nA;
-        a_stage[(i - row * nA) * R + row] = a_src[i];
+    struct Monomial {
+        int32_t factor[ORDER];
+        T coefficient;
+    };
+    auto fetch = [&](Monomial& to, int32_t j) {
+        const int32_t safe = min(j, n_monomials - 1);
+        const int32_t* factors = P + static_cast<size_t>(safe) * ORDER;
+#pragma unroll
+        for (int k = 0; k < ORDER; k++) {
+            to.factor[k] = factors[k];
+        }
+        to.coefficient = C[safe];
+    };
+    // A compute unit holds three of these wavefronts (their accumulators fill
+    // its LDS), so nobody else covers a thread's waits and every instruction
+    // counts. A thread works on BATCH monomials at a time, in three phases:
+    // all their values of A are asked for from LDS together, then all their
+    // terms are multiplied up in registers (BATCH independent chains), then
+    // all terms are added to the accumulators, in the order of the
+    // monomials. The factors of the next batch are on their way from global
+    // memory meanwhile, those of the first one while the tiles are set up.
+    constexpr int BATCH = 8;
+    Monomial queue[BATCH];
+#pragma unroll
+    for (int d = 0; d < BATCH; d++) {
+        fetch(queue[d], g + d * G);
     }
-    for (int32_t i = tid; i < G * feature_count * R; i += WAVE) {
-        accumulator[i] = T(0);
+    const T upstream = grad_output[min(row0 + r, n_rows - 1)];
+
+    // the rows of A, STAGE values per lane asked for together: with one load
+    // per turn of a loop, each turn would wait a whole round trip to memory
+    const T* a_src = A + static_cast<size_t>(row0) * nA;
+    constexpr int STAGE = 8;
+    for (int32_t base = 0; base < rows * nA; base += STAGE * WAVE) {
+        T staged[STAGE];
+#pragma unroll
+        for (int u = 0; u < STAGE; u++) {
+            const int32_t i = base + u * WAVE + tid;
+            staged[u] = a_src[min(i, rows * nA - 1)];
+        }
+#pragma unroll
+        for (int u = 0; u < STAGE; u++) {
+            const int32_t i = base + u * WAVE + tid;
+            if (i < rows * nA) {
+                const int32_t row = i / nA;
+                a_stage[((i - row * nA) << log2_R) + row] = staged[u];
+            }
+        }
+    }
+    if (tid < R) {
+        a_stage[nA * R + tid] = T(0);
+    }
+    // (G * R = 64 threads: every lane clears feature_count + 1 values, a
+    // wavefront's worth apart; unrolled, because a single wavefront pays for
+    // every instruction of the loop around a store)
+    {
+        T* clear = accumulator + tid;
+        int32_t k = 0;
+        for (; k + 8 <= feature_count + 1; k += 8) {
+#pragma unroll
+            for (int u = 0; u < 8; u++) {
+                clear[(k + u) * WAVE] = T(0);
+            }
+        }
+        for (; k < feature_count + 1; k++) {
+            clear[k * WAVE] = T(0);
+        }
     }
     __syncthreads();
 
     if (r < rows) {
-        T* mine = accumulator + static_cast<size_t>(g) * feature_count * R + r;
-        const T upstream = grad_output[row0 + r];
-        struct Monomial {
-            int32_t factor[ORDER];
-            T coefficient;
-        };
-        auto fetch = [&](Monomial& to, int32_t j) {
-            const int32_t safe = min(j, n_monomials - 1);
-            const int32_t* factors = P + static_cast<size_t>(safe) * ORDER;
+        T* mine = accumulator + static_cast<size_t>(g) * (feature_count + 1) * R + r;
+        const T* my_a = a_stage + r;
+        const uint32_t features = static_cast<uint32_t>(nA);
+        const uint32_t kept = static_cast<uint32_t>(feature_count);
+        // `whole`: all monomials of the batch exist
+        auto batch = [&](int32_t j0, auto whole) {
+            constexpr bool WHOLE = decltype(whole)::value;
+            Monomial now[BATCH];
+            T value[BATCH][ORDER];
 #pragma unroll
-            for (int k = 0; k < ORDER; k++) {
-                to.factor[k] = factors[k];
+            for (int d = 0; d < BATCH; d++) {
+                now[d] = queue[d];
+#pragma unroll
+                for (int k = 0; k < ORDER; k++) {
+                    // (as unsigned, a negative factor is a large one)
+                    const uint32_t feature = min(static_cast<uint32_t>(now[d].factor[k]), features);
+                    value[d][k] = my_a[feature << log2_R];
+                }
             }
-            to.coefficient = C[safe];
-        };
-        // A compute unit holds three of these wavefronts (their accumulators fill
-        // its LDS), so nobody else covers the wait for a monomial: a thread has
-        // the factors of its next AHEAD monomials on the way while it uses one.
-        constexpr int AHEAD = 8;
-        Monomial queue[AHEAD];
+            if constexpr (WHOLE) {
 #pragma unroll
-        for (int d = 0; d < AHEAD; d++) {
-            fetch(queue[d], g + d * G);
-        }
-        for (int32_t j0 = g; j0 < n_monomials; j0 += AHEAD * G) {
-#pragma unroll
-        for (int d = 0; d < AHEAD; d++) {
-            const int32_t j = j0 + d * G;
-            if (j >= n_monomials) {
-                break;
-            }
-            const Monomial now = queue[d];
-            fetch(queue[d], j + AHEAD * G);
-            T value[ORDER];
-            bool valid[ORDER];
-#pragma unroll
-            for (int k = 0; k < ORDER; k++) {
-                valid[k] = in_bounds(now.factor[k], nA);
-                value[k] = valid[k] ? a_stage[now.factor[k] * R + r] : T(0);
+                for (int d = 0; d < BATCH; d++) {
+                    fetch(queue[d], j0 + (d + BATCH) * G);
+                }
             }
             // term[f] = base * prod_{k != f} value[k], multiplied left to right
-            T prefix[ORDER];
-            prefix[0] = now.coefficient * upstream;
+            T term[BATCH][ORDER];
 #pragma unroll
-            for (int k = 1; k < ORDER; k++) {
-                prefix[k] = prefix[k - 1] * value[k - 1];
+            for (int d = 0; d < BATCH; d++) {
+                T prefix[ORDER];
+                prefix[0] = now[d].coefficient * upstream;
+#pragma unroll
+                for (int k = 1; k < ORDER; k++) {
+                    prefix[k] = prefix[k - 1] * value[d][k - 1];
+                }
+                T suffix = T(1);
+#pragma unroll
+                for (int f = ORDER - 1; f >= 0; f--) {
+                    term[d][f] = prefix[f] * suffix;
+                    suffix *= value[d][f];
+                }
             }
-            T suffix = T(1);
 #pragma unroll
-            for (int f = ORDER - 1; f >= 0; f--) {
-                const T term = prefix[f] * suffix;
-                suffix *= value[f];
-                const int32_t slot = now.factor[f] - feature_begin;
-                if (in_bounds(slot, feature_count)) {
+            for (int d = 0; d < BATCH; d++) {
+                const bool exists = WHOLE || j0 + d * G < n_monomials;
+#pragma unroll
+                for (int f = ORDER - 1; f >= 0; f--) {
+                    uint32_t slot = static_cast<uint32_t>(now[d].factor[f]);
+                    if constexpr (!ALL_FEATURES) {
+                        slot -= static_cast<uint32_t>(feature_begin);
+                    }
+                    slot = min(slot, kept);
+                    T* to = mine + ((exists ? slot : kept) << log2_R);
                     // a slot of my own. In f64 the LDS add instruction, which saves the
-                    // round trip of read, add, write (c0: 31 -> 27 us); in f32 that
-                    // instruction is the slower way here (53 us against 21)
+                    // round trip of read, add, write; in f32 that instruction is the
+                    // slower way here (53 us against 21)
                     if constexpr (sizeof(T) == 8) {
-                        unsafeAtomicAdd(&mine[slot * R], term);
+                        unsafeAtomicAdd(to, term[d][f]);
                     } else {
-                        mine[slot * R] += term;
+                        *to += term[d][f];
                     }
                 }
             }
+        };
+        int32_t j0 = g;
+        for (; j0 + (BATCH - 1) * G < n_monomials; j0 += BATCH * G) {
+            batch(j0, std::true_type{});
         }
+        if (j0 < n_monomials) {
+            batch(j0, std::false_type{});
         }
     }
     __syncthreads();
 
+    // The G copies added up, every (feature, row) by one lane: four running
+    // sums over the copies g = 0, 4, ... / 1, 5, ... / 2, 6, ... / 3, 7, ...
+    // and then (s0 + s1) + (s2 + s3): one fixed order, and chains of additions
+    // a quarter as long as one sum over all copies would be.
     T* dst = grad_A + static_cast<size_t>(row0) * nA + feature_begin;
-    for (int32_t i = tid; i < rows * feature_count; i += WAVE) {
-        int32_t row = i / feature_count;
-        int32_t feature = i - row * feature_count;
-        T total = T(0);
-        for (int group = 0; group < G; group++) {
-            total += accumulator[(static_cast<size_t>(group) * feature_count + feature) * R + row];
+    const int32_t copy_stride = (feature_count + 1) * R;
+    for (int32_t entry = tid; entry < feature_count * R; entry += WAVE) {
+        const int32_t row = entry & (R - 1);
+        const int32_t feature = entry >> log2_R;
+        const T* from = accumulator + entry;
+        T partial[4] = {T(0), T(0), T(0), T(0)};
+        int group = 0;
+        for (; group + 4 <= G; group += 4) {
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                partial[u] += from[(group + u) * copy_stride];
+            }
         }
-        dst[static_cast<size_t>(row) * nA + feature] = total;
+        for (; group < G; group++) {
+            partial[group & 3] += from[group * copy_stride];
+        }
+        if (row < rows) {
+            dst[static_cast<size_t>(row) * nA + feature] = (partial[0] + partial[1]) + (partial[2] + partial[3]);
+        }
     }
 }
 
@@ -1170,14 +1258,14 @@ void homogeneous_polynomial_evaluation_vjp(MOPS_HPE_VJP_PARAMS(MOPS_CXX_FIRST, M
         return;
     }
     // LDS holds R rows of A and WAVE private accumulator rows, whatever R is
-    const size_t accumulator_bytes = static_cast<size_t>(nA) * WAVE * sizeof(scalar_t);
+    const size_t accumulator_bytes = (static_cast<size_t>(nA) + 1) * WAVE * sizeof(scalar_t);
     // Rows per workgroup: the fewest for which all workgroups are on the
     // device at once (256 CUs, as many workgroups per CU as the 160 KB of LDS
     // hold): a second round of workgroups costs more than rows twice as long
     // (c0: 37 us with 1000 workgroups of one row, 31 us with 500 of two).
     int R = 0;
     for (int rows = 1; rows <= 64 && R == 0; rows <<= 1) {
-        const size_t lds = accumulator_bytes + static_cast<size_t>(nA) * rows * sizeof(scalar_t);
+        const size_t lds = accumulator_bytes + (static_cast<size_t>(nA) + 1) * rows * sizeof(scalar_t);
         if (lds > LDS_BUDGET) {
             break;
         }
@@ -1186,35 +1274,47 @@ void homogeneous_polynomial_evaluation_vjp(MOPS_HPE_VJP_PARAMS(MOPS_CXX_FIRST, M
             R = rows;
         }
     }
-    if (R == 0 && accumulator_bytes + static_cast<size_t>(nA) * sizeof(scalar_t) <= LDS_BUDGET) {
+    if (R == 0 && accumulator_bytes + (static_cast<size_t>(nA) + 1) * sizeof(scalar_t) <= LDS_BUDGET) {
         // the tiles of 64 rows do not fit: as many rows as do
         R = 1;
-        while (accumulator_bytes + static_cast<size_t>(nA) * (2 * R) * sizeof(scalar_t) <= LDS_BUDGET && R < 64) {
+        while (accumulator_bytes + (static_cast<size_t>(nA) + 1) * (2 * R) * sizeof(scalar_t) <= LDS_BUDGET && R < 64) {
             R <<= 1;
         }
     }
     int32_t span = nA; // features whose accumulators one workgroup keeps
-    if (R == 0 && static_cast<size_t>(nA) * sizeof(scalar_t) <= LDS_BUDGET / 2) {
+    if (R == 0 && (static_cast<size_t>(nA) + 1) * sizeof(scalar_t) <= LDS_BUDGET / 2) {
         // the accumulators of all features do not fit: one row per workgroup,
         // the features in ranges that do
         R = 1;
         span = static_cast<int32_t>(
-            (LDS_BUDGET - static_cast<size_t>(nA) * sizeof(scalar_t)) / (WAVE * sizeof(scalar_t))
+            (LDS_BUDGET - (static_cast<size_t>(nA) + 1) * sizeof(scalar_t)) / (WAVE * sizeof(scalar_t)) - 1
         );
     }
     if (R > 0) {
-        size_t lds =
-            static_cast<size_t>(span) * WAVE * sizeof(scalar_t) + static_cast<size_t>(nA) * R * sizeof(scalar_t);
+        // (one row more of each than there are features: see vjp_ordered_kernel)
+        size_t lds = (static_cast<size_t>(span) + 1) * WAVE * sizeof(scalar_t) +
+                     (static_cast<size_t>(nA) + 1) * R * sizeof(scalar_t);
+        int32_t log2_R = 0;
+        while ((1 << log2_R) < R) {
+            log2_R++;
+        }
         const dim3 blocks(
             static_cast<unsigned>(ceil_div(static_cast<size_t>(n_rows), R)),
             static_cast<unsigned>(ceil_div(static_cast<size_t>(nA), span))
         );
         MainKernelTimer timer(stream);
 #define MOPS_LAUNCH_ORDERED(ORDER)                                                                  \
-    vjp_ordered_kernel<scalar_t, ORDER><<<blocks, WAVE, lds, stream>>>(                            \
-        grad_A.data, grad_output.data, A.data, C.data, indices_A.data, n_rows, nA, n_monomials, R, \
-        span                                                                                       \
-    )
+    if (span == nA) {                                                                              \
+        vjp_ordered_kernel<scalar_t, ORDER, true><<<blocks, WAVE, lds, stream>>>(                  \
+            grad_A.data, grad_output.data, A.data, C.data, indices_A.data, n_rows, nA,             \
+            n_monomials, log2_R, span                                                              \
+        );                                                                                         \
+    } else {                                                                                       \
+        vjp_ordered_kernel<scalar_t, ORDER, false><<<blocks, WAVE, lds, stream>>>(                 \
+            grad_A.data, grad_output.data, A.data, C.data, indices_A.data, n_rows, nA,             \
+            n_monomials, log2_R, span                                                              \
+        );                                                                                         \
+    }
         switch (n_monomials > 0 ? order : 0) {
         case 1:
             MOPS_LAUNCH_ORDERED(1);
