@@ -59,8 +59,8 @@ MAIN_KERNELS = {
     ("opsa", "vjp"): "edge_rows_vjp_kernel<{T}, 1, 2, false, true, false, false>",
     ("opsaw", "forward"): "forward_kernel<{T}, 2, true>",
     ("opsaw", "vjp"): "edge_rows_vjp_kernel<{T}, 1, 2, true, true, false, true>",
-    ("sasaw", "forward"): "sasaw_segments::contract_kernel<{T}, 9, true, (sasaw_segments::(anonymous namespace)::Source)0",
-    ("sasaw", "vjp"): "sasaw_segments::(anonymous namespace)::gradients_kernel<{T}, 9, true>",
+    ("sasaw", "forward"): "sasaw_segments::contract_kernel<{T}, 9, true, ",
+    ("sasaw", "vjp"): "sasaw_segments::gradients_kernel<{T}, 9, true>",
 }
 
 

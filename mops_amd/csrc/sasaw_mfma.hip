@@ -1412,8 +1412,7 @@ void forward(
 template <typename T>
 void vjp(
     T* grad_A, T* grad_B, T* grad_W, const T* grad_output, const T* A, const T* B, const T* C,
-    const T* W, const Indices& indices, const Shape& s, void* workspace, hipStream_t stream,
-    const WeightsFromSlots* weights_from_slots
+    const T* W, const Indices& indices, const Shape& s, void* workspace, hipStream_t stream
 ) {
     const DenseLayout layout = dense_layout(s);
     const bool want_edges = grad_A != nullptr || grad_B != nullptr;
@@ -1523,13 +1522,7 @@ void vjp(
         MOPS_HIP_CHECK(hipGetLastError());
     };
 
-    if (slotted && weights_from_slots != nullptr) {
-        // grad_W by the caller's kernel, after the per-edge gradients
-        if (want_edges) {
-            for_each_column_block(s, [&](int32_t first, const Shape& block) { launch_edges(first, block, false); });
-        }
-        (*weights_from_slots)(slots);
-    } else if (want_edges && slotted && (s.n2 + 3) / 4 == (s.n3 + 3) / 4) {
+    if (want_edges && slotted && (s.n2 + 3) / 4 == (s.n3 + 3) / 4) {
         // sparse graphs: one launch for all three gradients
         for_each_column_block(s, [&](int32_t first, const Shape& block) { launch_edges(first, block, true); });
     } else if (want_edges && grad_W != nullptr) {
@@ -1577,11 +1570,11 @@ template void forward<double>(
 );
 template void vjp<float>(
     float*, float*, float*, const float*, const float*, const float*, const float*, const float*,
-    const Indices&, const Shape&, void*, hipStream_t, const WeightsFromSlots*
+    const Indices&, const Shape&, void*, hipStream_t
 );
 template void vjp<double>(
     double*, double*, double*, const double*, const double*, const double*, const double*, const double*,
-    const Indices&, const Shape&, void*, hipStream_t, const WeightsFromSlots*
+    const Indices&, const Shape&, void*, hipStream_t
 );
 
 } // namespace mops::amd::sasaw_mfma

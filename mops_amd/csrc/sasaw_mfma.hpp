@@ -8,11 +8,7 @@
 #include <cstddef>
 #include <cstdint>
 
-#include <functional>
-
 #include <hip/hip_runtime.h>
-
-#include "sender_buckets.hpp"
 
 namespace mops::amd::sasaw_mfma {
 
@@ -51,16 +47,11 @@ void forward(
 /// stream, no events, no allocation.
 bool vjp_allocates_nothing(const Shape& shape, size_t element_size, bool want_edge_gradients, bool want_grad_W);
 
-/// Any of grad_A, grad_B, grad_W may be null. `weights_from_slots`, when given
-/// and the senders' edges are listed in slots (sparse graphs), is called with
-/// the slots once the kernel that lists them is enqueued, and computes grad_W
-/// in their place.
-using WeightsFromSlots = std::function<void(const SenderSlots&)>;
+/// Any of grad_A, grad_B, grad_W may be null.
 template <typename T>
 void vjp(
     T* grad_A, T* grad_B, T* grad_W, const T* grad_output, const T* A, const T* B, const T* C,
-    const T* W, const Indices& indices, const Shape& shape, void* workspace, hipStream_t stream,
-    const WeightsFromSlots* weights_from_slots = nullptr
+    const T* W, const Indices& indices, const Shape& shape, void* workspace, hipStream_t stream
 );
 
 } // namespace mops::amd::sasaw_mfma

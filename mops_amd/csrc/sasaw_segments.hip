@@ -595,23 +595,12 @@ __device__ __forceinline__ bool sum_over_slots(
     return any;
 }
 
-/// Where the edges of a node come from.
-enum class Source {
-    SORTED, // the index that names the node is sorted: segments of consecutive edges
-    SLOTS   // the node's edges are listed in its slots (sender_buckets.hpp)
-};
-
 template <typename T> struct ContractArgs {
     Contraction<T> contraction;
     Table table;
     const T* C;
-    int32_t n_units; // (chunks of positions | nodes) x column tiles
-    // SORTED
+    int32_t n_units;             // chunks of positions x column tiles
     const int32_t* sorted_index; // [n_edges] node of every position, non-decreasing
-    // SLOTS
-    const int32_t* slot_edges;
-    const int32_t* slot_counts;
-    const int32_t* listed_index; // [n_edges] the index the slots were listed from (for nodes whose slots overflowed)
 };
 
 /// Wavefronts per SIMD the registers are limited to, by element type and
@@ -624,14 +613,9 @@ template <typename T, int NB> constexpr int group_threads() { return 4 * waves_p
 
 /// What a wavefront asks for ahead of a unit of work: nothing of it depends
 /// on anything but the unit's number.
-template <Source SOURCE> struct UnitAhead;
-template <> struct UnitAhead<Source::SORTED> {
+struct UnitAhead {
     ChunkIndex index;
     int32_t near_source[2]; // blocks of the 128 positions from the chunk's first
-};
-template <> struct UnitAhead<Source::SLOTS> {
-    int32_t first_half, second_half; // the node's slots
-    int4 part_counts;
 };
 
 // The kernel is PERSISTENT: one workgroup per compute unit builds the dense
@@ -643,7 +627,7 @@ template <> struct UnitAhead<Source::SLOTS> {
 // global memory has to be cleared, and every wavefront leaves when the
 // counter has passed the workgroup's last unit. While a wavefront works on a
 // unit, the index values of its next unit are on their way.
-template <typename T, int NB, bool EXACT, Source SOURCE, int CHUNK>
+template <typename T, int NB, bool EXACT, int CHUNK>
 __global__ __launch_bounds__((group_threads<T, NB>())) void contract_kernel(const ContractArgs<T> args) {
     constexpr int THREADS = group_threads<T, NB>();
     constexpr int GROUP_WAVES = THREADS / WAVE;
@@ -669,30 +653,22 @@ __global__ __launch_bounds__((group_threads<T, NB>())) void contract_kernel(cons
         }
         return __builtin_amdgcn_readfirstlane(turn);
     };
-    auto look_ahead = [&](UnitAhead<SOURCE>& ahead, int32_t unit) {
+    auto look_ahead = [&](UnitAhead& ahead, int32_t unit) {
         const bool exists = unit < args.n_units;
-        const int32_t item = exists ? unit / p.column_tiles : 0; // chunk or node
-        if constexpr (SOURCE == Source::SORTED) {
-            ahead.index = load_chunk_index<CHUNK>(args.sorted_index, p.n_edges, item);
+        const int32_t item = exists ? unit / p.column_tiles : 0; // chunk
+        ahead.index = load_chunk_index<CHUNK>(args.sorted_index, p.n_edges, item);
 #pragma unroll
-            for (int h = 0; h < 2; h++) {
-                const int32_t position = item * CHUNK + h * WAVE + lane;
-                const int32_t source =
-                    load_or_zero(p.gather_index, static_cast<size_t>(position), position < p.n_edges);
-                ahead.near_source[h] = position < p.n_edges ? source : -1;
-            }
-        } else {
-            const int32_t* mine = args.slot_edges + static_cast<size_t>(item) * SLOT_CAPACITY;
-            ahead.first_half = mine[lane];
-            ahead.second_half = mine[lane + WAVE];
-            ahead.part_counts = reinterpret_cast<const int4*>(args.slot_counts)[item];
+        for (int h = 0; h < 2; h++) {
+            const int32_t position = item * CHUNK + h * WAVE + lane;
+            const int32_t source = load_or_zero(p.gather_index, static_cast<size_t>(position), position < p.n_edges);
+            ahead.near_source[h] = position < p.n_edges ? source : -1;
         }
     };
 
     // everything that can be asked for without knowing anything is asked for
     // first; the table is built while it is on its way
     int32_t unit = unit_of_turn(wave);
-    UnitAhead<SOURCE> current;
+    UnitAhead current;
     MyEntries<T> entries;
     if (wave == 0) {
         load_entries<T>(entries, args.C, args.table, 0, lane);
@@ -727,46 +703,35 @@ __global__ __launch_bounds__((group_threads<T, NB>())) void contract_kernel(cons
 
     while (unit < args.n_units) {
         const int32_t next_unit = unit_of_turn(take_turn());
-        UnitAhead<SOURCE> next;
+        UnitAhead next;
         look_ahead(next, next_unit);
         const int32_t item = unit / p.column_tiles;
         sum.set_column_tile(unit - item * p.column_tiles);
-        if constexpr (SOURCE == Source::SLOTS) {
-            if (sum_over_slots(
-                    sum, current.first_half, current.second_half, current.part_counts, args.listed_index, item, lane
-                )) {
-                wait_for_table();
-                sum.finish(table, registers, item);
-            } else {
-                sum.clear_rows(item, item + 1);
-            }
-        } else {
-            const int32_t chunk_begin = item * CHUNK;
-            walk_owned_segments<CHUNK>(
-                args.sorted_index, p.n_edges, p.n_blocks, item, current.index,
-                [&](int32_t node, int32_t first, int32_t last) {
-                    sum.clear();
-                    for (int32_t base = first; base < last; base += WAVE) {
-                        const int32_t n = min(WAVE, last - base);
-                        const int32_t offset = base - chunk_begin; // >= 0: owned segments start in the chunk
-                        int32_t edges = lane < n ? base + lane : -1;
-                        int32_t sources;
-                        if (offset + WAVE <= 2 * WAVE) { // (uniform) all 64 positions are at hand
-                            const int from = offset + lane;
-                            const int32_t s0 = __shfl(current.near_source[0], from & (WAVE - 1));
-                            const int32_t s1 = __shfl(current.near_source[1], from & (WAVE - 1));
-                            sources = from < WAVE ? s0 : s1;
-                        } else {
-                            sources = load_or_zero(p.gather_index, static_cast<size_t>(max(edges, 0)), edges >= 0);
-                        }
-                        sum.add(edges, edges >= 0 ? sources : -1, n);
+        const int32_t chunk_begin = item * CHUNK;
+        walk_owned_segments<CHUNK>(
+            args.sorted_index, p.n_edges, p.n_blocks, item, current.index,
+            [&](int32_t node, int32_t first, int32_t last) {
+                sum.clear();
+                for (int32_t base = first; base < last; base += WAVE) {
+                    const int32_t n = min(WAVE, last - base);
+                    const int32_t offset = base - chunk_begin; // >= 0: owned segments start in the chunk
+                    int32_t edges = lane < n ? base + lane : -1;
+                    int32_t sources;
+                    if (offset + WAVE <= 2 * WAVE) { // (uniform) all 64 positions are at hand
+                        const int from = offset + lane;
+                        const int32_t s0 = __shfl(current.near_source[0], from & (WAVE - 1));
+                        const int32_t s1 = __shfl(current.near_source[1], from & (WAVE - 1));
+                        sources = from < WAVE ? s0 : s1;
+                    } else {
+                        sources = load_or_zero(p.gather_index, static_cast<size_t>(max(edges, 0)), edges >= 0);
                     }
-                    wait_for_table();
-                    sum.finish(table, registers, node);
-                },
-                [&](int32_t begin, int32_t end) { sum.clear_rows(begin, end); }
-            );
-        }
+                    sum.add(edges, edges >= 0 ? sources : -1, n);
+                }
+                wait_for_table();
+                sum.finish(table, registers, node);
+            },
+            [&](int32_t begin, int32_t end) { sum.clear_rows(begin, end); }
+        );
         unit = next_unit;
         current = next;
     }
@@ -1332,43 +1297,35 @@ int32_t compute_units() {
     return count;
 }
 
-template <typename T, Source SOURCE>
-void launch_contract(ContractArgs<T> args, hipStream_t stream) {
+template <typename T> void launch_contract(ContractArgs<T> args, hipStream_t stream) {
     const Contraction<T>& p = args.contraction;
     const size_t lds = table_lds(args.table, sizeof(T));
     with_block_rows(p.n_red, [&](auto block_rows, auto exact) {
         constexpr int NB = decltype(block_rows)::value;
         constexpr bool EXACT = decltype(exact)::value;
+        constexpr int64_t GROUP_WAVES = group_threads<T, NB>() / WAVE;
         auto go = [&](auto chunk_constant) {
             constexpr int CHUNK = decltype(chunk_constant)::value;
-            constexpr int GROUP_WAVES = group_threads<T, NB>() / WAVE;
-            const int64_t items = SOURCE == Source::SLOTS ? p.n_blocks
-                                                          : (static_cast<int64_t>(p.n_edges) + CHUNK - 1) / CHUNK;
-            const int64_t units = items * p.column_tiles;
+            const int64_t units = (static_cast<int64_t>(p.n_edges) + CHUNK - 1) / CHUNK * p.column_tiles;
             args.n_units = narrow_i32(static_cast<size_t>(units), "units of work");
             // one workgroup per compute unit, fewer when there is not a unit per wavefront
             const unsigned grid = static_cast<unsigned>(
                 std::min<int64_t>(compute_units(), (units + GROUP_WAVES - 1) / GROUP_WAVES)
             );
-            auto kernel = contract_kernel<T, NB, EXACT, SOURCE, CHUNK>;
+            auto kernel = contract_kernel<T, NB, EXACT, CHUNK>;
             allow_lds(kernel, lds);
             kernel<<<grid, group_threads<T, NB>(), lds, stream>>>(args);
         };
-        if constexpr (SOURCE == Source::SLOTS) {
+        switch (chunk_for(p.n_edges, p.column_tiles, GROUP_WAVES * compute_units())) {
+        case 16:
+            go(std::integral_constant<int, 16>{});
+            break;
+        case 32:
+            go(std::integral_constant<int, 32>{});
+            break;
+        default:
             go(std::integral_constant<int, 64>{});
-        } else {
-            constexpr int64_t GROUP_WAVES = group_threads<T, NB>() / WAVE;
-            switch (chunk_for(p.n_edges, p.column_tiles, GROUP_WAVES * compute_units())) {
-            case 16:
-                go(std::integral_constant<int, 16>{});
-                break;
-            case 32:
-                go(std::integral_constant<int, 32>{});
-                break;
-            default:
-                go(std::integral_constant<int, 64>{});
-                break;
-            }
+            break;
         }
     });
     MOPS_HIP_CHECK(hipGetLastError());
@@ -1423,7 +1380,7 @@ void forward(
     args.C = C;
     args.sorted_index = indices.output_1;
     MainKernelTimer timer(stream);
-    launch_contract<T, Source::SORTED>(args, stream);
+    launch_contract<T>(args, stream);
 }
 
 /// Whether the persistent gradient kernel serves this vjp: the senders' edges
@@ -1526,22 +1483,6 @@ void vjp(
     MOPS_HIP_CHECK(hipGetLastError());
 }
 
-template <typename T>
-void grad_W_from_slots(
-    T* grad_W, const T* grad_output, const T* A, const T* B, const T* C, const Indices& indices, const Shape& s,
-    const SenderSlots& slots, hipStream_t stream
-) {
-    ContractArgs<T> args{};
-    // the blocks that are gathered are rows of grad_output, named by the receiver
-    args.contraction = contraction_of<T>(s, A, B, grad_output, indices.output_1, grad_W, s.n3, s.n2);
-    args.table = table_of(s, indices.A, indices.output_2, indices.W_2, s.n3, s.n2);
-    args.C = C;
-    args.slot_edges = slots.edges;
-    args.slot_counts = slots.counts;
-    args.listed_index = indices.W_1;
-    launch_contract<T, Source::SLOTS>(args, stream);
-}
-
 template void forward<float>(
     float*, const float*, const float*, const float*, const float*, const Indices&, const Shape&, hipStream_t
 );
@@ -1555,14 +1496,6 @@ template void vjp<float>(
 template void vjp<double>(
     double*, double*, double*, const double*, const double*, const double*, const double*, const double*,
     const Indices&, const Shape&, void*, hipStream_t
-);
-template void grad_W_from_slots<float>(
-    float*, const float*, const float*, const float*, const float*, const Indices&, const Shape&, const SenderSlots&,
-    hipStream_t
-);
-template void grad_W_from_slots<double>(
-    double*, const double*, const double*, const double*, const double*, const Indices&, const Shape&,
-    const SenderSlots&, hipStream_t
 );
 
 } // namespace mops::amd::sasaw_segments

@@ -39,13 +39,6 @@ void vjp(
     const T* W, const Indices& indices, const Shape& shape, void* workspace, hipStream_t stream
 );
 
-/// grad_W from the lists of every sender's edges (sender_buckets.hpp).
-template <typename T>
-void grad_W_from_slots(
-    T* grad_W, const T* grad_output, const T* A, const T* B, const T* C, const Indices& indices,
-    const Shape& shape, const SenderSlots& slots, hipStream_t stream
-);
-
 } // namespace mops::amd::sasaw_segments
 
 #endif
