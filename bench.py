@@ -52,7 +52,7 @@ TRAFFIC_FILE = os.path.join(ROOT, "profiles", "all_ops_baseline_shapes_hbm_traff
 # per-kernel figures and to find the kernel in the counter summary.
 MAIN_KERNELS = {
     ("hpe", "forward"): "forward_ordered_kernel<{T}, 4>",
-    ("hpe", "vjp"): "vjp_ordered_kernel<{T}, 4>",
+    ("hpe", "vjp"): "vjp_ordered_kernel<{T}, 4, true>",
     ("sap", "forward"): "sap_mfma::forward_kernel<{T}, 2, 2>",
     ("sap", "vjp"): "sap_mfma::vjp_kernel<{T}, 5>",
     ("opsa", "forward"): "forward_kernel<{T}, 2, false>",
