@@ -286,6 +286,20 @@ __device__ __forceinline__ int opaque(int value) {
     return value;
 }
 
+/// The (uniform) value, made where it is used. The byte offsets of the rows
+/// of a block, c * row_bytes for every c, are the same in every turn of every
+/// loop, so the compiler computes them once in front of the loop over the units
+/// of work; a kernel with several roles has no scalar registers left for them,
+/// keeps them in lanes of a vector register, and every load then costs a
+/// `v_readlane` and the five idle cycles between it and the load that uses it.
+/// One scalar multiplication per load instead.
+__device__ __forceinline__ uint32_t fresh(uint32_t value) {
+    // (readfirstlane: where the compiler holds the uniform value in a vector register)
+    uint32_t uniform = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(value)));
+    asm volatile("" : "+s"(uniform));
+    return uniform;
+}
+
 /// All ones unless `wanted`: OR-ed into a byte offset it makes the load read
 /// zero. (Arithmetic instead of a choice between an offset and a constant: the
 /// compiler turns such a choice in front of a load into two branches.)
@@ -408,7 +422,8 @@ template <typename T, int NB, bool EXACT, bool COMPACT = false> struct NodeSum {
 #pragma unroll
             for (int c = 0; c < NB; c++) {
                 const uint32_t row = static_cast<uint32_t>(EXACT ? c : min(c, p.n_red - 1));
-                to.w[u][c] = rows.load(from, row * row_bytes);
+                // (COMPACT: the kernel with several roles, where the offsets would not stay in scalar registers)
+                to.w[u][c] = rows.load(from, (COMPACT ? fresh(row) : row) * row_bytes);
             }
         }
     }
@@ -496,15 +511,52 @@ template <typename T, int NB, bool EXACT, bool COMPACT = false> struct NodeSum {
 
     /// result[node] = D * (the sums so far), this wavefront's 16 columns.
     __device__ __forceinline__ void finish(const T* __restrict__ table, int32_t registers, int32_t node) {
-        typename M::Acc out[2] = {M::zero(), M::zero()};
+        // result = D * sums, one block of NB table operands per register r of the
+        // sums; four sums (double: two) take the products in turn, so that
+        // consecutive matrix instructions do not wait for each other.
+        typename M::Acc out[sizeof(T) == 4 ? 4 : 2];
 #pragma unroll
-        for (int r = 0; r < 4; r++) {
-            if (r < registers) { // (uniform)
+        for (auto& sum : out) {
+            sum = M::zero();
+        }
+        if constexpr (sizeof(T) == 4) {
+            // The operands of block r + 1 are read from LDS before the matrix
+            // instructions of block r (always: a read under a condition would
+            // have to be waited for where it stands).
+            T d[2][NB];
+            auto read = [&](T (&to)[NB], int r) {
+                const int32_t block = min(r, registers - 1);
 #pragma unroll
                 for (int c = 0; c < NB; c++) {
-                    if (has_row(c)) {
-                        const T d = table[(r * p.n_red + c) * WAVE + lane];
-                        out[(r * NB + c) & 1] = M::mma(d, acc[c][r], out[(r * NB + c) & 1]);
+                    to[c] = table[(block * p.n_red + (EXACT ? c : min(c, p.n_red - 1))) * WAVE + lane];
+                }
+            };
+            read(d[0], 0);
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                if (r + 1 < 4) {
+                    read(d[(r + 1) & 1], r + 1);
+                }
+                if (r < registers) { // (uniform)
+#pragma unroll
+                    for (int c = 0; c < NB; c++) {
+                        if (has_row(c)) {
+                            out[c & 3] = M::mma(d[r & 1][c], acc[c][r], out[c & 3]);
+                        }
+                    }
+                }
+            }
+        } else {
+            // (double: the registers for operands read ahead are not there)
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                if (r < registers) { // (uniform)
+#pragma unroll
+                    for (int c = 0; c < NB; c++) {
+                        if (has_row(c)) {
+                            const T d = table[(r * p.n_red + c) * WAVE + lane];
+                            out[(r * NB + c) & 1] = M::mma(d, acc[c][r], out[(r * NB + c) & 1]);
+                        }
                     }
                 }
             }
@@ -514,7 +566,11 @@ template <typename T, int NB, bool EXACT, bool COMPACT = false> struct NodeSum {
         for (int r = 0; r < 4; r++) {
             const int32_t row = M::row(lane, r);
             if (row < p.n_out && column_inside) {
-                target[static_cast<size_t>(row) * p.ld] = out[0][r] + out[1][r];
+                if constexpr (sizeof(T) == 4) {
+                    target[static_cast<size_t>(row) * p.ld] = (out[0][r] + out[1][r]) + (out[2][r] + out[3][r]);
+                } else {
+                    target[static_cast<size_t>(row) * p.ld] = out[0][r] + out[1][r];
+                }
             }
         }
     }
@@ -796,7 +852,7 @@ template <typename T, int NB, bool EXACT, bool VECTORS> struct EdgeGradients {
 
     const GradientArgs<T>& p;
     int lane, i, q;
-    int32_t steps1, steps3; // ceil(nA / 4), ceil(n3 / 4)
+    int32_t steps1, steps3_of_shape; // ceil(nA / 4), ceil(n3 / 4)
     uint32_t row_bytes, w_block_bytes, g_block_bytes, a_row_bytes;
     BufferOf<T> A, B, W, G;
 
@@ -805,7 +861,7 @@ template <typename T, int NB, bool EXACT, bool VECTORS> struct EdgeGradients {
         i = lane & 15;
         q = lane >> 4;
         steps1 = (p.nA + 3) / 4;
-        steps3 = (p.n3 + 3) / 4;
+        steps3_of_shape = (p.n3 + 3) / 4;
         row_bytes = static_cast<uint32_t>(p.L) * ELEMENT;
         w_block_bytes = static_cast<uint32_t>(p.n2) * row_bytes;
         g_block_bytes = static_cast<uint32_t>(p.n3) * row_bytes;
@@ -817,6 +873,11 @@ template <typename T, int NB, bool EXACT, bool VECTORS> struct EdgeGradients {
     }
 
     __device__ __forceinline__ bool has_row(int c) const { return EXACT || c < p.n2; }
+    /// ceil(n3 / 4): known when the kernel is compiled if no row is padding, and
+    /// the loops over it then have no branch between a read of the table and
+    /// the matrix instruction it feeds (with one, every such pair waits for
+    /// the LDS by itself).
+    __device__ __forceinline__ int32_t steps3_now() const { return EXACT ? (NB + 3) / 4 : steps3_of_shape; }
 
     /// grad_B[e, 16 tile .. 16 tile + 16] for the edges first .. last of `node`.
     /// `near_source`: senders of the 128 positions from `near_begin`.
@@ -846,11 +907,16 @@ template <typename T, int NB, bool EXACT, bool VECTORS> struct EdgeGradients {
 #pragma unroll
         for (int t = 0; t < NB; t++) {
             pairs[t] = M::zero();
-            if (t < pair_tiles) { // (uniform)
+        }
+        // (step by step over all tiles: consecutive matrix instructions belong to
+        // different tiles and do not wait for each other)
 #pragma unroll
-                for (int s3 = 0; s3 < 4; s3++) {
-                    if (s3 < steps3) {
-                        pairs[t] = M::mma(table[(t * steps3 + s3) * WAVE + lane], g_rows[s3], pairs[t]);
+        for (int s3 = 0; s3 < 4; s3++) {
+            if (s3 < steps3_now()) {
+#pragma unroll
+                for (int t = 0; t < NB; t++) {
+                    if (t < pair_tiles) { // (uniform)
+                        pairs[t] = M::mma(table[(t * steps3_now() + s3) * WAVE + lane], g_rows[s3], pairs[t]);
                     }
                 }
             }
@@ -895,7 +961,7 @@ template <typename T, int NB, bool EXACT, bool VECTORS> struct EdgeGradients {
                     (static_cast<uint32_t>(usable ? sender : 0) * w_block_bytes + column_bytes) | unless(usable);
 #pragma unroll
                 for (int c = 0; c < NB; c++) {
-                    w[r][c] = W.load(from, static_cast<uint32_t>(EXACT ? c : min(c, p.n2 - 1)) * row_bytes);
+                    w[r][c] = W.load(from, fresh(static_cast<uint32_t>(EXACT ? c : min(c, p.n2 - 1))) * row_bytes);
                 }
             }
             __builtin_amdgcn_sched_barrier(0);
@@ -980,11 +1046,14 @@ template <typename T, int NB, bool EXACT, bool VECTORS> struct EdgeGradients {
 #pragma unroll
                 for (int c = 0; c < NB; c++) {
                     z[c] = M::zero();
-                    if (has_row(c)) {
+                }
 #pragma unroll
-                        for (int s3 = 0; s3 < 4; s3++) {
-                            if (s3 < steps3) {
-                                z[c] = M::mma(g_columns[s3], table[(c * steps3 + s3) * WAVE + lane], z[c]);
+                for (int s3 = 0; s3 < 4; s3++) {
+                    if (s3 < steps3_now()) {
+#pragma unroll
+                        for (int c = 0; c < NB; c++) {
+                            if (has_row(c)) {
+                                z[c] = M::mma(g_columns[s3], table[(c * steps3_now() + s3) * WAVE + lane], z[c]);
                             }
                         }
                     }
@@ -1008,7 +1077,7 @@ template <typename T, int NB, bool EXACT, bool VECTORS> struct EdgeGradients {
 #pragma unroll
                         for (int c = 0; c < NB; c++) {
                             load_four<T, VECTORS>(
-                                w[c], W, from, static_cast<uint32_t>(EXACT ? c : min(c, p.n2 - 1)) * row_bytes, inside,
+                                w[c], W, from, fresh(static_cast<uint32_t>(EXACT ? c : min(c, p.n2 - 1))) * row_bytes, inside,
                                 unless(usable)
                             );
                         }
@@ -1055,9 +1124,10 @@ template <typename T, int NB> constexpr int gradient_group_threads() {
     return 4 * gradient_waves_per_simd<T, NB>() * WAVE;
 }
 
-template <typename T, int NB, bool VECTORS>
+/// EXACT: n2 = n3 = NB, no row of a block is padding (otherwise the block rows are
+/// compared with n2 / n3 as the loops go).
+template <typename T, int NB, bool EXACT, bool VECTORS>
 __global__ __launch_bounds__((gradient_group_threads<T, NB>())) void gradients_kernel(const GradientArgs<T> args) {
-    constexpr bool EXACT = false; // (the block rows are compared with n2 / n3 as the loops go)
     constexpr int THREADS = gradient_group_threads<T, NB>();
     constexpr int GROUP_WAVES = THREADS / WAVE;
     static_assert(GROUP_WAVES >= 3, "a wavefront per layout of the table");
@@ -1489,14 +1559,22 @@ void vjp(
         const unsigned grid =
             static_cast<unsigned>(std::min<int64_t>(compute_units(), (units + GROUP_WAVES - 1) / GROUP_WAVES));
         (void)fits;
-        if (vectors) {
-            auto kernel = gradients_kernel<T, NB, true>;
+        auto launch = [&](auto exact, auto with_vectors) {
+            auto kernel = gradients_kernel<T, NB, decltype(exact)::value, decltype(with_vectors)::value>;
             allow_lds(kernel, lds);
             kernel<<<grid, gradient_group_threads<T, NB>(), lds, stream>>>(args);
+        };
+        // (double: with the conditions gone the compiler moves so many reads ahead
+        // that registers spill, 121 against 105 us at 60 000 edges)
+        const bool exact = sizeof(T) == 4 && s.n2 == NB && s.n3 == NB;
+        if (exact && vectors) {
+            launch(std::true_type{}, std::true_type{});
+        } else if (exact) {
+            launch(std::true_type{}, std::false_type{});
+        } else if (vectors) {
+            launch(std::false_type{}, std::true_type{});
         } else {
-            auto kernel = gradients_kernel<T, NB, false>;
-            allow_lds(kernel, lds);
-            kernel<<<grid, gradient_group_threads<T, NB>(), lds, stream>>>(args);
+            launch(std::false_type{}, std::false_type{});
         }
     });
     MOPS_HIP_CHECK(hipGetLastError());
