@@ -273,8 +273,10 @@ __global__ __launch_bounds__(WAVE) void vjp_kernel(
 // (prefix * suffix, 3 K multiplications instead of K^2) live in registers, and
 // the factors of the next monomial are fetched while the current one is used.
 // ---------------------------------------------------------------------------
+constexpr int ORDERED_VJP_THREADS = 4 * WAVE; // one wavefront that walks the monomials and three helpers
+
 template <typename T, int ORDER, bool ALL_FEATURES>
-__global__ __launch_bounds__(WAVE) void vjp_ordered_kernel(
+__global__ __launch_bounds__(ORDERED_VJP_THREADS) void vjp_ordered_kernel(
     T* __restrict__ grad_A,
     const T* __restrict__ grad_output,
     const T* __restrict__ A,
@@ -299,10 +301,15 @@ __global__ __launch_bounds__(WAVE) void vjp_ordered_kernel(
     const int32_t feature_begin = ALL_FEATURES ? 0 : blockIdx.y * span;
     const int32_t feature_count = ALL_FEATURES ? nA : min(span, nA - feature_begin);
 
+    // Thread (r, g) of the FIRST wavefront walks the monomials; the other
+    // wavefronts of the workgroup only help to stage the rows, to clear the
+    // accumulators and to add up the copies, which a single wavefront would
+    // spend a third of the launch on.
     const int tid = threadIdx.x;
+    const bool walks = tid < WAVE;
     const int G = WAVE >> log2_R;
     const int r = tid & (R - 1);
-    const int g = tid >> log2_R;
+    const int g = (tid & (WAVE - 1)) >> log2_R;
     const int32_t row0 = blockIdx.x * R;
     const int32_t rows = min(R, n_rows - row0);
 
@@ -329,26 +336,29 @@ __global__ __launch_bounds__(WAVE) void vjp_ordered_kernel(
     // memory meanwhile, those of the first one while the tiles are set up.
     constexpr int BATCH = 8;
     Monomial queue[BATCH];
+    T upstream = T(0);
+    if (walks) {
 #pragma unroll
-    for (int d = 0; d < BATCH; d++) {
-        fetch(queue[d], g + d * G);
+        for (int d = 0; d < BATCH; d++) {
+            fetch(queue[d], g + d * G);
+        }
+        upstream = grad_output[min(row0 + r, n_rows - 1)];
     }
-    const T upstream = grad_output[min(row0 + r, n_rows - 1)];
 
     // the rows of A, STAGE values per lane asked for together: with one load
     // per turn of a loop, each turn would wait a whole round trip to memory
     const T* a_src = A + static_cast<size_t>(row0) * nA;
     constexpr int STAGE = 8;
-    for (int32_t base = 0; base < rows * nA; base += STAGE * WAVE) {
+    for (int32_t base = 0; base < rows * nA; base += STAGE * ORDERED_VJP_THREADS) {
         T staged[STAGE];
 #pragma unroll
         for (int u = 0; u < STAGE; u++) {
-            const int32_t i = base + u * WAVE + tid;
+            const int32_t i = base + u * ORDERED_VJP_THREADS + tid;
             staged[u] = a_src[min(i, rows * nA - 1)];
         }
 #pragma unroll
         for (int u = 0; u < STAGE; u++) {
-            const int32_t i = base + u * WAVE + tid;
+            const int32_t i = base + u * ORDERED_VJP_THREADS + tid;
             if (i < rows * nA) {
                 const int32_t row = i / nA;
                 a_stage[((i - row * nA) << log2_R) + row] = staged[u];
@@ -358,27 +368,36 @@ __global__ __launch_bounds__(WAVE) void vjp_ordered_kernel(
     if (tid < R) {
         a_stage[nA * R + tid] = T(0);
     }
-    // (G * R = 64 threads: every lane clears feature_count + 1 values, a
-    // wavefront's worth apart; unrolled, because a single wavefront pays for
-    // every instruction of the loop around a store)
+    // (G * R = 64: the accumulators are feature_count + 1 rows of 64 values, one
+    // per lane; wavefront w clears rows w, w + 4, ...; unrolled, because a
+    // wavefront pays for every instruction of the loop around a store)
     {
-        T* clear = accumulator + tid;
-        int32_t k = 0;
-        for (; k + 8 <= feature_count + 1; k += 8) {
+        constexpr int HELPERS = ORDERED_VJP_THREADS / WAVE;
+        T* clear = accumulator + (tid & (WAVE - 1));
+        int32_t k = tid >> 6;
+        for (; k + 7 * HELPERS < feature_count + 1; k += 8 * HELPERS) {
 #pragma unroll
             for (int u = 0; u < 8; u++) {
-                clear[(k + u) * WAVE] = T(0);
+                clear[(k + u * HELPERS) * WAVE] = T(0);
             }
         }
-        for (; k < feature_count + 1; k++) {
+        for (; k < feature_count + 1; k += HELPERS) {
             clear[k * WAVE] = T(0);
         }
     }
     __syncthreads();
 
-    if (r < rows) {
+    if (walks && r < rows) {
         T* mine = accumulator + static_cast<size_t>(g) * (feature_count + 1) * R + r;
         const T* my_a = a_stage + r;
+        // a feature's distance in bytes as a shift: address = base + (feature << shift), one
+        // instruction (shift-and-add) per LDS access instead of a shift, a scaling and an add
+        const int32_t byte_shift = log2_R + (sizeof(T) == 8 ? 3 : 2);
+        auto at = [&](auto* base, uint32_t feature) {
+            using Pointer = decltype(base);
+            using Bytes = std::conditional_t<std::is_const_v<std::remove_pointer_t<Pointer>>, const char*, char*>;
+            return reinterpret_cast<Pointer>(reinterpret_cast<Bytes>(base) + (feature << byte_shift));
+        };
         const uint32_t features = static_cast<uint32_t>(nA);
         const uint32_t kept = static_cast<uint32_t>(feature_count);
         // `whole`: all monomials of the batch exist
@@ -393,7 +412,7 @@ __global__ __launch_bounds__(WAVE) void vjp_ordered_kernel(
                 for (int k = 0; k < ORDER; k++) {
                     // (as unsigned, a negative factor is a large one)
                     const uint32_t feature = min(static_cast<uint32_t>(now[d].factor[k]), features);
-                    value[d][k] = my_a[feature << log2_R];
+                    value[d][k] = *at(my_a, feature);
                 }
             }
             if constexpr (WHOLE) {
@@ -429,7 +448,7 @@ __global__ __launch_bounds__(WAVE) void vjp_ordered_kernel(
                         slot -= static_cast<uint32_t>(feature_begin);
                     }
                     slot = min(slot, kept);
-                    T* to = mine + ((exists ? slot : kept) << log2_R);
+                    T* to = at(mine, exists ? slot : kept);
                     // a slot of my own. In f64 the LDS add instruction, which saves the
                     // round trip of read, add, write; in f32 that instruction is the
                     // slower way here (53 us against 21)
@@ -457,7 +476,7 @@ __global__ __launch_bounds__(WAVE) void vjp_ordered_kernel(
     // a quarter as long as one sum over all copies would be.
     T* dst = grad_A + static_cast<size_t>(row0) * nA + feature_begin;
     const int32_t copy_stride = (feature_count + 1) * R;
-    for (int32_t entry = tid; entry < feature_count * R; entry += WAVE) {
+    for (int32_t entry = tid; entry < feature_count * R; entry += ORDERED_VJP_THREADS) {
         const int32_t row = entry & (R - 1);
         const int32_t feature = entry >> log2_R;
         const T* from = accumulator + entry;
@@ -1305,12 +1324,12 @@ void homogeneous_polynomial_evaluation_vjp(MOPS_HPE_VJP_PARAMS(MOPS_CXX_FIRST, M
         MainKernelTimer timer(stream);
 #define MOPS_LAUNCH_ORDERED(ORDER)                                                                  \
     if (span == nA) {                                                                              \
-        vjp_ordered_kernel<scalar_t, ORDER, true><<<blocks, WAVE, lds, stream>>>(                  \
+        vjp_ordered_kernel<scalar_t, ORDER, true><<<blocks, ORDERED_VJP_THREADS, lds, stream>>>(                  \
             grad_A.data, grad_output.data, A.data, C.data, indices_A.data, n_rows, nA,             \
             n_monomials, log2_R, span                                                              \
         );                                                                                         \
     } else {                                                                                       \
-        vjp_ordered_kernel<scalar_t, ORDER, false><<<blocks, WAVE, lds, stream>>>(                 \
+        vjp_ordered_kernel<scalar_t, ORDER, false><<<blocks, ORDERED_VJP_THREADS, lds, stream>>>(                 \
             grad_A.data, grad_output.data, A.data, C.data, indices_A.data, n_rows, nA,             \
             n_monomials, log2_R, span                                                              \
         );                                                                                         \
