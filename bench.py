@@ -60,7 +60,7 @@ MAIN_KERNELS = {
     ("opsaw", "forward"): "forward_kernel<{T}, 2, true>",
     ("opsaw", "vjp"): "edge_rows_vjp_kernel<{T}, 1, 2, true, true, false, true>",
     ("sasaw", "forward"): "sasaw_segments::contract_kernel<{T}, 9, true, ",
-    ("sasaw", "vjp"): "sasaw_segments::gradients_kernel<{T}, 9, true>",
+    ("sasaw", "vjp"): "sasaw_segments::gradients_kernel<{T}, 9, ",
 }
 
 
