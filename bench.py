@@ -59,9 +59,23 @@ MAIN_KERNELS = {
     ("opsa", "vjp"): "edge_rows_vjp_kernel<{T}, 1, 2, false, true, false, false>",
     ("opsaw", "forward"): "forward_kernel<{T}, 2, true>",
     ("opsaw", "vjp"): "edge_rows_vjp_kernel<{T}, 1, 2, true, true, false, true>",
-    ("sasaw", "forward"): "sasaw_segments::contract_kernel<{T}, 9, true, ",
-    ("sasaw", "vjp"): "sasaw_segments::gradients_kernel<{T}, 9, ",
+    ("sasaw", "forward"): {
+        "float": "sasaw_segments::contract_kernel<float, 9, true, 32>",
+        "double": "sasaw_segments::contract_kernel<double, 9, true, 64>",
+    },
+    ("sasaw", "vjp"): {
+        "float": "sasaw_segments::gradients_kernel<float, 9, true, true>",
+        "double": "sasaw_segments::gradients_kernel<double, 9, false, true>",
+    },
 }
+
+
+def main_kernel_name(op, kind, type_name):
+    """Name of the main kernel of ``op``'s ``kind`` call for elements of C++ type ``type_name``."""
+    entry = MAIN_KERNELS.get((op, kind), "?")
+    if isinstance(entry, dict):
+        return entry[type_name]
+    return entry.format(T=type_name)
 
 
 def nbytes(arrays):
@@ -441,7 +455,7 @@ def main():
 
             if config.startswith("c"):
                 kernel_seconds, launches = main_kernel_time(library, function, 200)
-                name = MAIN_KERNELS.get((op_name, kind), "?").format(T=type_name)
+                name = main_kernel_name(op_name, kind, type_name)
                 timed_by = "HIP events around the kernel on its launch stream, eager calls, rotating inputs"
                 if kernel_seconds is None:
                     # this call's kernels carry no events: the whole call as one interval
@@ -478,7 +492,7 @@ def main():
         if kernel_seconds is None:
             kernel_seconds, _ = device_time_per_call(w.vjp, w.n_sets, 20, device)
             launches = w.n_sets * 20
-        name = MAIN_KERNELS[("sasaw", "vjp")].format(T="double")
+        name = main_kernel_name("sasaw", "vjp", "double")
         dominant = {
             "config": "c4", "op": "sasaw", "dtype": "float64", "function": "vjp", "kernel": name,
             "avg_us": round(kernel_seconds * 1e6, 3), "launches_timed": launches,
