@@ -463,7 +463,11 @@ template <typename T, int NB, bool EXACT, bool COMPACT = false> struct NodeSum {
         // instructions of this one. AHEAD batches are on their way while one is
         // multiplied: a round trip to memory lasts several times as long as the
         // matrix instructions of a batch.
-        constexpr int AHEAD = 2;
+        // (measured at 60 000 edges: the forward kernel with 1 / 2 / 3 batches ahead
+        // takes 22.3 / 24.9 / 27.8 us in float, 31.6 / 32.4 / 33.9 in double: operands
+        // further ahead cost registers, which are spilled; the kernel with several
+        // roles: no difference between 1, 2 and 3)
+        constexpr int AHEAD = COMPACT ? 2 : 1;
         constexpr int BATCHES = WAVE / BATCH;
         if constexpr (COMPACT) {
             // (a kernel with other roles beside this one: the same in rounds of
@@ -1354,9 +1358,8 @@ template <typename Kernel> void allow_lds(Kernel kernel, size_t lds) {
 
 /// Positions of the sorted index per unit of work: the fewest of 16, 32, 64
 /// with which every wavefront that is resident on the device has at most one
-/// unit (measured at 60 000 edges, 2 column tiles: float, 4096 wavefronts: 30 us
-/// with 8, 27 with 16, 25 with 32, 32 with 64; double, 2048 wavefronts: 41, 36,
-/// 36, 31).
+/// unit (measured at 60 000 edges, 2 column tiles: float, 4096 wavefronts: 25 us
+/// with 16, 22 with 32, 29 with 64; double, 2048 wavefronts: 41, 36, 31.5).
 int32_t chunk_for(int32_t n_edges, int32_t column_tiles, int64_t resident_waves) {
     for (int32_t chunk : {16, 32}) {
         if ((static_cast<int64_t>(n_edges) + chunk - 1) / chunk * column_tiles <= resident_waves) {
