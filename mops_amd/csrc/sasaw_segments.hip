@@ -1001,7 +1001,10 @@ template <typename T, int NB, bool EXACT, bool VECTORS> struct EdgeGradients {
         const T* __restrict__ table, int32_t node, int32_t first, int32_t last, const int32_t (&near_source)[2],
         int32_t near_begin
     ) const {
-        constexpr int TILES = 4; // tiles of 16 edges whose sums over the columns are in registers together
+        // tiles of 16 edges whose sums over the columns are in registers together (Z' of a
+        // column tile serves them all; measured at 60 000 edges with 1 / 2 / 4: float
+        // 62.7 / 59.9 / 62.9 us, double 111.7 / 106.2 / 121.6)
+        constexpr int TILES = 2;
         const int lane = opaque(this->lane);
         const int i = lane & 15, q = lane >> 4;
         // row `row` of a tile of Z' stands for column 4 q + r of the 16 (the lane
@@ -1567,9 +1570,7 @@ void vjp(
             allow_lds(kernel, lds);
             kernel<<<grid, gradient_group_threads<T, NB>(), lds, stream>>>(args);
         };
-        // (double: with the conditions gone the compiler moves so many reads ahead
-        // that registers spill, 121 against 105 us at 60 000 edges)
-        const bool exact = sizeof(T) == 4 && s.n2 == NB && s.n3 == NB;
+        const bool exact = s.n2 == NB && s.n3 == NB;
         if (exact && vectors) {
             launch(std::true_type{}, std::true_type{});
         } else if (exact) {
