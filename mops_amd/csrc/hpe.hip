@@ -116,8 +116,10 @@ __global__ __launch_bounds__(256) void forward_ordered_kernel(
     int32_t R
 ) {
     extern __shared__ __align__(16) unsigned char lds_bytes[];
+    // a[nA + 1][R]: the row after the last stays zero, a factor outside [0, nA)
+    // reads it, and the loop over the monomials has no branch in it
     T* a_stage = reinterpret_cast<T*>(lds_bytes);
-    T* partial = a_stage + static_cast<size_t>(nA) * R;
+    T* partial = a_stage + static_cast<size_t>(nA + 1) * R;
 
     const int tid = threadIdx.x;
     const int G = blockDim.x / R;
@@ -130,6 +132,9 @@ __global__ __launch_bounds__(256) void forward_ordered_kernel(
     for (int32_t i = tid; i < rows * nA; i += blockDim.x) {
         int32_t row = i / nA;
         a_stage[(i - row * nA) * R + row] = a_src[i];
+    }
+    if (tid < R) {
+        a_stage[nA * R + tid] = T(0);
     }
     __syncthreads();
 
@@ -146,19 +151,44 @@ __global__ __launch_bounds__(256) void forward_ordered_kernel(
         }
         to.coefficient = C[safe];
     };
+    // BATCH monomials at a time: their factors asked for together, then their
+    // values of A, then the products (independent chains); a monomial beyond
+    // the last counts with coefficient zero.
     T sum = T(0);
     if (r < rows && n_monomials > 0) {
-        Monomial next;
-        fetch(next, g);
-        for (int32_t j = g; j < n_monomials; j += G) {
-            const Monomial now = next;
-            fetch(next, j + G);
-            T product = now.coefficient;
+        constexpr int BATCH = 4;
+        const uint32_t features = static_cast<uint32_t>(nA);
+        const T* my_a = a_stage + r;
+        Monomial next[BATCH];
 #pragma unroll
-            for (int k = 0; k < ORDER; k++) {
-                product *= in_bounds(now.factor[k], nA) ? a_stage[now.factor[k] * R + r] : T(0);
+        for (int d = 0; d < BATCH; d++) {
+            fetch(next[d], g + d * G);
+        }
+        for (int32_t j0 = g; j0 < n_monomials; j0 += BATCH * G) {
+            Monomial now[BATCH];
+            T value[BATCH][ORDER > 0 ? ORDER : 1];
+#pragma unroll
+            for (int d = 0; d < BATCH; d++) {
+                now[d] = next[d];
+#pragma unroll
+                for (int k = 0; k < ORDER; k++) {
+                    // (as unsigned, a negative factor is a large one)
+                    value[d][k] = my_a[min(static_cast<uint32_t>(now[d].factor[k]), features) * R];
+                }
             }
-            sum += product;
+#pragma unroll
+            for (int d = 0; d < BATCH; d++) {
+                fetch(next[d], j0 + (d + BATCH) * G);
+            }
+#pragma unroll
+            for (int d = 0; d < BATCH; d++) {
+                T product = j0 + d * G < n_monomials ? now[d].coefficient : T(0);
+#pragma unroll
+                for (int k = 0; k < ORDER; k++) {
+                    product *= value[d][k];
+                }
+                sum += product;
+            }
         }
     }
     // lanes with the same r inside a wavefront, then the wavefronts
@@ -1144,9 +1174,9 @@ void homogeneous_polynomial_evaluation(MOPS_HPE_PARAMS(MOPS_CXX_FIRST, MOPS_CXX_
         return;
     }
     // per row: its A values plus one partial sum per group (G <= THREADS)
-    int R = pick_rows(n_rows, (static_cast<size_t>(nA) + THREADS) * sizeof(scalar_t));
+    int R = pick_rows(n_rows, (static_cast<size_t>(nA) + 1 + THREADS) * sizeof(scalar_t));
     if (R > 0) {
-        size_t lds = (static_cast<size_t>(nA) * R + THREADS) * sizeof(scalar_t);
+        size_t lds = ((static_cast<size_t>(nA) + 1) * R + THREADS) * sizeof(scalar_t);
         unsigned blocks = static_cast<unsigned>(ceil_div(static_cast<size_t>(n_rows), R));
         MainKernelTimer timer(stream);
 #define MOPS_LAUNCH_ORDERED(ORDER)                                                                  \
