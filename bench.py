@@ -65,7 +65,7 @@ MAIN_KERNELS = {
     },
     ("sasaw", "vjp"): {
         "float": "sasaw_segments::gradients_kernel<float, 9, true, true>",
-        "double": "sasaw_segments::gradients_kernel<double, 9, false, true>",
+        "double": "sasaw_segments::gradients_kernel<double, 9, true, true>",
     },
 }
 
