@@ -36,6 +36,14 @@
 //
 // The reference has no device implementation of this operation
 // (mops/src/sasaw/sasaw.cu:1, mops/src/sasaw/cuda.tpp:18).
+//
+// This file holds the entry points and the GENERAL kernels described above.
+// Tables whose component indices have at most 16 values each (equivariant
+// message passing) do not get here: the entry points hand them to the
+// persistent matrix-core kernels of sasaw_segments.hip (per-node sums of
+// rank-one updates; one launch for the forward pass, one for all three
+// gradients) and, where those refuse (grad_W on graphs too dense for the
+// senders' slots, byte offsets beyond 32 bits), to sasaw_mfma.hip.
 #include <algorithm>
 #include <atomic>
 #include <stdexcept>

@@ -22,7 +22,7 @@
 //
 //   grad_W[w, m2, l] = sum_{m1, m3} D[m3, m2, m1] * sum_{e: PW1[e] = w} A[e, m1] * (B[e, l] * G[PO1[e], m3, l])
 //
-// grad_A and grad_B: see edge_gradients below.
+// grad_A and grad_B: see "grad_A and grad_B" below (EdgeGradients).
 //
 // The dense table is built by every workgroup for itself in LDS, in operand
 // layout, entries of one cell added in ascending entry order (no launch of its
