@@ -59,8 +59,9 @@ constexpr int BLOCK = WAVES_PER_BLOCK * WAVE;
 // NT = number of 16-column tiles of L accumulated at once.
 // MFMA roles: D rows = k, D columns = l, reduction = edges (4 per instruction)
 // ---------------------------------------------------------------------------
+// (byte offsets beyond 32 bits: addresses of 64 bits, a choice of address and of result per load)
 template <typename T, int NT, bool WEIGHTED>
-__device__ __forceinline__ void forward_segment(
+__device__ __forceinline__ void forward_segment_wide(
     T* __restrict__ out_row,
     const T* __restrict__ A,
     const T* __restrict__ B,
@@ -165,7 +166,145 @@ __device__ __forceinline__ void forward_segment(
     }
 }
 
-template <typename T, int NT, bool WEIGHTED>
+/// A tensor as a buffer: a load is a uniform descriptor, a 32-bit byte offset
+/// per lane and a uniform byte offset (the hardware adds the three), and an
+/// offset beyond the tensor reads as zero without touching memory: a lane
+/// that has nothing to load gets all ones OR-ed into its offset, which costs
+/// one instruction where a choice of address and of result costs three.
+template <typename T> struct RowBuffer {
+    __amdgpu_buffer_rsrc_t descriptor;
+    __device__ __forceinline__ explicit RowBuffer(const T* base) {
+        descriptor = __builtin_amdgcn_make_buffer_rsrc(
+            const_cast<T*>(base), 0, static_cast<int>(0xfffffff0u), 0x00020000
+        );
+    }
+    __device__ __forceinline__ T load(uint32_t lane_bytes, uint32_t uniform_bytes) const {
+        if constexpr (sizeof(T) == 4) {
+            return __builtin_bit_cast(T, __builtin_amdgcn_raw_buffer_load_b32(descriptor, lane_bytes, uniform_bytes, 0));
+        } else {
+            return __builtin_bit_cast(T, __builtin_amdgcn_raw_buffer_load_b64(descriptor, lane_bytes, uniform_bytes, 0));
+        }
+    }
+};
+/// All ones unless `wanted`.
+__device__ __forceinline__ uint32_t unless(bool wanted) { return static_cast<uint32_t>(wanted) - 1u; }
+
+template <typename T, int NT, bool WEIGHTED, bool NARROW>
+__device__ __forceinline__ void forward_segment(
+    T* __restrict__ out_row,
+    const T* __restrict__ A,
+    const T* __restrict__ B,
+    const T* __restrict__ W,
+    const int32_t* __restrict__ indices_W,
+    int32_t n_weights,
+    int32_t first,
+    int32_t last,
+    int32_t K,
+    int32_t L
+) {
+    if constexpr (!NARROW) {
+        forward_segment_wide<T, NT, WEIGHTED>(out_row, A, B, W, indices_W, n_weights, first, last, K, L);
+        return;
+    }
+    using M = Mfma<T>;
+    constexpr int UNROLL = 8; // 32 edges in flight per iteration
+    constexpr uint32_t ES = sizeof(T);
+    const int lane = threadIdx.x & (WAVE - 1);
+    const int sub = lane & 15;
+    const int quarter = lane >> 4;
+    const RowBuffer<T> rows_A(A), rows_B(B), rows_W(W);
+    const RowBuffer<int32_t> rows_of_W(indices_W);
+    const uint32_t a_row_bytes = static_cast<uint32_t>(K) * ES;
+    const uint32_t b_row_bytes = static_cast<uint32_t>(L) * ES;
+
+    for (int32_t k0 = 0; k0 < K; k0 += 16) {
+        const int32_t k = k0 + sub;
+        const uint32_t a_lane = (static_cast<uint32_t>(quarter) * a_row_bytes + static_cast<uint32_t>(k) * ES) | unless(k < K);
+        for (int32_t l0 = 0; l0 < L; l0 += 16 * NT) {
+            uint32_t b_lane[NT], w_column[NT], no_column[NT];
+#pragma unroll
+            for (int t = 0; t < NT; t++) {
+                const int32_t col = l0 + 16 * t + sub;
+                no_column[t] = unless(col < L);
+                w_column[t] = static_cast<uint32_t>(col) * ES;
+                b_lane[t] = (static_cast<uint32_t>(quarter) * b_row_bytes + w_column[t]) | no_column[t];
+            }
+            typename M::Acc acc[NT];
+#pragma unroll
+            for (int t = 0; t < NT; t++) {
+                acc[t] = M::zero();
+            }
+            for (int32_t e0 = first; e0 < last; e0 += 4 * UNROLL) {
+                T a[UNROLL];
+                T b[UNROLL][NT];
+                T w[WEIGHTED ? UNROLL : 1][NT];
+                uint32_t beyond[UNROLL]; // all ones for a lane whose edge is not of this segment
+                int32_t w_row[UNROLL];
+#pragma unroll
+                for (int u = 0; u < UNROLL; u++) {
+                    beyond[u] = unless(e0 + 4 * u + quarter < last);
+                    if (WEIGHTED) {
+                        w_row[u] = rows_of_W.load(static_cast<uint32_t>(quarter) * 4u | beyond[u], static_cast<uint32_t>(e0 + 4 * u) * 4u);
+                    }
+                }
+#pragma unroll
+                for (int u = 0; u < UNROLL; u++) {
+                    const uint32_t row = static_cast<uint32_t>(e0 + 4 * u); // (uniform)
+                    a[u] = rows_A.load(a_lane | beyond[u], row * a_row_bytes);
+#pragma unroll
+                    for (int t = 0; t < NT; t++) {
+                        b[u][t] = rows_B.load(b_lane[t] | beyond[u], row * b_row_bytes);
+                    }
+                }
+                if (WEIGHTED) {
+#pragma unroll
+                    for (int u = 0; u < UNROLL; u++) {
+                        const uint32_t from = static_cast<uint32_t>(w_row[u]) * b_row_bytes;
+                        const uint32_t nothing = unless(in_bounds(w_row[u], n_weights)) | beyond[u];
+#pragma unroll
+                        for (int t = 0; t < NT; t++) {
+                            w[u][t] = rows_W.load((from + w_column[t]) | nothing | no_column[t], 0);
+                        }
+                    }
+                    if (NT >= 4) {
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+#pragma unroll
+                    for (int u = 0; u < UNROLL; u++) {
+#pragma unroll
+                        for (int t = 0; t < NT; t++) {
+                            b[u][t] *= w[u][t];
+                        }
+                    }
+                }
+                // keep every load above ahead of the first matrix instruction:
+                // the loads of all 32 edges are meant to be in flight together
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int u = 0; u < UNROLL; u++) {
+#pragma unroll
+                    for (int t = 0; t < NT; t++) {
+                        acc[t] = M::mma(a[u], b[u][t], acc[t]);
+                    }
+                }
+            }
+#pragma unroll
+            for (int t = 0; t < NT; t++) {
+                const int32_t col = l0 + 16 * t + sub;
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    const int32_t row_k = k0 + M::row(lane, r);
+                    if (row_k < K && col < L) {
+                        out_row[static_cast<size_t>(row_k) * L + col] = acc[t][r];
+                    }
+                }
+            }
+        }
+    }
+}
+
+/// NARROW: every tensor is smaller than 4 GB, byte offsets of 32 bits (see RowBuffer).
+template <typename T, int NT, bool WEIGHTED, bool NARROW>
 __global__ __launch_bounds__(BLOCK) void forward_kernel(
     T* __restrict__ output,
     const T* __restrict__ A,
@@ -188,7 +327,7 @@ __global__ __launch_bounds__(BLOCK) void forward_kernel(
         n_output,
         wave_index,
         [&](int32_t row, int32_t first, int32_t last) {
-            forward_segment<T, NT, WEIGHTED>(
+            forward_segment<T, NT, WEIGHTED, NARROW>(
                 output + row * row_elements, A, B, W, indices_W, n_output, first, last, K, L
             );
         },
@@ -215,7 +354,7 @@ __global__ __launch_bounds__(BLOCK) void forward_kernel(
 // ---------------------------------------------------------------------------
 constexpr int SPLIT = 256;
 
-template <typename T, int NT, bool WEIGHTED>
+template <typename T, int NT, bool WEIGHTED, bool NARROW>
 __global__ __launch_bounds__(BLOCK) void forward_split_kernel(
     T* __restrict__ output,
     T* __restrict__ tails,
@@ -244,7 +383,7 @@ __global__ __launch_bounds__(BLOCK) void forward_split_kernel(
             T* target = from_start && to_end ? output + row * row_elements
                         : from_start         ? tails + block * row_elements
                                              : heads + block * row_elements;
-            forward_segment<T, NT, WEIGHTED>(target, A, B, W, indices_W, n_output, first, last, K, L);
+            forward_segment<T, NT, WEIGHTED, NARROW>(target, A, B, W, indices_W, n_output, first, last, K, L);
         },
         [&](int32_t begin, int32_t end) {
             T* base = output + begin * row_elements;
@@ -1323,6 +1462,11 @@ void launch_forward(
         return;
     }
     const unsigned blocks = blocks_for(n_edges);
+    // byte offsets of 32 bits into A, B, W and the index of the weight rows (a wavefront asks
+    // for up to 36 positions past the end of a segment, with a mask: room for that too)
+    const uint64_t widest_row = static_cast<uint64_t>(std::max(K, L)) * sizeof(T);
+    const bool narrow = (static_cast<uint64_t>(n_edges) + 64) * std::max<uint64_t>(widest_row, 4) < (uint64_t(1) << 32) - 64 &&
+                        (static_cast<uint64_t>(n_output) + 1) * widest_row < (uint64_t(1) << 32) - 64;
     // few rows with many edges each: cut the segments and add the pieces up
     // (twice SPLIT edges per row on average, or it is not worth a second kernel)
     if (static_cast<size_t>(n_edges) >= static_cast<size_t>(n_output) * 2 * SPLIT && n_edges > SPLIT) {
@@ -1333,10 +1477,17 @@ void launch_forward(
         T* tails = reinterpret_cast<T*>(workspace);
         T* heads = reinterpret_cast<T*>(workspace + pieces_bytes);
 #define MOPS_LAUNCH_SPLIT(NT)                                                                      \
-    forward_split_kernel<T, NT, WEIGHTED><<<blocks, BLOCK, 0, stream>>>(                           \
-        output.data, tails, heads, A.data, B.data, W, indices_W, indices_output.data, n_edges,     \
-        n_output, K, L                                                                             \
-    )
+    if (narrow) {                                                                                  \
+        forward_split_kernel<T, NT, WEIGHTED, true><<<blocks, BLOCK, 0, stream>>>(                 \
+            output.data, tails, heads, A.data, B.data, W, indices_W, indices_output.data, n_edges, \
+            n_output, K, L                                                                         \
+        );                                                                                         \
+    } else {                                                                                       \
+        forward_split_kernel<T, NT, WEIGHTED, false><<<blocks, BLOCK, 0, stream>>>(                \
+            output.data, tails, heads, A.data, B.data, W, indices_W, indices_output.data, n_edges, \
+            n_output, K, L                                                                         \
+        );                                                                                         \
+    }
         if (L <= 16) {
             MOPS_LAUNCH_SPLIT(1);
         } else if (L <= 32) {
@@ -1355,9 +1506,17 @@ void launch_forward(
     {
     MainKernelTimer timer(stream);
 #define MOPS_LAUNCH_FORWARD(NT)                                                                    \
-    forward_kernel<T, NT, WEIGHTED><<<blocks, BLOCK, 0, stream>>>(                                 \
-        output.data, A.data, B.data, W, indices_W, indices_output.data, n_edges, n_output, K, L    \
-    )
+    if (narrow) {                                                                                  \
+        forward_kernel<T, NT, WEIGHTED, true><<<blocks, BLOCK, 0, stream>>>(                       \
+            output.data, A.data, B.data, W, indices_W, indices_output.data, n_edges, n_output, K,  \
+            L                                                                                      \
+        );                                                                                         \
+    } else {                                                                                       \
+        forward_kernel<T, NT, WEIGHTED, false><<<blocks, BLOCK, 0, stream>>>(                      \
+            output.data, A.data, B.data, W, indices_W, indices_output.data, n_edges, n_output, K,  \
+            L                                                                                      \
+        );                                                                                         \
+    }
     if (L <= 16) {
         MOPS_LAUNCH_FORWARD(1);
     } else if (L <= 32) {
