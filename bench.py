@@ -55,9 +55,9 @@ MAIN_KERNELS = {
     ("hpe", "vjp"): "vjp_ordered_kernel<{T}, 4, true>",
     ("sap", "forward"): "sap_mfma::forward_kernel<{T}, 2, 2>",
     ("sap", "vjp"): "sap_mfma::vjp_kernel<{T}, 5>",
-    ("opsa", "forward"): "forward_kernel<{T}, 2, false>",
+    ("opsa", "forward"): "forward_kernel<{T}, 2, false, true>",
     ("opsa", "vjp"): "edge_rows_vjp_kernel<{T}, 1, 2, false, true, false, false>",
-    ("opsaw", "forward"): "forward_kernel<{T}, 2, true>",
+    ("opsaw", "forward"): "forward_kernel<{T}, 2, true, true>",
     ("opsaw", "vjp"): "edge_rows_vjp_kernel<{T}, 1, 2, true, true, false, true>",
     ("sasaw", "forward"): {
         "float": "sasaw_segments::contract_kernel<float, 9, true, 32>",

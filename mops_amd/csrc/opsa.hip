@@ -30,6 +30,7 @@
 // order is fixed (ascending edge number in steps of four), so results are
 // bit-reproducible.
 #include <algorithm>
+#include <cstdlib>
 #include <memory>
 
 #include "mops/opsa.hpp"
@@ -1430,6 +1431,14 @@ __global__ __launch_bounds__(WIDE_WAVES* WAVE) void vjp_wide_kernel(
     }
 }
 
+/// Whether MOPS_AMD_WIDE_OFFSETS is set: the forward kernels for tensors of 4 GB
+/// and more are then used whatever the sizes (what the test of those kernels
+/// does; no other use).
+bool wide_offsets_forced() {
+    const char* value = std::getenv("MOPS_AMD_WIDE_OFFSETS");
+    return value != nullptr && value[0] != '\0' && value[0] != '0';
+}
+
 unsigned blocks_for(int32_t n_edges) {
     size_t waves = ceil_div(static_cast<size_t>(n_edges), CHUNK);
     return static_cast<unsigned>(ceil_div(waves, WAVES_PER_BLOCK));
@@ -1465,7 +1474,8 @@ void launch_forward(
     // byte offsets of 32 bits into A, B, W and the index of the weight rows (a wavefront asks
     // for up to 36 positions past the end of a segment, with a mask: room for that too)
     const uint64_t widest_row = static_cast<uint64_t>(std::max(K, L)) * sizeof(T);
-    const bool narrow = (static_cast<uint64_t>(n_edges) + 64) * std::max<uint64_t>(widest_row, 4) < (uint64_t(1) << 32) - 64 &&
+    const bool narrow = !wide_offsets_forced() &&
+                        (static_cast<uint64_t>(n_edges) + 64) * std::max<uint64_t>(widest_row, 4) < (uint64_t(1) << 32) - 64 &&
                         (static_cast<uint64_t>(n_output) + 1) * widest_row < (uint64_t(1) << 32) - 64;
     // few rows with many edges each: cut the segments and add the pieces up
     // (twice SPLIT edges per row on average, or it is not worth a second kernel)

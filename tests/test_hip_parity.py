@@ -195,6 +195,20 @@ def test_forward(oracle, device, op, name, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES, ids=["f32", "f64"])
+@pytest.mark.parametrize("op,name", [(op, name) for op, name in ALL if op in ("opsa", "opsaw")])
+def test_forward_with_64_bit_offsets(oracle, device, monkeypatch, op, name, dtype):
+    """The forward kernels for tensors of 4 GB and more, forced onto small inputs."""
+    case = CASES[op][name](101, dtype)
+    on_device = to_device(case, device)
+    narrow = hip_forward(op, on_device).cpu().numpy()
+    monkeypatch.setenv("MOPS_AMD_WIDE_OFFSETS", "1")
+    wide = hip_forward(op, on_device).cpu().numpy()
+    assert_close(wide, cpu_forward(oracle, op, case), dtype, f"{op}/{name} wide")
+    # same sums in the same order on both paths
+    assert np.array_equal(wide, narrow), f"{op}/{name}"
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=["f32", "f64"])
 @pytest.mark.parametrize("op,name", ALL)
 def test_vjp(oracle, device, op, name, dtype):
     case = CASES[op][name](202, dtype)
