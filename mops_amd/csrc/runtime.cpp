@@ -1,5 +1,7 @@
 #include "runtime.hpp"
 
+#include <algorithm>
+#include <atomic>
 #include <cstdlib>
 #include <limits>
 #include <mutex>
@@ -311,6 +313,22 @@ void* scratch(size_t bytes) {
 size_t scratch_capacity() {
     auto& st = state();
     return st.resources == nullptr ? 0 : st.resources->capacity;
+}
+
+int32_t compute_units() {
+    static std::atomic<int> cached[64];
+    int device = 0;
+    MOPS_HIP_CHECK(hipGetDevice(&device));
+    if (device < 0 || device >= 64) {
+        return 256;
+    }
+    int count = cached[device].load(std::memory_order_relaxed);
+    if (count == 0) {
+        MOPS_HIP_CHECK(hipDeviceGetAttribute(&count, hipDeviceAttributeMultiprocessorCount, device));
+        count = std::max(count, 1);
+        cached[device].store(count, std::memory_order_relaxed);
+    }
+    return count;
 }
 
 int32_t narrow_i32(size_t value, const char* what) {

@@ -101,6 +101,9 @@ bool set_kernel_timing(bool value);
 /// call on this thread.
 void collect_kernel_time(double* milliseconds, int64_t* launches);
 
+/// Compute units of the current device (asked for once per device).
+int32_t compute_units();
+
 /// ceil(a / b) for positive b.
 inline size_t ceil_div(size_t a, size_t b) { return (a + b - 1) / b; }
 

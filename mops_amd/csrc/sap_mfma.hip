@@ -631,6 +631,191 @@ __global__ __launch_bounds__(THREADS) void vjp_kernel(const Arguments<T> p) {
     }
 }
 
+// ---------------------------------------------------------------------------
+// Many rows (more tiles of 16 rows than a few for every wavefront the device
+// holds): workgroups that stay, build the table once and then let every
+// wavefront walk over tiles of its own, all the work of a tile in one
+// wavefront. After the build no wavefront waits for another; the rows of a
+// wavefront's next tile are asked for before the products of this one.
+
+constexpr int WALK_WAVES = 16;                  // wavefronts per workgroup
+constexpr int WALK_THREADS = WALK_WAVES * WAVE; // (= THREADS: build_operands counts on it)
+static_assert(WALK_THREADS == THREADS, "the table build is written for THREADS threads");
+constexpr int PREFETCH = 8; // loads per lane and tensor: tiles of up to 512 values, rows of up to 32
+
+__device__ __forceinline__ void wave_sync() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+/// The `valid_rows` x `width` values from `global` on (at most PREFETCH * 64), zeros after them.
+template <typename T>
+__device__ __forceinline__ void fetch_rows(
+    T (&values)[PREFETCH], const T* __restrict__ global, int32_t width, int32_t valid_rows, int lane
+) {
+    const int32_t valid = max(min(valid_rows, ROWS_PER_WAVE), 0) * width;
+    // (no branch around a load, not even a uniform one: every load would wait for the one before)
+#pragma unroll
+    for (int u = 0; u < PREFETCH; u++) {
+        const int32_t at = u * WAVE + lane;
+        values[u] = load_or_zero(global, at, at < valid);
+    }
+}
+
+template <typename T>
+__device__ __forceinline__ void place_rows(T* __restrict__ lds, const T (&values)[PREFETCH], int32_t total, int lane) {
+#pragma unroll
+    for (int u = 0; u < PREFETCH; u++) {
+        const int32_t at = u * WAVE + lane;
+        if (at < total) {
+            lds[at] = values[u];
+        }
+    }
+}
+
+template <typename T, int NT, int GROUPS>
+__global__ __launch_bounds__(WALK_THREADS) void forward_walk_kernel(const Arguments<T> p) {
+    using M = Mfma<T>;
+    extern __shared__ __align__(16) char lds_raw[];
+    char* cursor = lds_raw;
+    T* operand = reinterpret_cast<T*>(cursor);
+    cursor += align16(static_cast<size_t>(p.first.size()) * sizeof(T));
+    const BuildAreas<T> areas = carve_build_areas<T>(cursor, p.nA * p.nB * p.nO, p.K);
+    const int lane = threadIdx.x & (WAVE - 1);
+    const int wave = threadIdx.x >> 6;
+    MyEntries<T> entries;
+    entries.load(p.C, p.PA, p.PB, p.PO, p.K);
+    T* mine = reinterpret_cast<T*>(cursor) + wave * ROWS_PER_WAVE * max(p.nA + p.nB, p.nO);
+    T* a_tile = mine;                        // [16][nA]
+    T* b_tile = mine + ROWS_PER_WAVE * p.nA; // [16][nB]
+
+    const int32_t n_tiles = (p.n_rows + ROWS_PER_WAVE - 1) / ROWS_PER_WAVE;
+    const int32_t stride = static_cast<int32_t>(gridDim.x) * WALK_WAVES;
+    int32_t tile = static_cast<int32_t>(blockIdx.x) * WALK_WAVES + wave;
+    T next_a[PREFETCH], next_b[PREFETCH];
+    auto fetch = [&](int32_t which) {
+        const int32_t first_row = min(which, n_tiles - 1) * ROWS_PER_WAVE; // (beyond the end: a tile that exists, no rows of it)
+        const int32_t valid_rows = which < n_tiles ? p.n_rows - first_row : 0;
+        fetch_rows<T>(next_a, p.A + static_cast<size_t>(first_row) * p.nA, p.nA, valid_rows, lane);
+        fetch_rows<T>(next_b, p.B + static_cast<size_t>(first_row) * p.nB, p.nB, valid_rows, lane);
+    };
+    fetch(tile);
+    const OperandTarget<T> targets[1] = {{operand, p.first, {0, 1, 2}}};
+    build_operands<T, 1>(targets, areas, p.nA, p.nB, p.nO, entries); // ends with a barrier
+
+    const int i = lane & 15;
+    const int q = lane >> 4;
+    for (; tile < n_tiles; tile += stride) {
+        place_rows<T>(a_tile, next_a, ROWS_PER_WAVE * p.nA, lane);
+        place_rows<T>(b_tile, next_b, ROWS_PER_WAVE * p.nB, lane);
+        wave_sync();
+        fetch(tile + stride);
+        T inner[ROW_TILES][GROUPS];
+#pragma unroll
+        for (int r = 0; r < ROW_TILES; r++) {
+#pragma unroll
+            for (int g = 0; g < GROUPS; g++) {
+                const int32_t b = 4 * g + q;
+                inner[r][g] = load_or_zero(b_tile, (16 * r + i) * p.nB + b, b < p.nB);
+            }
+        }
+        typename M::Acc acc[ROW_TILES][NT];
+#pragma unroll
+        for (int r = 0; r < ROW_TILES; r++) {
+#pragma unroll
+            for (int t = 0; t < NT; t++) {
+                acc[r][t] = M::zero();
+            }
+        }
+        pair_products<T, NT, GROUPS>(acc, a_tile + i * p.nA, 16 * p.nA, p.nA, inner, operand, lane);
+        wave_sync(); // the tile has been read: its place becomes the staging area of the store
+        const int32_t first_row = tile * ROWS_PER_WAVE;
+        store_rows<T, NT>(p.output + static_cast<size_t>(first_row) * p.nO, mine, acc, p.nO, p.n_rows - first_row, lane);
+        wave_sync();
+    }
+}
+
+template <typename T, int GROUPS>
+__global__ __launch_bounds__(WALK_THREADS) void vjp_walk_kernel(const Arguments<T> p) {
+    using M = Mfma<T>;
+    extern __shared__ __align__(16) char lds_raw[];
+    char* cursor = lds_raw;
+    const bool want_A = p.grad_A != nullptr;
+    const bool want_B = p.grad_B != nullptr;
+    T* operand_A = reinterpret_cast<T*>(cursor);
+    cursor += align16(static_cast<size_t>(want_A ? p.first.size() : 0) * sizeof(T));
+    T* operand_B = reinterpret_cast<T*>(cursor);
+    cursor += align16(static_cast<size_t>(want_B ? p.second.size() : 0) * sizeof(T));
+    const BuildAreas<T> areas = carve_build_areas<T>(cursor, p.nA * p.nB * p.nO, p.K);
+    const int lane = threadIdx.x & (WAVE - 1);
+    const int wave = threadIdx.x >> 6;
+    MyEntries<T> entries;
+    entries.load(p.C, p.PA, p.PB, p.PO, p.K);
+    T* mine = reinterpret_cast<T*>(cursor) + wave * ROWS_PER_WAVE * (p.nA + p.nB + p.nO);
+    T* a_tile = mine;                          // [16][nA]
+    T* b_tile = a_tile + ROWS_PER_WAVE * p.nA; // [16][nB]
+    T* g_tile = b_tile + ROWS_PER_WAVE * p.nB; // [16][nO]
+
+    const int32_t n_tiles = (p.n_rows + ROWS_PER_WAVE - 1) / ROWS_PER_WAVE;
+    const int32_t stride = static_cast<int32_t>(gridDim.x) * WALK_WAVES;
+    int32_t tile = static_cast<int32_t>(blockIdx.x) * WALK_WAVES + wave;
+    T next_a[PREFETCH], next_b[PREFETCH], next_g[PREFETCH];
+    auto fetch = [&](int32_t which) {
+        const int32_t first_row = min(which, n_tiles - 1) * ROWS_PER_WAVE;
+        const int32_t valid_rows = which < n_tiles ? p.n_rows - first_row : 0;
+        fetch_rows<T>(next_a, p.A + static_cast<size_t>(first_row) * p.nA, p.nA, valid_rows, lane);
+        fetch_rows<T>(next_b, p.B + static_cast<size_t>(first_row) * p.nB, p.nB, valid_rows, lane);
+        fetch_rows<T>(next_g, p.G + static_cast<size_t>(first_row) * p.nO, p.nO, valid_rows, lane);
+    };
+    fetch(tile);
+    const OperandTarget<T> targets[2] = {
+        {want_A ? operand_A : nullptr, p.first, {1, 2, 0}},
+        {want_B ? operand_B : nullptr, p.second, {0, 2, 1}},
+    };
+    build_operands<T, 2>(targets, areas, p.nA, p.nB, p.nO, entries); // ends with a barrier
+
+    const int i = lane & 15;
+    const int q = lane >> 4;
+    for (; tile < n_tiles; tile += stride) {
+        place_rows<T>(a_tile, next_a, ROWS_PER_WAVE * p.nA, lane);
+        place_rows<T>(b_tile, next_b, ROWS_PER_WAVE * p.nB, lane);
+        place_rows<T>(g_tile, next_g, ROWS_PER_WAVE * p.nO, lane);
+        wave_sync();
+        fetch(tile + stride);
+        T inner[ROW_TILES][GROUPS]; // grad_output[row][4 g + q]
+#pragma unroll
+        for (int r = 0; r < ROW_TILES; r++) {
+#pragma unroll
+            for (int g = 0; g < GROUPS; g++) {
+                const int32_t o = 4 * g + q;
+                inner[r][g] = load_or_zero(g_tile, (16 * r + i) * p.nO + o, o < p.nO);
+            }
+        }
+        typename M::Acc for_A[ROW_TILES][1], for_B[ROW_TILES][1];
+#pragma unroll
+        for (int r = 0; r < ROW_TILES; r++) {
+            for_A[r][0] = M::zero();
+            for_B[r][0] = M::zero();
+        }
+        if (want_A) {
+            pair_products<T, 1, GROUPS>(for_A, b_tile + i * p.nB, 16 * p.nB, p.nB, inner, operand_A, lane);
+        }
+        if (want_B) {
+            pair_products<T, 1, GROUPS>(for_B, a_tile + i * p.nA, 16 * p.nA, p.nA, inner, operand_B, lane);
+        }
+        wave_sync(); // the tiles have been read: their places become the staging areas of the stores
+        const int32_t first_row = tile * ROWS_PER_WAVE;
+        if (want_A) {
+            store_rows<T, 1>(p.grad_A + static_cast<size_t>(first_row) * p.nA, a_tile, for_A, p.nA, p.n_rows - first_row, lane);
+        }
+        if (want_B) {
+            store_rows<T, 1>(p.grad_B + static_cast<size_t>(first_row) * p.nB, b_tile, for_B, p.nB, p.n_rows - first_row, lane);
+        }
+        wave_sync();
+    }
+}
+
 size_t forward_lds(const Shape& s, size_t element_size) {
     const OperandShape first = operand_shape(s.nA, s.nB, s.nO);
     return align16(static_cast<size_t>(first.size()) * element_size) +
@@ -646,6 +831,32 @@ size_t vjp_lds(const Shape& s, size_t element_size, bool want_A, bool want_B) {
     return align16(static_cast<size_t>(size_A) * element_size) + align16(static_cast<size_t>(size_B) * element_size) +
            build_areas_bytes(s, element_size) +
            static_cast<size_t>(WAVES) * ROWS_PER_WAVE * (s.nA + s.nB + s.nO) * element_size;
+}
+
+size_t forward_walk_lds(const Shape& s, size_t element_size) {
+    return forward_lds(s, element_size) +
+           static_cast<size_t>(WALK_WAVES - WAVES) * ROWS_PER_WAVE * std::max(s.nA + s.nB, s.nO) * element_size;
+}
+
+size_t vjp_walk_lds(const Shape& s, size_t element_size, bool want_A, bool want_B) {
+    return vjp_lds(s, element_size, want_A, want_B) +
+           static_cast<size_t>(WALK_WAVES - WAVES) * ROWS_PER_WAVE * (s.nA + s.nB + s.nO) * element_size;
+}
+
+/// Workgroups of a walking launch: as many as the device holds at once (two
+/// per compute unit by their wavefronts, one when their LDS does not fit twice).
+unsigned walking_workgroups(size_t lds) {
+    const int64_t per_unit = 2 * lds <= 160 * 1024 ? 2 : 1;
+    return static_cast<unsigned>(per_unit * compute_units());
+}
+
+/// Whether a launch walks: four tiles or more for every wavefront (below that
+/// the builds that are saved do not make up for one wavefront doing all the
+/// work of a tile), rows that fit the registers of fetch_rows, LDS that fits.
+bool walks(const Shape& s, int32_t widest_row, size_t lds) {
+    const int64_t tiles = (static_cast<int64_t>(s.n_rows) + ROWS_PER_WAVE - 1) / ROWS_PER_WAVE;
+    return lds <= 160 * 1024 && ROWS_PER_WAVE * widest_row <= PREFETCH * WAVE &&
+           tiles >= 4 * static_cast<int64_t>(walking_workgroups(lds)) * WALK_WAVES;
 }
 
 template <typename T> Arguments<T> arguments(const T* A, const T* B, const Table& table, const Shape& s) {
@@ -720,11 +931,15 @@ void forward(T* output, const T* A, const T* B, const Table& table, const Shape&
     Arguments<T> p = arguments<T>(A, B, table, s);
     p.output = output;
     p.first = operand_shape(s.nA, s.nB, s.nO);
-    const unsigned grid = static_cast<unsigned>((s.n_rows + ROWS_PER_GROUP - 1) / ROWS_PER_GROUP);
-    const size_t lds = forward_lds(s, sizeof(T));
+    const size_t walk_lds = forward_walk_lds(s, sizeof(T));
+    const bool walk = walks(s, std::max(s.nA, s.nB), walk_lds);
+    const unsigned grid =
+        walk ? walking_workgroups(walk_lds) : static_cast<unsigned>((s.n_rows + ROWS_PER_GROUP - 1) / ROWS_PER_GROUP);
+    const size_t lds = walk ? walk_lds : forward_lds(s, sizeof(T));
     const LaunchEvents events = launch_events(stream);
     with_constants<4, 4>(p.first.n_tiles, p.first.n_groups, [&](auto tiles, auto groups) {
-        auto kernel = forward_kernel<T, decltype(tiles)::value, decltype(groups)::value>;
+        auto kernel = walk ? forward_walk_kernel<T, decltype(tiles)::value, decltype(groups)::value>
+                           : forward_kernel<T, decltype(tiles)::value, decltype(groups)::value>;
         allow_lds(kernel, lds);
         hipExtLaunchKernelGGL(kernel, dim3(grid), dim3(THREADS), lds, stream, events.start, events.stop, 0, p);
     });
@@ -742,11 +957,14 @@ void vjp(
     p.G = grad_output;
     p.first = operand_shape(s.nB, s.nO, s.nA);
     p.second = operand_shape(s.nA, s.nO, s.nB);
-    const unsigned grid = static_cast<unsigned>((s.n_rows + ROWS_PER_GROUP - 1) / ROWS_PER_GROUP);
-    const size_t lds = vjp_lds(s, sizeof(T), grad_A != nullptr, grad_B != nullptr);
+    const size_t walk_lds = vjp_walk_lds(s, sizeof(T), grad_A != nullptr, grad_B != nullptr);
+    const bool walk = walks(s, std::max(std::max(s.nA, s.nB), s.nO), walk_lds);
+    const unsigned grid =
+        walk ? walking_workgroups(walk_lds) : static_cast<unsigned>((s.n_rows + ROWS_PER_GROUP - 1) / ROWS_PER_GROUP);
+    const size_t lds = walk ? walk_lds : vjp_lds(s, sizeof(T), grad_A != nullptr, grad_B != nullptr);
     const LaunchEvents events = launch_events(stream);
     with_constants<1, 16>(1, p.first.n_groups, [&](auto, auto groups) {
-        auto kernel = vjp_kernel<T, decltype(groups)::value>;
+        auto kernel = walk ? vjp_walk_kernel<T, decltype(groups)::value> : vjp_kernel<T, decltype(groups)::value>;
         allow_lds(kernel, lds);
         hipExtLaunchKernelGGL(kernel, dim3(grid), dim3(THREADS), lds, stream, events.start, events.stop, 0, p);
     });

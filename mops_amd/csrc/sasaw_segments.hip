@@ -1372,23 +1372,6 @@ int32_t chunk_for(int32_t n_edges, int32_t column_tiles, int64_t resident_waves)
     return 64;
 }
 
-/// Compute units of the current device (asked for once per device).
-int32_t compute_units() {
-    static std::atomic<int> cached[64];
-    int device = 0;
-    MOPS_HIP_CHECK(hipGetDevice(&device));
-    if (device < 0 || device >= 64) {
-        return 256;
-    }
-    int count = cached[device].load(std::memory_order_relaxed);
-    if (count == 0) {
-        MOPS_HIP_CHECK(hipDeviceGetAttribute(&count, hipDeviceAttributeMultiprocessorCount, device));
-        count = std::max(count, 1);
-        cached[device].store(count, std::memory_order_relaxed);
-    }
-    return count;
-}
-
 template <typename T> void launch_contract(ContractArgs<T> args, hipStream_t stream) {
     const Contraction<T>& p = args.contraction;
     const size_t lds = table_lds(args.table, sizeof(T));
