@@ -64,8 +64,8 @@ MAIN_KERNELS = {
         "double": "sasaw_segments::contract_kernel<double, 9, true, 64>",
     },
     ("sasaw", "vjp"): {
-        "float": "sasaw_segments::gradients_kernel<float, 9, true, true>",
-        "double": "sasaw_segments::gradients_kernel<double, 9, true, true>",
+        "float": "sasaw_segments::gradients_kernel<float, 9, true, true, false>",
+        "double": "sasaw_segments::gradients_kernel<double, 9, true, true, false>",
     },
 }
 

@@ -292,7 +292,10 @@ void* scratch(size_t bytes) {
         if (capacity < (size_t(1) << 20)) {
             capacity = size_t(1) << 20;
         }
-        MOPS_HIP_CHECK(hipMalloc(&res.block, capacity));
+        constexpr size_t counter_bytes = SCRATCH_COUNTERS * sizeof(int32_t);
+        MOPS_HIP_CHECK(hipMalloc(&res.block, counter_bytes + capacity));
+        // (not in a captured graph: a stream that is being captured got its error above)
+        MOPS_HIP_CHECK(hipMemsetAsync(res.block, 0, counter_bytes, st.stream));
         res.capacity = capacity;
         res.device = device;
     } else if (res.block_stream != st.stream && res.last_use_recorded && !st.capturing) {
@@ -307,7 +310,15 @@ void* scratch(size_t bytes) {
     res.block_stream = st.stream;
     res.block_in_graph = res.block_in_graph || st.capturing;
     st.used_scratch = true;
-    return res.block;
+    return static_cast<char*>(res.block) + SCRATCH_COUNTERS * sizeof(int32_t);
+}
+
+int32_t* scratch_counters() {
+    auto& st = state();
+    if (!st.used_scratch || st.resources == nullptr || st.resources->block == nullptr) {
+        throw std::runtime_error("mops: scratch_counters() without scratch() in the same call");
+    }
+    return static_cast<int32_t*>(st.resources->block);
 }
 
 size_t scratch_capacity() {

@@ -48,6 +48,15 @@ void* scratch(size_t bytes);
 /// Bytes of the calling thread's scratch block (0: none yet).
 size_t scratch_capacity();
 
+/// Counters that come with the scratch block: SCRATCH_COUNTERS integers of 32
+/// bits in front of the memory scratch() returned (call it first, in the same
+/// call of the library). They are zero when the block is made, and every kernel
+/// that counts in them sets what it has used back to zero before it ends, so
+/// that the next launch finds zeros without a launch that clears them (also
+/// the next replay of a graph the launches were captured into).
+constexpr size_t SCRATCH_COUNTERS = size_t(1) << 18;
+int32_t* scratch_counters();
+
 /// A second stream of the calling thread, for a kernel of a call that does not
 /// depend on the call's other kernels and leaves room on the device beside
 /// them. Construction makes the side stream wait for everything enqueued on

@@ -756,9 +756,10 @@ void sparse_accumulation_scatter_add_with_weights_vjp(MOPS_SASAW_VJP_PARAMS(MOPS
         };
         const size_t bytes = sasaw_segments::vjp_workspace_bytes(shape, want_W);
         void* workspace = bytes > 0 ? scratch(bytes) : nullptr;
+        int32_t* counters = bytes > 0 ? scratch_counters() : nullptr;
         sasaw_segments::vjp<scalar_t>(
             grad_A.data, grad_B.data, grad_W.data, grad_output.data, A.data, B.data, C.data, W.data, indices,
-            shape, workspace, stream
+            shape, workspace, counters, true, stream
         );
         finish_call(operation);
         return;
@@ -907,7 +908,10 @@ void sasaw_vjp_no_alloc(
     };
     if (s.L > 0 && sasaw_segments::vjp_supported(shape, sizeof(float), want_W)) {
         // (the same kernels as the existing entry point takes for these shapes)
-        const size_t needed = sasaw_segments::vjp_workspace_bytes(shape, want_W);
+        // (the places of the senders' edges, then their counters; the array is shared with the
+        // kernels of other shapes, so the counters are cleared by a launch in front)
+        const size_t places = sasaw_segments::vjp_workspace_bytes(shape, want_W);
+        const size_t needed = places + sasaw_segments::vjp_counters(shape, want_W) * sizeof(int32_t);
         if (needed > NO_ALLOC_SCRATCH_BYTES) {
             throw std::runtime_error(
                 std::string(who) + "these shapes need " + std::to_string(needed) + " bytes of temporary memory, the "
@@ -916,9 +920,10 @@ void sasaw_vjp_no_alloc(
                 "mops_cuda_sparse_accumulation_scatter_add_with_weights_vjp_f32"
             );
         }
+        char* const array = static_cast<char*>(no_alloc_scratch_of_current_device());
         sasaw_segments::vjp<float>(
             grad_A.data, grad_B.data, grad_W.data, grad_output.data, A.data, B.data, C.data, W.data, indices, shape,
-            no_alloc_scratch_of_current_device(), current_stream()
+            array, reinterpret_cast<int32_t*>(array + places), false, current_stream()
         );
         finish_call(operation);
         return;

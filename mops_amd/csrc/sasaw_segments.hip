@@ -655,6 +655,35 @@ __device__ __forceinline__ bool sum_over_slots(
     return any;
 }
 
+/// The same from the node's places by arrival (SenderArrivals in
+/// sender_buckets.hpp): `count` edges name the node, in no order; `area` is
+/// this wavefront's SLOT_CAPACITY integers in LDS.
+template <typename Sum>
+__device__ __forceinline__ bool sum_over_arrivals(
+    Sum& sum, int32_t first_half, int32_t second_half, int32_t count, int32_t* area,
+    const int32_t* __restrict__ listed_index, int32_t node, int lane
+) {
+    if (count > SLOT_CAPACITY) {
+        // (more edges than places: the slots' way of saying so makes sum_over_slots read the index)
+        return sum_over_slots(sum, 0, 0, make_int4(SLOT_PART_CAPACITY + 1, 0, 0, 0), listed_index, node, lane);
+    }
+    const auto& p = sum.p;
+    sum.clear();
+    auto hand_on = [&](int32_t edges, int32_t n) {
+        const int32_t mine = lane < n ? edges : -1;
+        const int32_t sources = load_or_zero(p.gather_index, static_cast<size_t>(max(mine, 0)), mine >= 0);
+        sum.add(mine, mine >= 0 ? sources : -1, n);
+    };
+    if (count > 0) {
+        arrivals_in_order(first_half, second_half, count, area, lane);
+        hand_on(first_half, min(count, WAVE));
+    }
+    if (count > WAVE) {
+        hand_on(second_half, count - WAVE);
+    }
+    return count > 0;
+}
+
 template <typename T> struct ContractArgs {
     Contraction<T> contraction;
     Table table;
@@ -846,8 +875,11 @@ template <typename T> struct GradientArgs {
     int32_t n_W_units;    // n_nodes * column_tiles when grad_W is wanted; these units come last (measured: 6 to 10 us
                           // slower at 60 000 edges when they come first)
     int32_t n_units;      // the sum
+    // the senders' edges: in slots (sender_buckets.hpp: SenderSlots), or, `by_arrival`, as SenderArrivals
+    // with a counter for every (column tile, node), which the unit that reads it sets back to zero
     const int32_t* slot_edges;
-    const int32_t* slot_counts;
+    int32_t* slot_counts;
+    bool by_arrival;
 };
 
 template <typename T, int NB, bool EXACT, bool VECTORS> struct EdgeGradients {
@@ -1133,7 +1165,7 @@ template <typename T, int NB> constexpr int gradient_group_threads() {
 
 /// EXACT: n2 = n3 = NB, no row of a block is padding (otherwise the block rows are
 /// compared with n2 / n3 as the loops go).
-template <typename T, int NB, bool EXACT, bool VECTORS>
+template <typename T, int NB, bool EXACT, bool VECTORS, bool ARRIVALS>
 __global__ __launch_bounds__((gradient_group_threads<T, NB>())) void gradients_kernel(const GradientArgs<T> args) {
     constexpr int THREADS = gradient_group_threads<T, NB>();
     constexpr int GROUP_WAVES = THREADS / WAVE;
@@ -1151,6 +1183,7 @@ __global__ __launch_bounds__((gradient_group_threads<T, NB>())) void gradients_k
 
     const int lane = threadIdx.x & (WAVE - 1);
     const int32_t wave = threadIdx.x >> 6;
+    int32_t* const sorting_area = table_ready + 3 + wave * SLOT_CAPACITY; // (arrivals_in_order)
     const int32_t group = static_cast<int32_t>(blockIdx.x);
     const int32_t n_groups = static_cast<int32_t>(gridDim.x);
     const bool want_W = args.grad_W != nullptr, want_A = args.grad_A != nullptr, want_B = args.grad_B != nullptr;
@@ -1207,15 +1240,24 @@ __global__ __launch_bounds__((gradient_group_threads<T, NB>())) void gradients_k
             }
             ahead.v[5] = 0;
         } else {
-            const int32_t node = (unit - args.n_edge_units) / args.column_tiles;
+            const int32_t item = unit - args.n_edge_units;
+            const int32_t node = item / args.column_tiles;
             const int32_t* mine = args.slot_edges + static_cast<size_t>(node) * SLOT_CAPACITY;
             ahead.v[0] = mine[lane];
             ahead.v[1] = mine[lane + WAVE];
-            const int4 counts = reinterpret_cast<const int4*>(args.slot_counts)[node];
-            ahead.v[2] = counts.x;
-            ahead.v[3] = counts.y;
-            ahead.v[4] = counts.z;
-            ahead.v[5] = counts.w;
+            if constexpr (ARRIVALS) {
+                const int32_t tile = item - node * args.column_tiles;
+                ahead.v[2] = args.slot_counts[static_cast<size_t>(tile) * args.n_nodes + node];
+                ahead.v[3] = 0;
+                ahead.v[4] = 0;
+                ahead.v[5] = 0;
+            } else {
+                const int4 counts = reinterpret_cast<const int4*>(args.slot_counts)[node];
+                ahead.v[2] = counts.x;
+                ahead.v[3] = counts.y;
+                ahead.v[4] = counts.z;
+                ahead.v[5] = counts.w;
+            }
         }
     };
 
@@ -1290,9 +1332,21 @@ __global__ __launch_bounds__((gradient_group_threads<T, NB>())) void gradients_k
         } else {
             const int32_t item = unit - args.n_edge_units;
             const int32_t node = item / args.column_tiles;
-            sum.set_column_tile(item - node * args.column_tiles);
-            const int4 counts = make_int4(current.v[2], current.v[3], current.v[4], current.v[5]);
-            if (sum_over_slots(sum, current.v[0], current.v[1], counts, args.senders, node, lane)) {
+            const int32_t tile = item - node * args.column_tiles;
+            sum.set_column_tile(tile);
+            bool any;
+            if constexpr (ARRIVALS) {
+                const int32_t count = __builtin_amdgcn_readfirstlane(current.v[2]);
+                if (lane == 0) {
+                    // (nobody else reads this counter in this launch: zero again for the next one)
+                    args.slot_counts[static_cast<size_t>(tile) * args.n_nodes + node] = 0;
+                }
+                any = sum_over_arrivals(sum, current.v[0], current.v[1], count, sorting_area, args.senders, node, lane);
+            } else {
+                const int4 counts = make_int4(current.v[2], current.v[3], current.v[4], current.v[5]);
+                any = sum_over_slots(sum, current.v[0], current.v[1], counts, args.senders, node, lane);
+            }
+            if (any) {
                 wait_for(seen_W, 0);
                 sum.finish(table_W, args.table_W.registers, node);
             } else {
@@ -1463,6 +1517,15 @@ void forward(
 
 /// Whether the persistent gradient kernel serves this vjp: the senders' edges
 /// fit the slots on average (sparse graphs), which grad_W needs.
+/// Whether the senders' edges are listed by arrival (one look at every edge,
+/// an atomic for each) rather than in slots (every 16 senders look at the whole
+/// index): measured at 30 edges per node, 2000 nodes: 13.6 + 3 us (the
+/// consumers put the lists in order) against 8.5 us; 32 000 nodes: about 200
+/// against 457 us. The cost of the slots grows with edges x nodes.
+static bool lists_by_arrival(const Shape& s) {
+    return s.n_nodes > 6000 && static_cast<size_t>(s.n_nodes) * ((s.L + 15) / 16) <= SCRATCH_COUNTERS;
+}
+
 bool vjp_supported(const Shape& s, size_t element_size, bool want_grad_W) {
     if (!sasaw_segments::supports(s, element_size)) {
         return false;
@@ -1471,7 +1534,11 @@ bool vjp_supported(const Shape& s, size_t element_size, bool want_grad_W) {
 }
 
 size_t vjp_workspace_bytes(const Shape& s, bool want_grad_W) {
-    return want_grad_W ? sender_slots_bytes(s.n_nodes) : 0;
+    return want_grad_W ? sender_slots_bytes(s.n_nodes) : 0; // (enough for either way of listing)
+}
+
+size_t vjp_counters(const Shape& s, bool want_grad_W) {
+    return want_grad_W && lists_by_arrival(s) ? static_cast<size_t>(s.n_nodes) * ((s.L + 15) / 16) : 0;
 }
 
 /// Positions of the sorted index per unit of the per-edge gradients: the most
@@ -1493,7 +1560,8 @@ int32_t edge_chunk_for(int32_t n_edges, int32_t edge_roles, int64_t wanted_units
 template <typename T>
 void vjp(
     T* grad_A, T* grad_B, T* grad_W, const T* grad_output, const T* A, const T* B, const T* C, const T* W,
-    const Indices& indices, const Shape& s, void* workspace, hipStream_t stream
+    const Indices& indices, const Shape& s, void* workspace, int32_t* counters, bool counters_are_zero,
+    hipStream_t stream
 ) {
     GradientArgs<T> args{};
     args.A = A;
@@ -1515,9 +1583,21 @@ void vjp(
     args.column_tiles = (s.L + 15) / 16;
     if (grad_W != nullptr) {
         // the edges of every sender, listed by a launch of its own in front
-        const SenderSlots slots = list_edges_in_slots(indices.W_1, s.n_edges, s.n_nodes, workspace, stream);
-        args.slot_edges = slots.edges;
-        args.slot_counts = slots.counts;
+        args.by_arrival = lists_by_arrival(s);
+        if (args.by_arrival) {
+            if (!counters_are_zero) {
+                clear_counters(counters, vjp_counters(s, true), stream);
+            }
+            const SenderArrivals lists = list_edges_by_arrival(
+                indices.W_1, s.n_edges, s.n_nodes, args.column_tiles, workspace, counters, stream
+            );
+            args.slot_edges = lists.edges;
+            args.slot_counts = lists.counts;
+        } else {
+            const SenderSlots slots = list_edges_in_slots(indices.W_1, s.n_edges, s.n_nodes, workspace, stream);
+            args.slot_edges = slots.edges;
+            args.slot_counts = const_cast<int32_t*>(slots.counts);
+        }
     }
     args.edge_roles = (grad_A != nullptr ? 1 : 0) + (grad_B != nullptr ? args.column_tiles : 0);
     const int64_t W_units = grad_W != nullptr ? static_cast<int64_t>(s.n_nodes) * args.column_tiles : 0;
@@ -1537,8 +1617,10 @@ void vjp(
         args.table_beta.layout = Layout::BETA;
         args.table_beta.bucket = NB;
         const size_t slots = static_cast<size_t>(args.table_W.slots()) + args.table_alpha.slots() + args.table_beta.slots();
-        const size_t lds = slots * (sizeof(T) + sizeof(int32_t)) + 32;
         constexpr int GROUP_WAVES = gradient_group_threads<T, NB>() / WAVE;
+        // (the tables, a counter and three flags, every wavefront's area for putting a sender's edges in order)
+        const size_t lds = slots * (sizeof(T) + sizeof(int32_t)) + 32 +
+                           (args.by_arrival ? GROUP_WAVES * SLOT_CAPACITY * sizeof(int32_t) : 0);
         const int64_t resident_waves = static_cast<int64_t>(GROUP_WAVES) * compute_units();
         args.edge_chunk = edge_chunk_for(s.n_edges, args.edge_roles, resident_waves * sizeof(T) / 4);
         const int64_t chunks = (static_cast<int64_t>(s.n_edges) + args.edge_chunk - 1) / args.edge_chunk;
@@ -1549,7 +1631,9 @@ void vjp(
             static_cast<unsigned>(std::min<int64_t>(compute_units(), (units + GROUP_WAVES - 1) / GROUP_WAVES));
         (void)fits;
         auto launch = [&](auto exact, auto with_vectors) {
-            auto kernel = gradients_kernel<T, NB, decltype(exact)::value, decltype(with_vectors)::value>;
+            auto kernel = args.by_arrival
+                              ? gradients_kernel<T, NB, decltype(exact)::value, decltype(with_vectors)::value, true>
+                              : gradients_kernel<T, NB, decltype(exact)::value, decltype(with_vectors)::value, false>;
             allow_lds(kernel, lds);
             kernel<<<grid, gradient_group_threads<T, NB>(), lds, stream>>>(args);
         };
@@ -1575,11 +1659,11 @@ template void forward<double>(
 );
 template void vjp<float>(
     float*, float*, float*, const float*, const float*, const float*, const float*, const float*, const Indices&,
-    const Shape&, void*, hipStream_t
+    const Shape&, void*, int32_t*, bool, hipStream_t
 );
 template void vjp<double>(
     double*, double*, double*, const double*, const double*, const double*, const double*, const double*,
-    const Indices&, const Shape&, void*, hipStream_t
+    const Indices&, const Shape&, void*, int32_t*, bool, hipStream_t
 );
 
 } // namespace mops::amd::sasaw_segments

@@ -27,16 +27,22 @@ void forward(
 );
 
 /// Whether vjp() serves the shape (grad_W needs a sparse graph: at most 48
-/// edges per node on average), and the device scratch it needs. vjp() makes no
+/// edges per node on average), the device scratch it needs and the number of
+/// 32-bit counters (see SenderArrivals in sender_buckets.hpp). vjp() makes no
 /// allocation and uses no second stream.
 bool vjp_supported(const Shape& shape, size_t element_size, bool want_grad_W);
 size_t vjp_workspace_bytes(const Shape& shape, bool want_grad_W);
+size_t vjp_counters(const Shape& shape, bool want_grad_W);
 
-/// Any of grad_A, grad_B, grad_W may be null (not all).
+/// Any of grad_A, grad_B, grad_W may be null (not all). `counters`: the
+/// vjp_counters() counters; they are zero again when the kernels have run.
+/// `counters_are_zero`: whether they are zero now (otherwise a launch in front
+/// clears them).
 template <typename T>
 void vjp(
     T* grad_A, T* grad_B, T* grad_W, const T* grad_output, const T* A, const T* B, const T* C,
-    const T* W, const Indices& indices, const Shape& shape, void* workspace, hipStream_t stream
+    const T* W, const Indices& indices, const Shape& shape, void* workspace, int32_t* counters,
+    bool counters_are_zero, hipStream_t stream
 );
 
 } // namespace mops::amd::sasaw_segments

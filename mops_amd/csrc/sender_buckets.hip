@@ -264,6 +264,25 @@ __global__ __launch_bounds__(SLOT_THREADS) void list_in_slots_kernel(
     list_in_slots_block<SLOT_THREADS>(lists, slots, counts, senders, n_edges, n_nodes, aligned, blockIdx.x);
 }
 
+// Sparse graphs, by arrival: one thread per edge.
+constexpr int ARRIVAL_THREADS = 4 * WAVE;
+
+__global__ __launch_bounds__(ARRIVAL_THREADS) void list_by_arrival_kernel(
+    const SenderArrivals lists, const int32_t* __restrict__ senders, int32_t n_edges, int32_t n_nodes
+) {
+    const int32_t edge = static_cast<int32_t>(blockIdx.x) * ARRIVAL_THREADS + static_cast<int32_t>(threadIdx.x);
+    if (edge < n_edges) {
+        list_arrival(lists, n_nodes, senders[edge], edge);
+    }
+}
+
+__global__ __launch_bounds__(ARRIVAL_THREADS) void clear_counters_kernel(int32_t* __restrict__ counters, size_t count) {
+    const size_t at = static_cast<size_t>(blockIdx.x) * ARRIVAL_THREADS + threadIdx.x;
+    if (at < count) {
+        counters[at] = 0;
+    }
+}
+
 } // namespace
 
 size_t sender_slots_bytes(int32_t n_nodes) {
@@ -295,6 +314,27 @@ SenderSlots list_edges_in_slots(
         MOPS_HIP_CHECK(hipGetLastError());
     }
     return slots;
+}
+
+SenderArrivals list_edges_by_arrival(
+    const int32_t* senders, int32_t n_edges, int32_t n_nodes, int32_t copies, void* workspace, int32_t* counts,
+    hipStream_t stream
+) {
+    const SenderArrivals lists{static_cast<int32_t*>(workspace), counts, copies};
+    if (n_nodes > 0 && n_edges > 0) {
+        const unsigned blocks = static_cast<unsigned>(ceil_div(static_cast<size_t>(n_edges), ARRIVAL_THREADS));
+        list_by_arrival_kernel<<<blocks, ARRIVAL_THREADS, 0, stream>>>(lists, senders, n_edges, n_nodes);
+        MOPS_HIP_CHECK(hipGetLastError());
+    }
+    return lists;
+}
+
+void clear_counters(int32_t* counters, size_t count, hipStream_t stream) {
+    if (count > 0) {
+        const unsigned blocks = static_cast<unsigned>(ceil_div(count, ARRIVAL_THREADS));
+        clear_counters_kernel<<<blocks, ARRIVAL_THREADS, 0, stream>>>(counters, count);
+        MOPS_HIP_CHECK(hipGetLastError());
+    }
 }
 
 size_t edges_by_sender_bytes(int32_t n_nodes, int32_t n_edges) {

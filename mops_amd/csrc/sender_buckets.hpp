@@ -11,12 +11,14 @@
 #ifndef MOPS_AMD_SENDER_BUCKETS_HPP
 #define MOPS_AMD_SENDER_BUCKETS_HPP
 
+#include <climits>
 #include <cstddef>
 #include <cstdint>
 
 #include <hip/hip_runtime.h>
 
 #include "device_common.hpp"
+#include "runtime.hpp"
 
 namespace mops::amd {
 
@@ -229,6 +231,101 @@ __device__ __forceinline__ void list_in_slots_block(
             counts[static_cast<size_t>(node0 + which) * SLOT_PARTS + part] = n;
         }
     }
+}
+
+/// Sparse graphs, with ONE look at every edge: a sender owns SLOT_CAPACITY
+/// places and a counter in global memory, and an edge takes the next place of
+/// its sender (an integer atomic that returns the count before it). The places
+/// of a sender then hold its edges in the order of arrival, which whoever uses
+/// them puts right first (arrivals_in_order). No workgroup reads more of the
+/// index than its own share: 4 bytes per edge instead of 4 bytes per edge and
+/// 16 senders.
+///
+/// The counters have to be zero before the listing. Every counter is read by
+/// exactly one wavefront of the consuming launch, which sets it back to zero:
+/// nothing has to be cleared between calls (or between replays of a graph).
+/// A consuming launch in which `copies` wavefronts want the list of the same
+/// sender gets `copies` counters per sender, all of which count every edge.
+struct SenderArrivals {
+    /// [n_nodes][SLOT_CAPACITY] edges that name the node, in the order of arrival
+    int32_t* edges;
+    /// [copies][n_nodes] number of edges that name the node (may exceed
+    /// SLOT_CAPACITY: the consumer then has to find the node's edges itself)
+    int32_t* counts;
+    int32_t copies;
+};
+
+/// Bytes of scratch memory the places take (the counters are elsewhere).
+inline size_t sender_arrivals_bytes(int32_t n_nodes) {
+    return align256(static_cast<size_t>(n_nodes) * SLOT_CAPACITY * 4);
+}
+
+/// Edge `edge` names `sender`: called by one thread per edge.
+__device__ __forceinline__ void list_arrival(
+    const SenderArrivals& lists, int32_t n_nodes, int32_t sender, int32_t edge
+) {
+    if (in_bounds(sender, n_nodes)) {
+        const int32_t place = atomicAdd(&lists.counts[sender], 1);
+        for (int32_t c = 1; c < lists.copies; c++) {
+            atomicAdd(&lists.counts[static_cast<size_t>(c) * n_nodes + sender], 1);
+        }
+        if (place < SLOT_CAPACITY) {
+            lists.edges[static_cast<size_t>(sender) * SLOT_CAPACITY + place] = edge;
+        }
+    }
+}
+
+/// Enqueue the kernel that lists the edges of every sender by arrival (values
+/// outside [0, n_nodes) are dropped). `counts`: copies x n_nodes counters, zero.
+SenderArrivals list_edges_by_arrival(
+    const int32_t* senders, int32_t n_edges, int32_t n_nodes, int32_t copies, void* workspace, int32_t* counts,
+    hipStream_t stream
+);
+
+/// Enqueue a kernel that sets `count` counters to zero (for counters whose
+/// earlier contents are not known).
+void clear_counters(int32_t* counters, size_t count, hipStream_t stream);
+
+/// A sender's `count` <= SLOT_CAPACITY places (lane k holds places k and
+/// k + 64 in `first_half`, `second_half`) in ascending order: lane k gets
+/// entries k and k + 64 of the sorted list. Edge numbers are distinct, so the
+/// rank of one is the number of smaller ones. `area`: SLOT_CAPACITY integers in
+/// LDS for this wavefront alone (used for lists of more than 64 edges).
+__device__ __forceinline__ void arrivals_in_order(
+    int32_t& first_half, int32_t& second_half, int32_t count, int32_t* area, int lane
+) {
+    const int32_t mine0 = lane < count ? first_half : INT32_MAX;
+    const int32_t mine1 = lane + WAVE < count ? second_half : INT32_MAX;
+    int32_t rank0 = 0, rank1 = 0;
+    if (count <= WAVE) {
+        for (int32_t k = 0; k < count; k++) {
+            rank0 += __builtin_amdgcn_readlane(mine0, k) < mine0 ? 1 : 0;
+        }
+        // (lanes without an edge send to themselves)
+        first_half = __builtin_amdgcn_ds_permute((lane < count ? rank0 : lane) << 2, mine0);
+        second_half = mine1;
+        return;
+    }
+    for (int32_t k = 0; k < WAVE; k++) {
+        const int32_t other = __builtin_amdgcn_readlane(mine0, k);
+        rank0 += other < mine0 ? 1 : 0;
+        rank1 += other < mine1 ? 1 : 0;
+    }
+    for (int32_t k = 0; k < count - WAVE; k++) {
+        const int32_t other = __builtin_amdgcn_readlane(mine1, k);
+        rank0 += other < mine0 ? 1 : 0;
+        rank1 += other < mine1 ? 1 : 0;
+    }
+    area[rank0] = mine0;
+    area[lane + WAVE < count ? rank1 : lane + WAVE] = mine1;
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    first_half = area[lane];
+    second_half = area[lane + WAVE];
+    // (the next list of this wavefront is written after these reads)
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
 }
 
 /// Capacity (in edges) of the LDS array passed to sorted_bucket.

@@ -82,6 +82,11 @@ CASES = {
             support.sasaw_case(s, d, E=6000, nA=4, L=8, n_nodes=300, n2=3, n3=5, N=40, allow_empty=True),
             "indices_W_1", SENDER_COUNTS
         ),
+        # (more than 6000 nodes: the senders' edges are listed in the order of arrival and sorted by their users)
+        "many_nodes_with_hubs": lambda s, d: _with_sender_counts(
+            support.sasaw_case(s, d, E=70000, nA=4, L=24, n_nodes=6500, n2=3, n3=5, N=40, allow_empty=True),
+            "indices_W_1", SENDER_COUNTS
+        ),
         "forty_five_per_sender": lambda s, d: support.sasaw_case(s, d, E=2250, nA=4, L=16, n_nodes=50, n2=4, n3=3, N=30),
         "many_columns": lambda s, d: support.sasaw_case(s, d, E=500, nA=9, L=128, n_nodes=21, n2=9, n3=9, N=120, allow_empty=True),
         "ragged_columns": lambda s, d: support.sasaw_case(s, d, E=400, nA=4, L=70, n_nodes=17, n2=6, n3=11, N=80, allow_empty=True),
