@@ -310,9 +310,11 @@ def measured_traffic(kernel_prefix):
             lines = handle.read().split("\n")
     except OSError:
         return None
+    # (the summary cuts long names: compare without the closing bracket of the template list)
+    prefix = kernel_prefix[:95].rstrip(">")
     for line in lines:
-        if line.startswith(kernel_prefix[:95]):
-            columns = re.findall(r"[-+]?\d+\.\d+", line[len(kernel_prefix[:95]):])
+        if line.startswith(prefix):
+            columns = re.findall(r"[-+]?\d+\.\d+", line[len(prefix):])
             if len(columns) >= 5:
                 return int(round(float(columns[-1]) * 1e6))
     return None
