@@ -108,6 +108,8 @@ LARGE = {
     },
     "sap": {
         "many_rows": lambda s, d: support.sap_case(s, d, I=1000003, nA=13, nB=7, K=900, nO=20),
+        # (enough rows for the forward kernel whose wavefronts walk over tiles, too few for the vjp's in float32)
+        "rows_between": lambda s, d: support.sap_case(s, d, I=150001, nA=13, nB=7, K=900, nO=20),
         "long_table": lambda s, d: support.sap_case(s, d, I=20000, nA=16, nB=16, K=6000, nO=30),
         "big_table_dimensions": lambda s, d: support.sap_case(s, d, I=5000, nA=40, nB=30, K=3000, nO=50),
         "tiles_beyond_64k": lambda s, d: support.sap_case(s, d, I=2000, nA=40, nB=40, K=3000, nO=60),
