@@ -78,6 +78,27 @@ def test_two_calls_in_a_row_the_second_smaller(oracle, device):
             assert torch.equal(got[name], want[name]), (wanted, name)
 
 
+def test_more_than_6000_nodes(oracle, device):
+    """Graphs of this size list the senders' edges by arrival, on counters that have to start at
+    zero: here they lie in the built-in array, behind whatever an earlier call left there."""
+    import torch
+
+    from mops_amd._c_lib import device_library
+
+    library = device_library()
+    support._bind_stream(library, device)
+    host_case = support.sasaw_case(44, np.float32, E=40000, nA=4, L=20, n_nodes=7000, n2=3, n3=4, N=30, allow_empty=True)
+    case = support.to_device(host_case, device)
+    expected = support.cpu_vjp(oracle, "sasaw", host_case)
+    for number in range(2):
+        print(f"no-alloc call {number} with 7000 nodes", flush=True)
+        got = gradients_of(library, case, "no_alloc")
+        want = gradients_of(library, case, "existing")
+        for name in ("A", "B", "W"):
+            assert torch.equal(got[name], want[name]), (number, name)
+            support.assert_close(got[name].cpu().numpy(), expected[name], np.float32, f"call {number} grad_{name}")
+
+
 def test_shapes_beyond_the_built_in_array_are_refused(device):
     import torch
 
