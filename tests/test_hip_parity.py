@@ -265,6 +265,21 @@ def test_vjp_subsets_of_gradients(oracle, device, op):
                     assert partial[key] is None
 
 
+@pytest.mark.parametrize("dtype", DTYPES, ids=["f32", "f64"])
+def test_sap_many_rows_subsets_of_gradients(device, dtype):
+    """The same for the SAP kernels whose wavefronts walk over the rows (300 000 rows and more)."""
+    case = support.sap_case(305, dtype, I=300011, nA=13, nB=7, K=900, nO=20)
+    on_device = to_device(case, device)
+    full = hip_vjp("sap", on_device)
+    for wanted in (["A"], ["B"]):
+        partial = hip_vjp("sap", on_device, wanted=wanted)
+        for key in ("A", "B"):
+            if key in wanted:
+                assert np.array_equal(partial[key].cpu().numpy(), full[key].cpu().numpy()), (wanted, key)
+            else:
+                assert partial[key] is None
+
+
 @pytest.mark.parametrize("op", ["opsa", "opsaw", "sasaw"])
 def test_rows_without_edges_are_exactly_zero(device, op):
     case = CASES[op]["ragged"](404, np.float32)
