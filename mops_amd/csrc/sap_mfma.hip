@@ -641,38 +641,44 @@ __global__ __launch_bounds__(THREADS) void vjp_kernel(const Arguments<T> p) {
 constexpr int WALK_WAVES = 16;                  // wavefronts per workgroup
 constexpr int WALK_THREADS = WALK_WAVES * WAVE; // (= THREADS: build_operands counts on it)
 static_assert(WALK_THREADS == THREADS, "the table build is written for THREADS threads");
-constexpr int PREFETCH = 8; // loads per lane and tensor: tiles of up to 512 values, rows of up to 32
-
 __device__ __forceinline__ void wave_sync() {
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
-/// The `valid_rows` x `width` values from `global` on (at most PREFETCH * 64), zeros after them.
-template <typename T>
+/// The `valid_rows` x `width` values from `global` on (at most N * 64: N loads per lane); after them
+/// comes a repeat of the first value, which the rows of a tile that do not exist may hold: every row
+/// of the results depends on its own row of the operands only, and rows that do not exist are not
+/// stored. (No zero is put in their place: a choice that follows a load is a wait for that load
+/// wherever the compiler moves it, and it moved all of them to the end of the loop, behind the
+/// loads of the tile after the next.)
+template <typename T, int N>
 __device__ __forceinline__ void fetch_rows(
-    T (&values)[PREFETCH], const T* __restrict__ global, int32_t width, int32_t valid_rows, int lane
+    T (&values)[N], const T* __restrict__ global, int32_t width, int32_t valid_rows, int lane
 ) {
     const int32_t valid = max(min(valid_rows, ROWS_PER_WAVE), 0) * width;
-    // (no branch around a load, not even a uniform one: every load would wait for the one before)
+    // (no branch around a load either, not even a uniform one: every load would wait for the one before)
 #pragma unroll
-    for (int u = 0; u < PREFETCH; u++) {
+    for (int u = 0; u < N; u++) {
         const int32_t at = u * WAVE + lane;
-        values[u] = load_or_zero(global, at, at < valid);
+        values[u] = global[at < valid ? at : 0];
     }
 }
 
-template <typename T>
-__device__ __forceinline__ void place_rows(T* __restrict__ lds, const T (&values)[PREFETCH], int32_t total, int lane) {
+template <typename T, int N>
+__device__ __forceinline__ void place_rows(T* __restrict__ lds, const T (&values)[N], int32_t total, int lane) {
 #pragma unroll
-    for (int u = 0; u < PREFETCH; u++) {
+    for (int u = 0; u < N; u++) {
         const int32_t at = u * WAVE + lane;
         if (at < total) {
             lds[at] = values[u];
         }
     }
 }
+
+/// Loads per lane for a tile of 16 rows of up to 16 values (A and B of the vjp, A of the forward pass).
+constexpr int SHORT_ROW_LOADS = 4;
 
 template <typename T, int NT, int GROUPS>
 __global__ __launch_bounds__(WALK_THREADS) void forward_walk_kernel(const Arguments<T> p) {
@@ -693,24 +699,30 @@ __global__ __launch_bounds__(WALK_THREADS) void forward_walk_kernel(const Argume
     const int32_t n_tiles = (p.n_rows + ROWS_PER_WAVE - 1) / ROWS_PER_WAVE;
     const int32_t stride = static_cast<int32_t>(gridDim.x) * WALK_WAVES;
     int32_t tile = static_cast<int32_t>(blockIdx.x) * WALK_WAVES + wave;
-    T next_a[PREFETCH], next_b[PREFETCH];
-    auto fetch = [&](int32_t which) {
+    // the rows of the next two tiles of this wavefront are on their way while it works on one
+    struct Rows {
+        T a[SHORT_ROW_LOADS];
+        T b[GROUPS];
+    };
+    auto fetch = [&](Rows& rows, int32_t which) {
         const int32_t first_row = min(which, n_tiles - 1) * ROWS_PER_WAVE; // (beyond the end: a tile that exists, no rows of it)
         const int32_t valid_rows = which < n_tiles ? p.n_rows - first_row : 0;
-        fetch_rows<T>(next_a, p.A + static_cast<size_t>(first_row) * p.nA, p.nA, valid_rows, lane);
-        fetch_rows<T>(next_b, p.B + static_cast<size_t>(first_row) * p.nB, p.nB, valid_rows, lane);
+        fetch_rows<T, SHORT_ROW_LOADS>(rows.a, p.A + static_cast<size_t>(first_row) * p.nA, p.nA, valid_rows, lane);
+        fetch_rows<T, GROUPS>(rows.b, p.B + static_cast<size_t>(first_row) * p.nB, p.nB, valid_rows, lane);
     };
-    fetch(tile);
+    Rows even, odd;
+    fetch(even, tile);
+    fetch(odd, tile + stride);
     const OperandTarget<T> targets[1] = {{operand, p.first, {0, 1, 2}}};
     build_operands<T, 1>(targets, areas, p.nA, p.nB, p.nO, entries); // ends with a barrier
 
     const int i = lane & 15;
     const int q = lane >> 4;
-    for (; tile < n_tiles; tile += stride) {
-        place_rows<T>(a_tile, next_a, ROWS_PER_WAVE * p.nA, lane);
-        place_rows<T>(b_tile, next_b, ROWS_PER_WAVE * p.nB, lane);
+    auto work = [&](Rows& rows) {
+        place_rows<T, SHORT_ROW_LOADS>(a_tile, rows.a, ROWS_PER_WAVE * p.nA, lane);
+        place_rows<T, GROUPS>(b_tile, rows.b, ROWS_PER_WAVE * p.nB, lane);
         wave_sync();
-        fetch(tile + stride);
+        fetch(rows, tile + 2 * stride);
         T inner[ROW_TILES][GROUPS];
 #pragma unroll
         for (int r = 0; r < ROW_TILES; r++) {
@@ -733,6 +745,14 @@ __global__ __launch_bounds__(WALK_THREADS) void forward_walk_kernel(const Argume
         const int32_t first_row = tile * ROWS_PER_WAVE;
         store_rows<T, NT>(p.output + static_cast<size_t>(first_row) * p.nO, mine, acc, p.nO, p.n_rows - first_row, lane);
         wave_sync();
+        tile += stride;
+    };
+    while (tile < n_tiles) {
+        work(even);
+        if (tile >= n_tiles) {
+            break;
+        }
+        work(odd);
     }
 }
 
@@ -760,15 +780,22 @@ __global__ __launch_bounds__(WALK_THREADS) void vjp_walk_kernel(const Arguments<
     const int32_t n_tiles = (p.n_rows + ROWS_PER_WAVE - 1) / ROWS_PER_WAVE;
     const int32_t stride = static_cast<int32_t>(gridDim.x) * WALK_WAVES;
     int32_t tile = static_cast<int32_t>(blockIdx.x) * WALK_WAVES + wave;
-    T next_a[PREFETCH], next_b[PREFETCH], next_g[PREFETCH];
-    auto fetch = [&](int32_t which) {
+    // the rows of the next two tiles of this wavefront are on their way while it works on one
+    struct Rows {
+        T a[SHORT_ROW_LOADS];
+        T b[SHORT_ROW_LOADS];
+        T g[GROUPS];
+    };
+    auto fetch = [&](Rows& rows, int32_t which) {
         const int32_t first_row = min(which, n_tiles - 1) * ROWS_PER_WAVE;
         const int32_t valid_rows = which < n_tiles ? p.n_rows - first_row : 0;
-        fetch_rows<T>(next_a, p.A + static_cast<size_t>(first_row) * p.nA, p.nA, valid_rows, lane);
-        fetch_rows<T>(next_b, p.B + static_cast<size_t>(first_row) * p.nB, p.nB, valid_rows, lane);
-        fetch_rows<T>(next_g, p.G + static_cast<size_t>(first_row) * p.nO, p.nO, valid_rows, lane);
+        fetch_rows<T, SHORT_ROW_LOADS>(rows.a, p.A + static_cast<size_t>(first_row) * p.nA, p.nA, valid_rows, lane);
+        fetch_rows<T, SHORT_ROW_LOADS>(rows.b, p.B + static_cast<size_t>(first_row) * p.nB, p.nB, valid_rows, lane);
+        fetch_rows<T, GROUPS>(rows.g, p.G + static_cast<size_t>(first_row) * p.nO, p.nO, valid_rows, lane);
     };
-    fetch(tile);
+    Rows even, odd;
+    fetch(even, tile);
+    fetch(odd, tile + stride);
     const OperandTarget<T> targets[2] = {
         {want_A ? operand_A : nullptr, p.first, {1, 2, 0}},
         {want_B ? operand_B : nullptr, p.second, {0, 2, 1}},
@@ -777,12 +804,12 @@ __global__ __launch_bounds__(WALK_THREADS) void vjp_walk_kernel(const Arguments<
 
     const int i = lane & 15;
     const int q = lane >> 4;
-    for (; tile < n_tiles; tile += stride) {
-        place_rows<T>(a_tile, next_a, ROWS_PER_WAVE * p.nA, lane);
-        place_rows<T>(b_tile, next_b, ROWS_PER_WAVE * p.nB, lane);
-        place_rows<T>(g_tile, next_g, ROWS_PER_WAVE * p.nO, lane);
+    auto work = [&](Rows& rows) {
+        place_rows<T, SHORT_ROW_LOADS>(a_tile, rows.a, ROWS_PER_WAVE * p.nA, lane);
+        place_rows<T, SHORT_ROW_LOADS>(b_tile, rows.b, ROWS_PER_WAVE * p.nB, lane);
+        place_rows<T, GROUPS>(g_tile, rows.g, ROWS_PER_WAVE * p.nO, lane);
         wave_sync();
-        fetch(tile + stride);
+        fetch(rows, tile + 2 * stride);
         T inner[ROW_TILES][GROUPS]; // grad_output[row][4 g + q]
 #pragma unroll
         for (int r = 0; r < ROW_TILES; r++) {
@@ -813,6 +840,14 @@ __global__ __launch_bounds__(WALK_THREADS) void vjp_walk_kernel(const Arguments<
             store_rows<T, 1>(p.grad_B + static_cast<size_t>(first_row) * p.nB, b_tile, for_B, p.nB, p.n_rows - first_row, lane);
         }
         wave_sync();
+        tile += stride;
+    };
+    while (tile < n_tiles) {
+        work(even);
+        if (tile >= n_tiles) {
+            break;
+        }
+        work(odd);
     }
 }
 
@@ -852,14 +887,14 @@ unsigned walking_workgroups(size_t lds) {
 
 /// Whether a launch walks: `tiles_per_wave` tiles or more for every wavefront
 /// (below that the builds that are saved do not make up for one wavefront doing
-/// all the work of a tile), rows that fit the registers of fetch_rows, LDS that
-/// fits. Measured with nA, nB, nO = 13, 7, 20 over 65 000 to 560 000 rows: the
+/// all the work of a tile), rows of A (and of B in the vjp) that fit the registers
+/// of fetch_rows (the others fit by the limits of these kernels), LDS that fits. Measured with nA, nB, nO = 13, 7, 20 over 65 000 to 560 000 rows: the
 /// forward pass gains from one tile per wavefront on (200 000 rows, f32: 33.3
 /// -> 30.0 us; f64 at 100 000: 30.0 -> 25.9), the vjp from two (400 000 rows,
 /// f32: 88.9 -> 83.5 us; with one, 140 000 rows take 41.4 instead of 35.9 us).
-bool walks(const Shape& s, int32_t widest_row, size_t lds, int64_t tiles_per_wave) {
+bool walks(const Shape& s, int32_t widest_short_row, size_t lds, int64_t tiles_per_wave) {
     const int64_t tiles = (static_cast<int64_t>(s.n_rows) + ROWS_PER_WAVE - 1) / ROWS_PER_WAVE;
-    return lds <= 160 * 1024 && ROWS_PER_WAVE * widest_row <= PREFETCH * WAVE &&
+    return lds <= 160 * 1024 && ROWS_PER_WAVE * widest_short_row <= SHORT_ROW_LOADS * WAVE &&
            tiles >= tiles_per_wave * static_cast<int64_t>(walking_workgroups(lds)) * WALK_WAVES;
 }
 
@@ -936,7 +971,7 @@ void forward(T* output, const T* A, const T* B, const Table& table, const Shape&
     p.output = output;
     p.first = operand_shape(s.nA, s.nB, s.nO);
     const size_t walk_lds = forward_walk_lds(s, sizeof(T));
-    const bool walk = walks(s, std::max(s.nA, s.nB), walk_lds, 1);
+    const bool walk = walks(s, s.nA, walk_lds, 1);
     const unsigned grid =
         walk ? walking_workgroups(walk_lds) : static_cast<unsigned>((s.n_rows + ROWS_PER_GROUP - 1) / ROWS_PER_GROUP);
     const size_t lds = walk ? walk_lds : forward_lds(s, sizeof(T));
@@ -962,7 +997,7 @@ void vjp(
     p.first = operand_shape(s.nB, s.nO, s.nA);
     p.second = operand_shape(s.nA, s.nO, s.nB);
     const size_t walk_lds = vjp_walk_lds(s, sizeof(T), grad_A != nullptr, grad_B != nullptr);
-    const bool walk = walks(s, std::max(std::max(s.nA, s.nB), s.nO), walk_lds, 2);
+    const bool walk = walks(s, std::max(s.nA, s.nB), walk_lds, 2);
     const unsigned grid =
         walk ? walking_workgroups(walk_lds) : static_cast<unsigned>((s.n_rows + ROWS_PER_GROUP - 1) / ROWS_PER_GROUP);
     const size_t lds = walk ? walk_lds : vjp_lds(s, sizeof(T), grad_A != nullptr, grad_B != nullptr);
