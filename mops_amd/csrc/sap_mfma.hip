@@ -447,6 +447,56 @@ __device__ __forceinline__ void store_rows(
     }
 }
 
+/// store_rows for the walking kernels: always the same number of store instructions, each a buffer
+/// store whose descriptor ends with the rows that exist (the hardware drops what lies beyond), so
+/// that a later wait for loads that were asked for before these stores can leave exactly them in
+/// flight. With stores under a condition the compiler does not know how many there are and such a
+/// wait ends up waiting for younger loads as well.
+template <typename T, int NT>
+__device__ __forceinline__ void store_rows_counted(
+    T* __restrict__ global, T* __restrict__ lds, const typename Mfma<T>::Acc (&acc)[ROW_TILES][NT],
+    int32_t width, int32_t valid_rows, int lane
+) {
+    using M = Mfma<T>;
+    const int j = lane & 15;
+#pragma unroll
+    for (int r = 0; r < ROW_TILES; r++) {
+#pragma unroll
+        for (int t = 0; t < NT; t++) {
+            const int32_t column = 16 * t + j;
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                if (column < width) {
+                    lds[(16 * r + M::row(lane, e)) * width + column] = acc[r][t][e];
+                }
+            }
+        }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    // (uniform, and said to be: a descriptor that the compiler takes for different from lane to
+    // lane costs a loop around every store)
+    const int32_t total = __builtin_amdgcn_readfirstlane(max(min(valid_rows, ROWS_PER_WAVE), 0) * width);
+    const __amdgpu_buffer_rsrc_t target = __builtin_amdgcn_make_buffer_rsrc(
+        global, 0, total * static_cast<int32_t>(sizeof(T)), 0x00020000
+    );
+    // (ROW_TILES * NT * 4 stores cover 16 rows of up to 16 NT values; the LDS reads stay inside
+    // the wavefront's own area, which holds 16 rows of the widest of its tensors)
+    const int32_t area = ROWS_PER_WAVE * width;
+#pragma unroll
+    for (int u = 0; u < ROW_TILES * NT * 4; u++) {
+        const int32_t at = u * WAVE + lane;
+        const T value = lds[min(at, area - 1)];
+        if constexpr (sizeof(T) == 4) {
+            __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, value), target, at * 4, 0, 0);
+        } else {
+            typedef unsigned int two_words __attribute__((__vector_size__(2 * sizeof(unsigned int))));
+            __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(two_words, value), target, at * 8, 0, 0);
+        }
+    }
+}
+
 template <typename T> struct Arguments {
     T* output;  // forward: O; vjp: unused
     T* grad_A;  // vjp, may be null
@@ -742,8 +792,9 @@ __global__ __launch_bounds__(WALK_THREADS) void forward_walk_kernel(const Argume
         }
         pair_products<T, NT, GROUPS>(acc, a_tile + i * p.nA, 16 * p.nA, p.nA, inner, operand, lane);
         wave_sync(); // the tile has been read: its place becomes the staging area of the store
-        const int32_t first_row = tile * ROWS_PER_WAVE;
-        store_rows<T, NT>(p.output + static_cast<size_t>(first_row) * p.nO, mine, acc, p.nO, p.n_rows - first_row, lane);
+        // (the same in all lanes, which the compiler cannot know: a wavefront's number comes from threadIdx)
+        const int32_t first_row = __builtin_amdgcn_readfirstlane(tile) * ROWS_PER_WAVE;
+        store_rows_counted<T, NT>(p.output + static_cast<size_t>(first_row) * p.nO, mine, acc, p.nO, p.n_rows - first_row, lane);
         wave_sync();
         tile += stride;
     };
@@ -832,12 +883,12 @@ __global__ __launch_bounds__(WALK_THREADS) void vjp_walk_kernel(const Arguments<
             pair_products<T, 1, GROUPS>(for_B, a_tile + i * p.nA, 16 * p.nA, p.nA, inner, operand_B, lane);
         }
         wave_sync(); // the tiles have been read: their places become the staging areas of the stores
-        const int32_t first_row = tile * ROWS_PER_WAVE;
+        const int32_t first_row = __builtin_amdgcn_readfirstlane(tile) * ROWS_PER_WAVE; // (the same in all lanes)
         if (want_A) {
-            store_rows<T, 1>(p.grad_A + static_cast<size_t>(first_row) * p.nA, a_tile, for_A, p.nA, p.n_rows - first_row, lane);
+            store_rows_counted<T, 1>(p.grad_A + static_cast<size_t>(first_row) * p.nA, a_tile, for_A, p.nA, p.n_rows - first_row, lane);
         }
         if (want_B) {
-            store_rows<T, 1>(p.grad_B + static_cast<size_t>(first_row) * p.nB, b_tile, for_B, p.nB, p.n_rows - first_row, lane);
+            store_rows_counted<T, 1>(p.grad_B + static_cast<size_t>(first_row) * p.nB, b_tile, for_B, p.nB, p.n_rows - first_row, lane);
         }
         wave_sync();
         tile += stride;
