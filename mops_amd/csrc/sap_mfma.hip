@@ -24,6 +24,13 @@
 // Every workgroup builds the reshaped M it needs in LDS from the raw table
 // (build_operand): no second kernel, no table in global memory, and the same
 // bits in every workgroup and on every run.
+//
+// Two sets of kernels. forward_kernel / vjp_kernel: a workgroup for every 128
+// rows, two wavefronts per tile of 16 rows; what launches of up to a few
+// tiles per wavefront of the device take. forward_walk_kernel /
+// vjp_walk_kernel: as many workgroups as the device holds, each builds M once
+// and its wavefronts then walk over tiles of their own; what launches of
+// hundreds of thousands of rows take (walks() has the measured thresholds).
 #include "sap_mfma.hpp"
 
 #include <algorithm>
