@@ -1519,11 +1519,12 @@ void forward(
 /// fit the slots on average (sparse graphs), which grad_W needs.
 /// Whether the senders' edges are listed by arrival (one look at every edge,
 /// an atomic for each) rather than in slots (every 16 senders look at the whole
-/// index): measured at 30 edges per node, 2000 nodes: 13.6 + 3 us (the
-/// consumers put the lists in order) against 8.5 us; 32 000 nodes: about 200
-/// against 457 us. The cost of the slots grows with edges x nodes.
+/// index, which costs edges x nodes). Measured at 30 edges per node, whole vjp
+/// in float, by arrival / in slots: 2000 nodes 66.7 / 60.7 us, 3000: 93.8 /
+/// 92.8, 4000: 113.7 / 114.0, 6000: 170 / 179, 8000: 233 / 255, 20 000: 682 /
+/// 820 (double alike).
 static bool lists_by_arrival(const Shape& s) {
-    return s.n_nodes > 6000 && static_cast<size_t>(s.n_nodes) * ((s.L + 15) / 16) <= SCRATCH_COUNTERS;
+    return s.n_nodes > 4000 && static_cast<size_t>(s.n_nodes) * ((s.L + 15) / 16) <= SCRATCH_COUNTERS;
 }
 
 bool vjp_supported(const Shape& s, size_t element_size, bool want_grad_W) {

@@ -82,7 +82,7 @@ CASES = {
             support.sasaw_case(s, d, E=6000, nA=4, L=8, n_nodes=300, n2=3, n3=5, N=40, allow_empty=True),
             "indices_W_1", SENDER_COUNTS
         ),
-        # (more than 6000 nodes: the senders' edges are listed in the order of arrival and sorted by their users)
+        # (more than 4000 nodes: the senders' edges are listed in the order of arrival and sorted by their users)
         "many_nodes_with_hubs": lambda s, d: _with_sender_counts(
             support.sasaw_case(s, d, E=70000, nA=4, L=24, n_nodes=6500, n2=3, n3=5, N=40, allow_empty=True),
             "indices_W_1", SENDER_COUNTS

@@ -2,7 +2,7 @@
 
 Shapes are drawn (fixed seed) from lists that straddle the limits at which the library changes
 kernels: 16 / 17 and 32 / 33 values of a component or feature index, 64 / 65 columns, one row or
-edge, 47 / 49 edges per node, 6000 nodes, tables of 2047 / 2049 entries, the row counts at which
+edge, 47 / 49 edges per node, 4000 nodes, tables of 2047 / 2049 entries, the row counts at which
 SAP's wavefronts start to walk. Every output and gradient is compared with the oracle run in
 float64 on the same (already rounded) inputs.
 

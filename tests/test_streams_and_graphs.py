@@ -28,7 +28,7 @@ CASES = {
     "opsa_pooling": lambda d: support.opsa_case(26, d, J=6000, K=13, L=20, n_out=8),
     # blocks of 64 columns, grad_A added to by one launch after the other
     "sasaw_many_columns": lambda d: support.sasaw_case(27, d, E=1500, nA=9, L=160, n_nodes=50, allow_empty=True),
-    # more than 6000 nodes: the senders' edges listed by arrival, on counters that every replay must find at zero
+    # more than 4000 nodes: the senders' edges listed by arrival, on counters that every replay must find at zero
     "sasaw_many_senders": lambda d: support.sasaw_case(28, d, E=30000, nA=4, L=16, n_nodes=16000, n2=4, n3=4, N=30, allow_empty=True),
 }
 

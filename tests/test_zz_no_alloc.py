@@ -78,7 +78,7 @@ def test_two_calls_in_a_row_the_second_smaller(oracle, device):
             assert torch.equal(got[name], want[name]), (wanted, name)
 
 
-def test_more_than_6000_nodes(oracle, device):
+def test_nodes_beyond_the_slots(oracle, device):
     """Graphs of this size list the senders' edges by arrival, on counters that have to start at
     zero: here they lie in the built-in array, behind whatever an earlier call left there."""
     import torch
