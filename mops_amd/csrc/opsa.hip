@@ -868,6 +868,13 @@ __global__ __launch_bounds__((LISTS ? LISTING_WAVES : 1) * WAVE) void edge_rows_
     int32_t my_sender = 0;
     if constexpr (WEIGHTED) {
         my_sender = my_edge >= 0 ? indices_W[my_edge] : -1;
+        if constexpr (!LISTS) {
+            // large sparse graphs: every edge takes the next of its sender's places
+            // (sender_buckets.hpp: SenderArrivals; `slots` is null when nobody wants the lists)
+            if (slots != nullptr && q == 0 && my_edge >= 0) {
+                list_arrival(SenderArrivals{slots, slot_counts, 1}, n_output, my_sender, my_edge);
+            }
+        }
     }
     const bool sender_ok = !WEIGHTED || in_bounds(my_sender, n_output);
 
@@ -1191,12 +1198,15 @@ constexpr int SLOT_MEAN_LIMIT = 48;
 // index itself.
 constexpr int LISTED_WAVES = 4;
 
-template <typename T, int COLUMNS>
+/// ARRIVALS: the places hold the sender's edges in the order of arrival, with one
+/// count (SenderArrivals), which this kernel sets back to zero.
+template <typename T, int COLUMNS, bool ARRIVALS = false>
 __global__ __launch_bounds__(LISTED_WAVES* WAVE) void sum_slotted_rows_kernel(
     T* __restrict__ grad_W, const T* __restrict__ edge_W, const int32_t* __restrict__ slots,
-    const int32_t* __restrict__ counts, const int32_t* __restrict__ senders, int32_t n_edges,
+    int32_t* __restrict__ counts, const int32_t* __restrict__ senders, int32_t n_edges,
     int32_t n_nodes, int32_t L
 ) {
+    __shared__ int32_t sorting_areas[ARRIVALS ? LISTED_WAVES : 1][ARRIVALS ? SLOT_CAPACITY : 1];
     const int lane = threadIdx.x & (WAVE - 1);
     const int32_t node = __builtin_amdgcn_readfirstlane(blockIdx.x * LISTED_WAVES + (threadIdx.x >> 6));
     if (node >= n_nodes) {
@@ -1204,16 +1214,27 @@ __global__ __launch_bounds__(LISTED_WAVES* WAVE) void sum_slotted_rows_kernel(
     }
     const int32_t* mine = slots + static_cast<size_t>(node) * SLOT_CAPACITY;
     // all places asked for before the counts are known
-    const int32_t first_half = mine[lane];
-    const int32_t second_half = mine[lane + WAVE];
+    int32_t first_half = mine[lane];
+    int32_t second_half = mine[lane + WAVE];
     static_assert(SLOT_PARTS == 4 && SLOT_CAPACITY == 2 * WAVE, "the four parts of a sender's places in two registers");
-    const int4 part_counts = reinterpret_cast<const int4*>(counts)[node];
-    const int32_t c0 = __builtin_amdgcn_readfirstlane(part_counts.x);
-    const int32_t c1 = __builtin_amdgcn_readfirstlane(part_counts.y);
-    const int32_t c2 = __builtin_amdgcn_readfirstlane(part_counts.z);
-    const int32_t c3 = __builtin_amdgcn_readfirstlane(part_counts.w);
-    const bool listed = max(max(c0, c1), max(c2, c3)) <= SLOT_PART_CAPACITY;
-    const int32_t count = c0 + c1 + c2 + c3;
+    int32_t c0 = 0, c1 = 0, c2 = 0, c3 = 0;
+    bool listed;
+    int32_t count;
+    if constexpr (ARRIVALS) {
+        count = __builtin_amdgcn_readfirstlane(counts[node]);
+        if (lane == 0) {
+            counts[node] = 0; // (nobody else reads it: zero again for the next launch)
+        }
+        listed = count <= SLOT_CAPACITY;
+    } else {
+        const int4 part_counts = reinterpret_cast<const int4*>(counts)[node];
+        c0 = __builtin_amdgcn_readfirstlane(part_counts.x);
+        c1 = __builtin_amdgcn_readfirstlane(part_counts.y);
+        c2 = __builtin_amdgcn_readfirstlane(part_counts.z);
+        c3 = __builtin_amdgcn_readfirstlane(part_counts.w);
+        listed = max(max(c0, c1), max(c2, c3)) <= SLOT_PART_CAPACITY;
+        count = c0 + c1 + c2 + c3;
+    }
     T sum[COLUMNS];
     uint32_t column[COLUMNS];
 #pragma unroll
@@ -1260,11 +1281,16 @@ __global__ __launch_bounds__(LISTED_WAVES* WAVE) void sum_slotted_rows_kernel(
             return place < WAVE ? low : high;
         };
         const int32_t n_first = min(count, WAVE);
-        const int32_t first = edge_at(lane);
+        if constexpr (ARRIVALS) {
+            if (count > 0) {
+                arrivals_in_order(first_half, second_half, count, sorting_areas[threadIdx.x >> 6], lane);
+            }
+        }
+        const int32_t first = ARRIVALS ? first_half : edge_at(lane);
         add_rows(lane < n_first ? first : 0, n_first);
         if (count > WAVE) {
             const int32_t n_second = count - WAVE;
-            const int32_t second = edge_at(lane + WAVE);
+            const int32_t second = ARRIVALS ? second_half : edge_at(lane + WAVE);
             add_rows(lane < n_second ? second : 0, n_second);
         }
     } else {
@@ -1575,15 +1601,24 @@ void launch_vjp(
     const bool narrow_rows = L <= GATHER_COLUMNS * WAVE;
     // (at 60 000 edges the lists cost more than the scans: 52 us against 32 for the whole vjp)
     const bool gather_in_kernel = narrow_rows && n_edges > 0 && index_reads <= SENDER_SCAN_LIMIT;
-    // sparse graphs: the pass over the sender index is done by workgroups of the
+    const bool sparse = n_output > 0 && L > 0 &&
+                        static_cast<size_t>(n_edges) <= static_cast<size_t>(n_output) * SLOT_MEAN_LIMIT;
+    // large sparse graphs: every edge takes the next of its sender's places in the per-edge
+    // kernel itself, an atomic each, and the sum puts the places in order. Whole vjp at 30 edges
+    // per sender, L = 32, f32, this way against the slots below (up to 4000 senders) or the
+    // counting sort beside the per-edge kernel (beyond): 2000 senders 27.6 / 22.6 us, 3000:
+    // 33.4 / 29.6, 4000: 37.6 / 39.3, 6000: 48 / 75, 20 000: 156 / 212
+    const bool by_arrival = want_W && narrow_rows && sparse && K > 0 && K <= 32 &&
+                            (n_output > 4000 || !gather_in_kernel) &&
+                            static_cast<size_t>(n_output) <= SCRATCH_COUNTERS;
+    // small sparse graphs: the pass over the sender index is done by workgroups of the
     // per-edge kernel's launch and leaves every sender's edges in places of its own
     // (60 000 edges over 2000 senders, L = 32, f32: 33 -> 22 us for the whole vjp;
     // graphs with more edges per sender keep the gather)
-    const bool slotted = want_W && gather_in_kernel && n_output > 0 && L > 0 &&
-                         static_cast<size_t>(n_edges) <= static_cast<size_t>(n_output) * SLOT_MEAN_LIMIT;
-    const size_t slots_bytes = slotted ? sender_slots_bytes(n_output) : 0;
+    const bool slotted = want_W && gather_in_kernel && sparse && !by_arrival;
+    const size_t slots_bytes = slotted ? sender_slots_bytes(n_output) : by_arrival ? sender_arrivals_bytes(n_output) : 0;
     const size_t buckets_bytes =
-        want_W && !gather_in_kernel ? edges_by_sender_bytes(n_output, n_edges) : slots_bytes;
+        want_W && !gather_in_kernel && !by_arrival ? edges_by_sender_bytes(n_output, n_edges) : slots_bytes;
     char* workspace =
         want_W ? static_cast<char*>(scratch(edge_w_bytes + buckets_bytes)) : nullptr;
     T* edge_W = want_W ? reinterpret_cast<T*>(workspace) : nullptr;
@@ -1593,7 +1628,7 @@ void launch_vjp(
     SenderBuckets buckets{};
     EdgesBySender by_sender{};
     SenderSlots slots{};
-    const bool use_buckets = want_W && n_output > 0 && L > 0 && !gather_in_kernel;
+    const bool use_buckets = want_W && n_output > 0 && L > 0 && !gather_in_kernel && !by_arrival;
     std::unique_ptr<SideStream> beside;
     bool listed = false; // the slots are being filled by a kernel that is already enqueued
     if (use_buckets) {
@@ -1687,6 +1722,9 @@ void launch_vjp(
                 slots = sender_slots_in(workspace + edge_w_bytes, n_output);
                 listed = true;
             }
+            if (by_arrival) {
+                slots = SenderSlots{reinterpret_cast<int32_t*>(workspace + edge_w_bytes), scratch_counters()};
+            }
             if (K <= 16) {
                 if (L <= 16) {
                     MOPS_LAUNCH_ROWS(1, 1);
@@ -1721,14 +1759,28 @@ void launch_vjp(
         }
     }
 
-    if (slotted) {
+    if (by_arrival) {
+        const unsigned blocks = static_cast<unsigned>(ceil_div(static_cast<size_t>(n_output), LISTED_WAVES));
+#define MOPS_LAUNCH_ARRIVED(COLUMNS)                                                               \
+    sum_slotted_rows_kernel<T, COLUMNS, true><<<blocks, LISTED_WAVES * WAVE, 0, stream>>>(         \
+        grad_W.data, edge_W, slots.edges, const_cast<int32_t*>(slots.counts), indices_W, n_edges, n_output, L \
+    )
+        if (L <= WAVE) {
+            MOPS_LAUNCH_ARRIVED(1);
+        } else if (L <= 2 * WAVE) {
+            MOPS_LAUNCH_ARRIVED(2);
+        } else {
+            MOPS_LAUNCH_ARRIVED(4);
+        }
+#undef MOPS_LAUNCH_ARRIVED
+    } else if (slotted) {
         if (!listed) {
             slots = list_edges_in_slots(indices_W, n_edges, n_output, workspace + edge_w_bytes, stream);
         }
         const unsigned blocks = static_cast<unsigned>(ceil_div(static_cast<size_t>(n_output), LISTED_WAVES));
 #define MOPS_LAUNCH_SLOTTED(COLUMNS)                                                                \
     sum_slotted_rows_kernel<T, COLUMNS><<<blocks, LISTED_WAVES * WAVE, 0, stream>>>(               \
-        grad_W.data, edge_W, slots.edges, slots.counts, indices_W, n_edges, n_output, L                   \
+        grad_W.data, edge_W, slots.edges, const_cast<int32_t*>(slots.counts), indices_W, n_edges, n_output, L \
     )
         if (L <= WAVE) {
             MOPS_LAUNCH_SLOTTED(1);

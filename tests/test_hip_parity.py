@@ -61,6 +61,10 @@ CASES = {
         "sparse_with_hubs": lambda s, d: _with_sender_counts(
             support.opsaw_case(s, d, E=6000, K=4, L=32, n_nodes=300, allow_empty=True), "indices_W", SENDER_COUNTS
         ),
+        # (more than 4000 nodes: the senders' edges are listed in the order of arrival and sorted by their users)
+        "many_nodes_with_hubs": lambda s, d: _with_sender_counts(
+            support.opsaw_case(s, d, E=70000, K=4, L=24, n_nodes=4500, allow_empty=True), "indices_W", SENDER_COUNTS
+        ),
         "forty_five_per_sender": lambda s, d: support.opsaw_case(s, d, E=4500, K=6, L=32, n_nodes=100),
         "sparse_tall": lambda s, d: support.opsaw_case(s, d, E=700, K=40, L=24, n_nodes=60, allow_empty=True),
         "pooling": lambda s, d: support.opsaw_case(s, d, E=5000, K=13, L=32, n_nodes=7),

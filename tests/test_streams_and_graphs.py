@@ -29,6 +29,7 @@ CASES = {
     # blocks of 64 columns, grad_A added to by one launch after the other
     "sasaw_many_columns": lambda d: support.sasaw_case(27, d, E=1500, nA=9, L=160, n_nodes=50, allow_empty=True),
     # more than 4000 nodes: the senders' edges listed by arrival, on counters that every replay must find at zero
+    "opsaw_many_senders": lambda d: support.opsaw_case(29, d, E=30000, K=4, L=16, n_nodes=9000, allow_empty=True),
     "sasaw_many_senders": lambda d: support.sasaw_case(28, d, E=30000, nA=4, L=16, n_nodes=16000, n2=4, n3=4, N=30, allow_empty=True),
 }
 
