@@ -1608,7 +1608,9 @@ void launch_vjp(
     // per sender, L = 32, f32, this way against the slots below (up to 4000 senders) or the
     // counting sort beside the per-edge kernel (beyond): 2000 senders 27.6 / 22.6 us, 3000:
     // 33.4 / 29.6, 4000: 37.6 / 39.3, 6000: 48 / 75, 20 000: 156 / 212
-    const bool by_arrival = want_W && narrow_rows && sparse && K > 0 && K <= 32 &&
+    // (with no edges at all gather_in_kernel is false too: the per-edge kernel that would fill the
+    // places is not launched then, so this way needs edges)
+    const bool by_arrival = want_W && narrow_rows && sparse && n_edges > 0 && K > 0 && K <= 32 &&
                             (n_output > 4000 || !gather_in_kernel) &&
                             static_cast<size_t>(n_output) <= SCRATCH_COUNTERS;
     // small sparse graphs: the pass over the sender index is done by workgroups of the
@@ -1628,6 +1630,10 @@ void launch_vjp(
     SenderBuckets buckets{};
     EdgesBySender by_sender{};
     SenderSlots slots{};
+    if (by_arrival) {
+        // (places and counters of SenderArrivals: filled by the per-edge kernel, used by the sum)
+        slots = SenderSlots{reinterpret_cast<int32_t*>(workspace + edge_w_bytes), scratch_counters()};
+    }
     const bool use_buckets = want_W && n_output > 0 && L > 0 && !gather_in_kernel && !by_arrival;
     std::unique_ptr<SideStream> beside;
     bool listed = false; // the slots are being filled by a kernel that is already enqueued
@@ -1722,9 +1728,7 @@ void launch_vjp(
                 slots = sender_slots_in(workspace + edge_w_bytes, n_output);
                 listed = true;
             }
-            if (by_arrival) {
-                slots = SenderSlots{reinterpret_cast<int32_t*>(workspace + edge_w_bytes), scratch_counters()};
-            }
+
             if (K <= 16) {
                 if (L <= 16) {
                     MOPS_LAUNCH_ROWS(1, 1);

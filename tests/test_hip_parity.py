@@ -297,9 +297,10 @@ def test_rows_without_edges_are_exactly_zero(device, op):
 
 
 def test_no_edges_at_all(device):
-    """Zero input rows: outputs are all zero, gradients are empty."""
-    for op in ("opsa", "opsaw", "sasaw"):
-        case = CASES[op]["tiny"](1, np.float64)
+    """Zero input rows: outputs are all zero, gradients are empty. (Also for many nodes: the
+    ways of listing the senders' edges that large graphs take need edges to list.)"""
+    for op, name in (("opsa", "tiny"), ("opsaw", "tiny"), ("sasaw", "tiny"), ("opsaw", "many_nodes_with_hubs"), ("sasaw", "many_nodes_with_hubs")):
+        case = CASES[op][name](1, np.float64)
         for key in ("A", "B"):
             case[key] = case[key][:0]
         for key in ("indices_output", "indices_W", "indices_output_1", "indices_W_1"):
