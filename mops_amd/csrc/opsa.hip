@@ -1221,7 +1221,7 @@ __global__ __launch_bounds__(LISTED_WAVES* WAVE) void sum_slotted_rows_kernel(
     bool listed;
     int32_t count;
     if constexpr (ARRIVALS) {
-        count = __builtin_amdgcn_readfirstlane(counts[node]);
+        count = max(__builtin_amdgcn_readfirstlane(counts[node]), 0);
         if (lane == 0) {
             counts[node] = 0; // (nobody else reads it: zero again for the next launch)
         }
@@ -1285,6 +1285,10 @@ __global__ __launch_bounds__(LISTED_WAVES* WAVE) void sum_slotted_rows_kernel(
             if (count > 0) {
                 arrivals_in_order(first_half, second_half, count, sorting_areas[threadIdx.x >> 6], lane);
             }
+            // (the counters outlive a call: should a failed launch ever leave a count without its
+            // list, what the places hold is kept inside the tensor all the same)
+            first_half = min(max(first_half, 0), n_edges - 1);
+            second_half = min(max(second_half, 0), n_edges - 1);
         }
         const int32_t first = ARRIVALS ? first_half : edge_at(lane);
         add_rows(lane < n_first ? first : 0, n_first);

@@ -669,8 +669,13 @@ __device__ __forceinline__ bool sum_over_arrivals(
     }
     const auto& p = sum.p;
     sum.clear();
+    // (A negative count is no count. The counters outlive a call, so a launch that failed
+    // between a listing and its readers can leave counts without lists behind them: what a
+    // place holds is used as an edge only if it can be one, so that such a remnant gives wrong
+    // sums in the next call but no access outside the tensors.)
+    count = max(count, 0);
     auto hand_on = [&](int32_t edges, int32_t n) {
-        const int32_t mine = lane < n ? edges : -1;
+        const int32_t mine = lane < n && in_bounds(edges, p.n_edges) ? edges : -1;
         const int32_t sources = load_or_zero(p.gather_index, static_cast<size_t>(max(mine, 0)), mine >= 0);
         sum.add(mine, mine >= 0 ? sources : -1, n);
     };
