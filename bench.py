@@ -13,17 +13,35 @@ so that the Infinity Cache cannot serve them. The timed region is an integer
 number of replays of one HIP graph that holds a divisor of K steps, so the
 figure does not depend on K.
 
+The step is timed ``--repetitions`` times (25 by default), each repetition
+being exactly ``--steps`` steps between two host synchronisations;
+``ms_per_step`` and ``value`` are the MEDIAN repetition, ``repetitions`` holds
+the minimum, median and maximum.
+
 ``per_op`` has one entry per function: the device time of a call (every kernel
 the call launches; HIP-graph replays between HIP events), the same with the
-same buffers every call (``device_us_same_buffers``), the time a plain copy
-kernel takes to read and write exactly the tensors the call reads and writes
-(``copy_us``: the yardstick; ``frac_of_copy`` = copy_us / device_us), and the
-CPU oracle on the host cores. ``roofline`` is the kernel with the most time in
-a step; ``roofline_per_op`` lists the main kernel of every call. Their
-durations come from pairs of HIP events that the library puts around that
-kernel on the stream it launches it on (mops_amd_kernel_timing in
-include/mops/amd.h); ``traffic`` is read from the rocprofv3 counter summary in
-profiles/ (kernels are matched by name).
+same buffers every call (``device_us_same_buffers``), two copy yardsticks timed
+the same way (``copy_spans_us``: a copy kernel that reads and writes exactly
+the tensors the call reads and writes; ``copy_flat_us``: one flat grid-stride
+copy, 16 bytes per lane, of the same number of bytes read and written;
+``copy_us`` is the smaller of the two and ``frac_of_copy`` = copy_us /
+device_us), the useful floating-point operations of the call (``flops``: the
+factored count, see ``useful_flops``) with ``flop_frac`` = flops / device time
+/ the vector-or-matrix peak of the dtype, and the CPU oracle on the host cores.
+``per_op_scaled`` is the same (without the CPU leg) at 16 to 100 times the rows
+or edges of the BASELINE shapes: sizes at which a launch lasts long enough to
+be bound by bandwidth or arithmetic rather than by latency.
+
+``roofline`` is the kernel with the most time in a step; ``roofline_per_op``
+lists the main kernel of every call. Their durations come from pairs of HIP
+events that the library puts around that kernel on the stream it launches it on
+(mops_amd_kernel_timing in include/mops/amd.h). Each entry carries both
+fractions (``hbm_frac`` of 8 TB/s on the algorithmic bytes, ``flop_frac`` of
+the dtype's peak on the useful flops) and ``bound`` = the ceiling that is the
+nearer one for that kernel's shape (the larger of bytes / 8 TB/s and flops /
+peak); ``frac`` is the fraction of THAT ceiling. ``traffic`` is read from the
+rocprofv3 counter summary in profiles/ (kernels are matched by name), so it is
+as fresh as that file.
 
 ``cpu_baseline`` times the CPU oracle (a port of the reference's OpenMP
 algorithm, oracle/oracle.cpp) on the same step on this machine's host cores,
@@ -44,6 +62,7 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X, published
+FLOP_PEAK_TFLOPS = {"float32": 157.3, "float64": 78.6}  # MI355X, published (vector = dense matrix for these types)
 ROTATE_BYTES = 320 * 1024 * 1024  # > 256 MB Infinity Cache
 TRAFFIC_FILE = os.path.join(ROOT, "profiles", "all_ops_baseline_shapes_hbm_traffic.txt")
 
@@ -95,6 +114,76 @@ def algorithmic_bytes(op, case, kind):
     return nbytes(inputs) + case["grad_output"].nbytes + nbytes(grads)
 
 
+def useful_flops(op, case, kind):
+    """Floating-point operations of one call in the cheapest formulation known (what a kernel
+    must do, not what it pads to): a multiply and an add count one each.
+
+    HPE       forward I J (K + 1); vjp I J (K^2 + 1) (every factor's partial product afresh)
+    SAP       forward 3 I K; vjp 5 I K
+    OPSA      forward 2 J K L; vjp 4 J K L
+    OPSAW     forward E L + 2 E K L (b * w once per edge);
+              vjp 4 E K L + 3 E L (t = sum_k g A once, then grad_B = t w, grad_W = t b)
+    SASAW     with the table factored out of the sum over edges (per node Z = sum_e a (b w), then
+              O = D Z with the N table entries): forward E (2 nA n2 L + n2 L) + 2 nodes N L;
+              vjp three such contractions (grad_A, grad_B, grad_W) and two passes over the table:
+              3 E 2 nA n2 L + E (4 n2 L) + 4 nodes N L
+    """
+    A = case["A"]
+    if op == "hpe":
+        I, (J, K) = A.shape[0], case["indices_A"].shape
+        return I * J * (K + 1) if kind == "forward" else I * J * (K * K + 1)
+    if op == "sap":
+        I, K = A.shape[0], case["C"].shape[0]
+        return (3 if kind == "forward" else 5) * I * K
+    if op == "opsa":
+        J, K, L = A.shape[0], A.shape[1], case["B"].shape[1]
+        return (2 if kind == "forward" else 4) * J * K * L
+    if op == "opsaw":
+        E, K, L = A.shape[0], A.shape[1], case["B"].shape[1]
+        return E * L + 2 * E * K * L if kind == "forward" else 4 * E * K * L + 3 * E * L
+    if op == "sasaw":
+        E, nA, L = A.shape[0], A.shape[1], case["B"].shape[1]
+        nodes, n2 = case["W"].shape[0], case["W"].shape[1]
+        N = case["C"].shape[0]
+        if kind == "forward":
+            return E * (2 * nA * n2 * L + n2 * L) + 2 * nodes * N * L
+        return 3 * E * 2 * nA * n2 * L + E * 4 * n2 * L + 4 * nodes * N * L
+    raise ValueError(op)
+
+
+def ceilings(abytes, flops, dtype_name, seconds):
+    """Both roofline fractions of a call or launch that took ``seconds``, and which ceiling binds."""
+    peak = FLOP_PEAK_TFLOPS[dtype_name]
+    hbm_seconds = abytes / (HBM_PEAK_GBS * 1e9)
+    flop_seconds = flops / (peak * 1e12)
+    bound = "hbm" if hbm_seconds >= flop_seconds else "mfma"
+    return {
+        "hbm_frac": round(hbm_seconds / seconds, 4),
+        "flops": int(flops),
+        "TFLOPs": round(flops / seconds / 1e12, 3),
+        "flop_peak_TFLOPs": peak,
+        "flop_frac": round(flop_seconds / seconds, 4),
+        "bound": bound,
+        "frac": round(max(hbm_seconds, flop_seconds) / seconds, 4),
+    }
+
+
+def build_scaled_configs():
+    """16 to 100 times the rows or edges of the BASELINE shapes, same feature counts."""
+    from tests import support
+
+    return [
+        ("c0x100", "hpe", np.float64, lambda: support.hpe_case(0, np.float64, I=100000)),
+        ("c1x31", "sap", np.float32, lambda: support.sap_case(1, np.float32, I=1000000)),
+        ("c1x31", "sap", np.float64, lambda: support.sap_case(1, np.float64, I=1000000)),
+        ("c2x16", "opsa", np.float32, lambda: support.opsa_case(2, np.float32, J=1000000, n_out=33000)),
+        ("c2x16", "opsa", np.float64, lambda: support.opsa_case(2, np.float64, J=1000000, n_out=33000)),
+        ("c3x16", "opsaw", np.float32, lambda: support.opsaw_case(3, np.float32, E=1000000, n_nodes=33000)),
+        ("c4x16", "sasaw", np.float32, lambda: support.sasaw_case(4, np.float32, E=1000000, n_nodes=33000)),
+        ("c4x16", "sasaw", np.float64, lambda: support.sasaw_case(4, np.float64, E=1000000, n_nodes=33000)),
+    ]
+
+
 def build_configs(extra):
     from tests import support
 
@@ -127,8 +216,63 @@ class Span(ctypes.Structure):
     _fields_ = [("data", ctypes.c_void_p), ("bytes", ctypes.c_int64)]
 
 
+class Yardstick:
+    """The two copy kernels of mops_amd/lib/libmops_yardstick.so (a library of the benchmark's
+    own, built from mops_amd/csrc/yardstick.hip; not part of libmops.so)."""
+
+    def __init__(self, device):
+        import torch
+
+        path = os.path.join(ROOT, "mops_amd", "lib", "libmops_yardstick.so")
+        if not os.path.exists(path):
+            raise RuntimeError(f"{path} is missing: build it with `make -C mops_amd/csrc`")
+        self.cdll = ctypes.CDLL(path)
+        self.cdll.mops_yardstick_copy_spans.argtypes = [
+            ctypes.c_void_p, ctypes.c_int32, ctypes.c_void_p, ctypes.c_int32, ctypes.c_void_p,
+        ]  # fmt: skip
+        self.cdll.mops_yardstick_copy_flat.argtypes = [
+            ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p,
+        ]  # fmt: skip
+        self.device = device
+        self.torch = torch
+        self.pool = None
+        self.cursor = 0
+
+    def _stream(self):
+        return ctypes.c_void_p(self.torch.cuda.current_stream(self.device).cuda_stream)
+
+    def spans(self, reads, writes):
+        status = self.cdll.mops_yardstick_copy_spans(reads, len(reads), writes, len(writes), self._stream())
+        if status != 0:
+            raise RuntimeError(f"mops_yardstick_copy_spans: HIP error {status}")
+
+    def flat(self, read_bytes, write_bytes):
+        """One flat copy that reads ``read_bytes`` and writes ``write_bytes`` (rounded up to 16),
+        at a place of a pool of more than 320 MB that moves on with every call."""
+        read_bytes = (read_bytes + 15) // 16 * 16
+        write_bytes = (write_bytes + 15) // 16 * 16
+        both = (read_bytes + write_bytes + 255) // 256 * 256
+        need = max(2 * ROTATE_BYTES, 2 * both)
+        if self.pool is None or self.pool.numel() < need:
+            self.pool = None
+            self.torch.cuda.empty_cache()
+            self.pool = self.torch.zeros(need, dtype=self.torch.uint8, device=self.device)
+            self.cursor = 0
+        if self.cursor + both > self.pool.numel():
+            self.cursor = 0
+        base = self.pool.data_ptr() + self.cursor
+        self.cursor += both
+        status = self.cdll.mops_yardstick_copy_flat(
+            ctypes.c_void_p(base), read_bytes, ctypes.c_void_p(base + read_bytes), write_bytes, self._stream()
+        )
+        if status != 0:
+            raise RuntimeError(f"mops_yardstick_copy_flat: HIP error {status}")
+
+
 class DeviceWorkload:
     """One operation with its inputs replicated over enough buffer sets to defeat the caches."""
+
+    yardstick = None  # a Yardstick, set by main()
 
     def __init__(self, op, case, device):
         import torch
@@ -178,22 +322,40 @@ class DeviceWorkload:
         self.forward()
         self.vjp()
 
-    # the copy yardstick on the tensors the call reads and writes
-    def _copy(self, read_names, write_names):
+    # the copy yardsticks: on the tensors the call reads and writes, and flat
+    def _names(self, kind):
+        if kind == "forward":
+            return list(self.spec.inputs), ["output"]
+        return ["grad_output", *self.spec.inputs], ["grad_" + n for n in self.spec.differentiable]
+
+    def _copy(self, kind):
         t = self._next()
+        read_names, write_names = self._names(kind)
         reads = (Span * len(read_names))(*[Span(t[n].data_ptr(), t[n].numel() * t[n].element_size()) for n in read_names])
         writes = (Span * len(write_names))(
             *[Span(t[n].data_ptr(), t[n].numel() * t[n].element_size()) for n in write_names]
         )
-        status = self.library.cdll.mops_amd_copy_yardstick(reads, len(read_names), writes, len(write_names))
-        if status != 0:
-            raise RuntimeError(self.library.last_error())
+        self.yardstick.spans(reads, writes)
+
+    def _flat(self, kind):
+        t = self.sets[0]
+        read_names, write_names = self._names(kind)
+        self.yardstick.flat(
+            sum(t[n].numel() * t[n].element_size() for n in read_names),
+            sum(t[n].numel() * t[n].element_size() for n in write_names),
+        )
 
     def copy_forward(self):
-        self._copy(list(self.spec.inputs), ["output"])
+        self._copy("forward")
 
     def copy_vjp(self):
-        self._copy(["grad_output", *self.spec.inputs], ["grad_" + n for n in self.spec.differentiable])
+        self._copy("vjp")
+
+    def flat_forward(self):
+        self._flat("forward")
+
+    def flat_vjp(self):
+        self._flat("vjp")
 
 
 def bind_library_to_torch_stream(device):
@@ -342,6 +504,13 @@ def main():
         "shapes (all their dtypes), each followed by the copy yardstick on the same tensors, and 20 element-wise "
         "passes over 64 MiB (read 64 MiB, write 64 MiB) as a yardstick for the HBM counters, print nothing, exit",
     )
+    parser.add_argument(
+        "--profile-scaled", action="store_true",
+        help="with --profile: also 10 eager forward+vjp calls at the scaled shapes (per_op_scaled), each followed "
+        "by the flat copy of the same number of bytes",
+    )  # fmt: skip
+    parser.add_argument("--repetitions", type=int, default=25, help="how often the region of --steps steps is timed")
+    parser.add_argument("--no-scaled", action="store_true", help="leave per_op_scaled out")
     args = parser.parse_args()
 
     if args.gpus != 1:
@@ -362,7 +531,7 @@ def main():
         sys.exit(2)
     device = torch.device("cuda:0")
     library = bind_library_to_torch_stream(device)
-    library.cdll.mops_amd_copy_yardstick.argtypes = [ctypes.c_void_p, ctypes.c_int32, ctypes.c_void_p, ctypes.c_int32]
+    DeviceWorkload.yardstick = Yardstick(device)
     oracle = support.oracle_library()
     configs = build_configs(args.extra_shapes)
     baseline = [c for c in configs if c[0].startswith("c")]
@@ -374,11 +543,25 @@ def main():
                 for _ in range(50):
                     w.forward()
                     w.copy_forward()
+                    w.flat_forward()
                     w.vjp()
                     w.copy_vjp()
+                    w.flat_vjp()
                 torch.cuda.synchronize()
                 del w
                 torch.cuda.empty_cache()
+        if args.profile_scaled:
+            for config, op_name, _, make_case in build_scaled_configs():
+                if args.profile in (op_name, "all"):
+                    w = DeviceWorkload(op_name, make_case(), device)
+                    for _ in range(10):
+                        w.forward()
+                        w.flat_forward()
+                        w.vjp()
+                        w.flat_vjp()
+                    torch.cuda.synchronize()
+                    del w
+                    torch.cuda.empty_cache()
         source = torch.empty(64 * 1024 * 1024 // 4, dtype=torch.float32, device=device).normal_()
         target = torch.empty_like(source)
         for _ in range(20):
@@ -403,48 +586,57 @@ def main():
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
-    begin = time.perf_counter()
-    if graph is not None:
-        for _ in range(args.steps // steps_per_graph):
-            graph.replay()
-    else:
-        for _ in range(args.steps):
-            step()
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - begin
-    seconds_per_step = elapsed / args.steps
+    region_seconds = []
+    for _ in range(max(1, args.repetitions)):
+        torch.cuda.synchronize()
+        begin = time.perf_counter()
+        if graph is not None:
+            for _ in range(args.steps // steps_per_graph):
+                graph.replay()
+        else:
+            for _ in range(args.steps):
+                step()
+        torch.cuda.synchronize()
+        region_seconds.append(time.perf_counter() - begin)
+    seconds_per_step = float(np.median(region_seconds)) / args.steps
     value = step_bytes / seconds_per_step / 1e9
+    step_flops = {"float32": 0, "float64": 0}
+    for (_, _, dtype_name), w in workloads.items():
+        step_flops[dtype_name] += useful_flops(w.op, w.case, "forward") + useful_flops(w.op, w.case, "vjp")
 
-    # ---------------- per function: call, copy yardstick, main kernel, CPU ------------------
-    per_op = []
-    roofline_per_op = []
-    selected = [] if args.no_per_op else configs
-    for config, op_name, op_dtype, op_case in selected:
-        key = (config, op_name, np.dtype(op_dtype).name)
-        w = workloads.get(key) or DeviceWorkload(op_name, op_case, device)
-        type_name = "float" if op_dtype == np.float32 else "double"
-        for kind, function, copy in (("forward", w.forward, w.copy_forward), ("vjp", w.vjp, w.copy_vjp)):
-            calls = min(w.n_sets, 64)
-            seconds, captured = device_time_per_call(function, calls, 20, device)
-            copy_seconds, _ = device_time_per_call(copy, calls, 20, device)
-            abytes = algorithmic_bytes(op_name, op_case, kind)
-            entry = {
-                "config": config,
-                "op": op_name,
-                "dtype": np.dtype(op_dtype).name,
-                "function": kind,
-                "device_us": round(seconds * 1e6, 3),
-                "algorithmic_bytes": abytes,
-                "GBps": round(abytes / seconds / 1e9, 1),
-                "hbm_frac": round(abytes / seconds / 1e9 / HBM_PEAK_GBS, 4),
-                "copy_us": round(copy_seconds * 1e6, 3),
-                "frac_of_copy": round(copy_seconds / seconds, 3),
-                "timed": "hip-graph replay, HIP events" if captured else "eager launches, HIP events",
-            }
-            w.rotate = False
-            warm_seconds, _ = device_time_per_call(function, calls, 20, device)
-            w.rotate = True
-            entry["device_us_same_buffers"] = round(warm_seconds * 1e6, 3)
+    # ---------------- per function: call, copy yardsticks, main kernel, CPU ------------------
+    def measure(config, op_name, op_dtype, op_case, w, kind, with_cpu):
+        function = w.forward if kind == "forward" else w.vjp
+        copy = w.copy_forward if kind == "forward" else w.copy_vjp
+        flat = w.flat_forward if kind == "forward" else w.flat_vjp
+        dtype_name = np.dtype(op_dtype).name
+        calls = min(w.n_sets, 64)
+        seconds, captured = device_time_per_call(function, calls, 20, device)
+        spans_seconds, _ = device_time_per_call(copy, calls, 20, device)
+        flat_seconds, _ = device_time_per_call(flat, calls, 20, device)
+        copy_seconds = min(spans_seconds, flat_seconds)
+        abytes = algorithmic_bytes(op_name, op_case, kind)
+        flops = useful_flops(op_name, op_case, kind)
+        entry = {
+            "config": config,
+            "op": op_name,
+            "dtype": dtype_name,
+            "function": kind,
+            "device_us": round(seconds * 1e6, 3),
+            "algorithmic_bytes": abytes,
+            "GBps": round(abytes / seconds / 1e9, 1),
+            **ceilings(abytes, flops, dtype_name, seconds),
+            "copy_us": round(copy_seconds * 1e6, 3),
+            "copy_spans_us": round(spans_seconds * 1e6, 3),
+            "copy_flat_us": round(flat_seconds * 1e6, 3),
+            "frac_of_copy": round(copy_seconds / seconds, 3),
+            "timed": "hip-graph replay, HIP events" if captured else "eager launches, HIP events",
+        }
+        w.rotate = False
+        warm_seconds, _ = device_time_per_call(function, calls, 20, device)
+        w.rotate = True
+        entry["device_us_same_buffers"] = round(warm_seconds * 1e6, 3)
+        if with_cpu:
             cpu_function = (
                 (lambda c=op_case, o=op_name: support.cpu_forward(oracle, o, c))
                 if kind == "forward"
@@ -453,7 +645,20 @@ def main():
             times = cpu_time(cpu_function, 0.4, 20)
             entry["cpu_ms"] = round(float(np.median(times)) * 1e3, 3)
             entry["cpu_GBps"] = round(abytes / float(np.median(times)) / 1e9, 3)
+        return entry, seconds, calls
+
+    per_op = []
+    roofline_per_op = []
+    selected = [] if args.no_per_op else configs
+    for config, op_name, op_dtype, op_case in selected:
+        key = (config, op_name, np.dtype(op_dtype).name)
+        w = workloads.get(key) or DeviceWorkload(op_name, op_case, device)
+        type_name = "float" if op_dtype == np.float32 else "double"
+        for kind in ("forward", "vjp"):
+            entry, seconds, calls = measure(config, op_name, op_dtype, op_case, w, kind, True)
             per_op.append(entry)
+            function = w.forward if kind == "forward" else w.vjp
+            abytes = entry["algorithmic_bytes"]
 
             if config.startswith("c"):
                 kernel_seconds, launches = main_kernel_time(library, function, 200)
@@ -474,13 +679,26 @@ def main():
                         "launches_timed": launches,
                         "algorithmic_bytes_per_launch": abytes,
                         "achieved_GBps": round(abytes / kernel_seconds / 1e9, 1),
-                        "frac": round(abytes / kernel_seconds / 1e9 / HBM_PEAK_GBS, 4),
+                        **ceilings(abytes, entry["flops"], np.dtype(op_dtype).name, kernel_seconds),
                         "traffic": measured_traffic(name),
                         "timed": timed_by,
                     }
                 )
         if key not in workloads:
             del w
+            torch.cuda.empty_cache()
+
+    # ---------------- the same at sizes that can reach a ceiling -------------------------------
+    per_op_scaled = []
+    if not (args.no_per_op or args.no_scaled):
+        for config, op_name, op_dtype, make_case in build_scaled_configs():
+            op_case = make_case()
+            w = DeviceWorkload(op_name, op_case, device)
+            for kind in ("forward", "vjp"):
+                entry, _, _ = measure(config, op_name, op_dtype, op_case, w, kind, False)
+                entry["shape"] = {name: list(np.shape(op_case[name])) for name in w.spec.inputs}
+                per_op_scaled.append(entry)
+            del w, op_case
             torch.cuda.empty_cache()
 
     # ---------------- roofline of the kernel with the most time in a step -------------------
@@ -499,17 +717,28 @@ def main():
             "config": "c4", "op": "sasaw", "dtype": "float64", "function": "vjp", "kernel": name,
             "avg_us": round(kernel_seconds * 1e6, 3), "launches_timed": launches,
             "algorithmic_bytes_per_launch": abytes, "achieved_GBps": round(abytes / kernel_seconds / 1e9, 1),
-            "frac": round(abytes / kernel_seconds / 1e9 / HBM_PEAK_GBS, 4), "traffic": measured_traffic(name),
+            **ceilings(abytes, useful_flops("sasaw", w.case, "vjp"), "float64", kernel_seconds),
+            "traffic": measured_traffic(name),
             "timed": "HIP events around the kernel on its launch stream",
         }  # fmt: skip
+    # the ceiling that binds this kernel's shape: bytes / 8 TB/s against useful flops / peak
+    if dominant["bound"] == "hbm":
+        achieved, peak, unit = dominant["achieved_GBps"], HBM_PEAK_GBS, "GB/s"
+    else:
+        achieved, peak, unit = dominant["TFLOPs"], dominant["flop_peak_TFLOPs"], "TFLOP/s"
     roofline = {
-        "bound": "hbm",
+        "bound": dominant["bound"],
         "kernel": dominant["kernel"],
         "of": f"{dominant['config']} {dominant['op']} {dominant['dtype']} {dominant['function']}",
-        "achieved": dominant["achieved_GBps"],
-        "peak": HBM_PEAK_GBS,
-        "unit": "GB/s",
+        "achieved": achieved,
+        "peak": peak,
+        "unit": unit,
         "frac": dominant["frac"],
+        "hbm": {"achieved": dominant["achieved_GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": dominant["hbm_frac"]},
+        "flop": {
+            "achieved": dominant["TFLOPs"], "peak": dominant["flop_peak_TFLOPs"], "unit": "TFLOP/s",
+            "frac": dominant["flop_frac"], "useful_flops_per_launch": dominant["flops"],
+        },  # fmt: skip
         "traffic": dominant["traffic"],
         "traffic_from": os.path.relpath(TRAFFIC_FILE, ROOT),
         "algorithmic_bytes_per_launch": dominant["algorithmic_bytes_per_launch"],
@@ -555,6 +784,13 @@ def main():
         "steps": args.steps,
         "warmup": args.warmup,
         "ms_per_step": round(seconds_per_step * 1e3, 5),
+        "repetitions": {
+            "count": len(region_seconds),
+            "each": f"{args.steps} steps between two host synchronisations",
+            "ms_per_step_min": round(min(region_seconds) / args.steps * 1e3, 5),
+            "ms_per_step_median": round(float(np.median(region_seconds)) / args.steps * 1e3, 5),
+            "ms_per_step_max": round(max(region_seconds) / args.steps * 1e3, 5),
+        },
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
@@ -566,12 +802,17 @@ def main():
             f"(sixteen calls); inputs rotated over > 320 MB of buffer sets per operation; timed as "
             f"{args.steps // steps_per_graph} replays of one HIP graph of {steps_per_graph} steps",
             "algorithmic_bytes_per_step": step_bytes,
-            "value_is": "algorithmic bytes per step / wall time per step",
+            "value_is": "algorithmic bytes per step / wall time per step (median repetition)",
+            "useful_flops_per_step": step_flops,
+            "step_flop_frac": round(
+                sum(step_flops[d] / (FLOP_PEAK_TFLOPS[d] * 1e12) for d in step_flops) / seconds_per_step, 4
+            ),
         },
         "roofline": roofline,
         "cpu_baseline": cpu_baseline,
         "roofline_per_op": roofline_per_op,
         "per_op": per_op,
+        "per_op_scaled": per_op_scaled,
         "device": torch.cuda.get_device_name(0),
     }
     print(json.dumps(result))

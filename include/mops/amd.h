@@ -95,24 +95,6 @@ MOPS_EXPORT int mops_amd_accept_unsorted_indices(int accept);
 MOPS_EXPORT int mops_amd_reserve_scratch(int64_t bytes);
 MOPS_EXPORT int64_t mops_amd_scratch_capacity(void);
 
-/* A plain copy kernel, as the yardstick of benchmarks.
- *
- * One launch on the calling thread's stream that reads every span of `reads`
- * (device memory; start a multiple of 16 bytes, length a multiple of 4) once
- * and writes every span of `writes` once, 16 bytes per lane, at most 16 spans
- * each. Pointed at the tensors an operation reads and writes, its duration is
- * what moving that operation's bytes costs on the device at that size: the
- * scale on which a few-megabyte kernel should be read, since no kernel of
- * that size gets near the peak bandwidth. What is written is arbitrary.
- * Returns 0 / 1 / 2. */
-typedef struct {
-    const void* data;
-    int64_t bytes;
-} mops_amd_span_t;
-MOPS_EXPORT int mops_amd_copy_yardstick(
-    const mops_amd_span_t* reads, int32_t n_reads, const mops_amd_span_t* writes, int32_t n_writes
-);
-
 /* The entry point that allocates nothing.
  *
  * No counterpart in lab-cosmo/mops. It is for callers that cannot allocate

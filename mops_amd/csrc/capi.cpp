@@ -16,7 +16,6 @@
 #include "no_alloc.hpp"
 #include "edge_order.hpp"
 #include "runtime.hpp"
-#include "yardstick.hpp"
 
 namespace {
 
@@ -165,19 +164,5 @@ extern "C" int mops_amd_sparse_accumulation_scatter_add_with_weights_vjp_no_allo
 ) {
     MOPS_CATCH_EXCEPTIONS_BEGIN
     mops::amd::sasaw_vjp_no_alloc(MOPS_SASAW_VJP_PARAMS(MOPS_FORWARD_FIRST, MOPS_FORWARD_NEXT));
-    MOPS_CATCH_EXCEPTIONS_END
-}
-
-static_assert(sizeof(mops_amd_span_t) == sizeof(mops::amd::YardstickSpan), "the same two fields");
-
-extern "C" int mops_amd_copy_yardstick(
-    const mops_amd_span_t* reads, int32_t n_reads, const mops_amd_span_t* writes, int32_t n_writes
-) {
-    MOPS_CATCH_EXCEPTIONS_BEGIN
-    mops::amd::copy_yardstick(
-        reinterpret_cast<const mops::amd::YardstickSpan*>(reads), n_reads,
-        reinterpret_cast<const mops::amd::YardstickSpan*>(writes), n_writes, mops::amd::current_stream()
-    );
-    mops::amd::finish_call("copy_yardstick");
     MOPS_CATCH_EXCEPTIONS_END
 }

@@ -1,17 +1,33 @@
-// A plain copy kernel as a yardstick for the operations' kernels: it reads a
-// list of spans of device memory once and writes another list once, 16 bytes
-// per lane, and does nothing else. A benchmark points it at the very tensors
-// an operation reads and writes; the time it takes is what moving the
-// operation's algorithmic bytes costs on this device at this size.
-#include "yardstick.hpp"
-
+// Two plain copy kernels as yardsticks for the operations' kernels. They are
+// NOT part of libmops.so: this file is a library of its own
+// (mops_amd/lib/libmops_yardstick.so) that only the benchmark loads.
+//
+//   mops_yardstick_copy_spans  reads a list of spans of device memory once and
+//                              writes another list once, 16 bytes per lane. A
+//                              benchmark points it at the very tensors an
+//                              operation reads and writes.
+//   mops_yardstick_copy_flat   reads ONE range once and writes ONE range once,
+//                              16 bytes per lane, grid-stride, no span search:
+//                              the cheapest way this device moves that many
+//                              bytes in one launch.
+//
+// Both return the hipError_t of the launch (0 = launched) and run on the
+// stream they are given.
 #include <algorithm>
-#include <stdexcept>
+#include <cstdint>
 
-#include "runtime.hpp"
+#include <hip/hip_runtime.h>
 
-namespace mops::amd {
 namespace {
+
+constexpr int YARDSTICK_MAX_SPANS = 16;
+
+struct YardstickSpan {
+    const void* data;
+    int64_t bytes;
+};
+
+inline uint64_t ceil_div(uint64_t a, uint64_t b) { return (a + b - 1) / b; }
 
 constexpr int THREADS = 256;
 
@@ -86,20 +102,19 @@ __global__ __launch_bounds__(THREADS) void copy_yardstick_kernel(const Spans rea
     }
 }
 
-Spans pack(const YardstickSpan* spans, int count, const char* what) {
+/// False when the spans cannot be packed: more than 16, a start that is not a multiple of 16
+/// bytes, a length that is not a multiple of 4 bytes or is 16 GiB or more.
+bool pack(const YardstickSpan* spans, int count, Spans& packed) {
     if (count < 0 || count > YARDSTICK_MAX_SPANS) {
-        throw std::runtime_error(std::string("copy yardstick: at most 16 spans to ") + what);
+        return false;
     }
-    Spans packed{};
+    packed = Spans{};
     packed.count = count;
     uint64_t pieces = 0;
     for (int s = 0; s < count; s++) {
         if (spans[s].bytes < 0 || spans[s].bytes % 4 != 0 || reinterpret_cast<uintptr_t>(spans[s].data) % 16 != 0 ||
             spans[s].bytes / 4 > 0xffffffffll) {
-            throw std::runtime_error(
-                std::string("copy yardstick: every span to ") + what +
-                " must start at a multiple of 16 bytes and hold a multiple of 4 bytes (fewer than 16 GiB)"
-            );
+            return false;
         }
         packed.data[s] = static_cast<const uint32_t*>(spans[s].data);
         packed.words[s] = static_cast<uint32_t>(spans[s].bytes / 4);
@@ -109,26 +124,102 @@ Spans pack(const YardstickSpan* spans, int count, const char* what) {
     for (int s = count; s <= YARDSTICK_MAX_SPANS; s++) {
         packed.first_piece[s] = pieces;
     }
-    return packed;
+    return true;
+}
+
+// ---- the flat copy: one range in, one range out -------------------------------------------
+
+constexpr int FLAT_IN_FLIGHT = 4;
+
+__global__ __launch_bounds__(THREADS) void flat_copy_kernel(
+    const uint4* __restrict__ from, uint64_t read_pieces, uint4* __restrict__ to, uint64_t write_pieces
+) {
+    const uint64_t stride = static_cast<uint64_t>(gridDim.x) * THREADS;
+    const uint64_t start = static_cast<uint64_t>(blockIdx.x) * THREADS + threadIdx.x;
+    const uint64_t both = read_pieces < write_pieces ? read_pieces : write_pieces;
+    uint4 seen = make_uint4(0u, 0u, 0u, 0u);
+    uint64_t piece = start;
+    // the part that is read AND written: a piece is stored as it was loaded
+    for (; piece + (FLAT_IN_FLIGHT - 1) * stride < both; piece += FLAT_IN_FLIGHT * stride) {
+        uint4 value[FLAT_IN_FLIGHT];
+#pragma unroll
+        for (int u = 0; u < FLAT_IN_FLIGHT; u++) {
+            value[u] = from[piece + u * stride];
+        }
+#pragma unroll
+        for (int u = 0; u < FLAT_IN_FLIGHT; u++) {
+            to[piece + u * stride] = value[u];
+        }
+    }
+    for (; piece < both; piece += stride) {
+        to[piece] = from[piece];
+    }
+    // what is only read (kept alive by a store that never happens) ...
+    for (; piece + (FLAT_IN_FLIGHT - 1) * stride < read_pieces; piece += FLAT_IN_FLIGHT * stride) {
+        uint4 value[FLAT_IN_FLIGHT];
+#pragma unroll
+        for (int u = 0; u < FLAT_IN_FLIGHT; u++) {
+            value[u] = from[piece + u * stride];
+        }
+#pragma unroll
+        for (int u = 0; u < FLAT_IN_FLIGHT; u++) {
+            seen.x ^= value[u].x;
+            seen.y ^= value[u].y;
+            seen.z ^= value[u].z;
+            seen.w ^= value[u].w;
+        }
+    }
+    for (; piece < read_pieces; piece += stride) {
+        const uint4 value = from[piece];
+        seen.x ^= value.x ^ value.y ^ value.z ^ value.w;
+    }
+    // ... or only written
+    for (; piece < write_pieces; piece += stride) {
+        to[piece] = seen;
+    }
+    if (read_pieces > write_pieces && (seen.x ^ seen.y ^ seen.z ^ seen.w) == 0x9e3779b9u && write_pieces > 0 &&
+        start == 0xffffffffffull) {
+        to[0] = seen; // never true: start is below 2^40
+    }
 }
 
 } // namespace
 
-void copy_yardstick(
-    const YardstickSpan* reads, int n_reads, const YardstickSpan* writes, int n_writes, hipStream_t stream
+extern "C" __attribute__((visibility("default"))) int mops_yardstick_copy_spans(
+    const YardstickSpan* reads, int32_t n_reads, const YardstickSpan* writes, int32_t n_writes, void* stream
 ) {
-    const Spans from = pack(reads, n_reads, "read");
-    const Spans to = pack(writes, n_writes, "write");
+    Spans from, to;
+    if (!pack(reads, n_reads, from) || !pack(writes, n_writes, to)) {
+        return static_cast<int>(hipErrorInvalidValue);
+    }
     const uint64_t pieces = std::max(from.first_piece[from.count], to.first_piece[to.count]);
     if (pieces == 0) {
-        return;
+        return 0;
     }
     // a few pieces per thread, all of a thread's loads in flight together, and no more than
     // eight workgroups per compute unit
     const unsigned blocks =
         static_cast<unsigned>(std::min<uint64_t>(ceil_div(pieces, THREADS * IN_FLIGHT), 256 * 8));
-    copy_yardstick_kernel<<<blocks, THREADS, 0, stream>>>(from, to);
-    MOPS_HIP_CHECK(hipGetLastError());
+    copy_yardstick_kernel<<<blocks, THREADS, 0, static_cast<hipStream_t>(stream)>>>(from, to);
+    return static_cast<int>(hipGetLastError());
 }
 
-} // namespace mops::amd
+extern "C" __attribute__((visibility("default"))) int mops_yardstick_copy_flat(
+    const void* from, int64_t read_bytes, void* to, int64_t write_bytes, void* stream
+) {
+    if (read_bytes < 0 || write_bytes < 0 || read_bytes % 16 != 0 || write_bytes % 16 != 0 ||
+        reinterpret_cast<uintptr_t>(from) % 16 != 0 || reinterpret_cast<uintptr_t>(to) % 16 != 0) {
+        return static_cast<int>(hipErrorInvalidValue);
+    }
+    const uint64_t pieces = static_cast<uint64_t>(std::max(read_bytes, write_bytes)) / 16;
+    if (pieces == 0) {
+        return 0;
+    }
+    const unsigned blocks =
+        static_cast<unsigned>(std::min<uint64_t>(ceil_div(pieces, THREADS * FLAT_IN_FLIGHT), 256 * 8));
+    flat_copy_kernel<<<blocks, THREADS, 0, static_cast<hipStream_t>(stream)>>>(
+        static_cast<const uint4*>(from), static_cast<uint64_t>(read_bytes) / 16, static_cast<uint4*>(to),
+        static_cast<uint64_t>(write_bytes) / 16
+    );
+    return static_cast<int>(hipGetLastError());
+}
