@@ -70,14 +70,14 @@ TRAFFIC_FILE = os.path.join(ROOT, "profiles", "all_ops_baseline_shapes_hbm_traff
 # rocprofv3 prints it (a prefix; {T} = float / double). Used to label the
 # per-kernel figures and to find the kernel in the counter summary.
 MAIN_KERNELS = {
-    ("hpe", "forward"): "forward_ordered_kernel<{T}, 4>",
-    ("hpe", "vjp"): "vjp_ordered_kernel<{T}, 4, true>",
+    ("hpe", "forward"): "hpe::forward_ordered_kernel<{T}, 4>",
+    ("hpe", "vjp"): "hpe::vjp_ordered_kernel<{T}, 4, true>",
     ("sap", "forward"): "sap_mfma::forward_kernel<{T}, 2, 2>",
     ("sap", "vjp"): "sap_mfma::vjp_kernel<{T}, 5>",
-    ("opsa", "forward"): "forward_kernel<{T}, 2, false, true>",
-    ("opsa", "vjp"): "edge_rows_vjp_kernel<{T}, 1, 2, false, true, false, false>",
-    ("opsaw", "forward"): "forward_kernel<{T}, 2, true, true>",
-    ("opsaw", "vjp"): "edge_rows_vjp_kernel<{T}, 1, 2, true, true, false, true>",
+    ("opsa", "forward"): "opsa::forward_kernel<{T}, 2, false, true>",
+    ("opsa", "vjp"): "opsa::edge_rows_vjp_kernel<{T}, 1, 2, false, true, false, false>",
+    ("opsaw", "forward"): "opsa::forward_kernel<{T}, 2, true, true>",
+    ("opsaw", "vjp"): "opsa::edge_rows_vjp_kernel<{T}, 1, 2, true, true, false, true>",
     ("sasaw", "forward"): {
         "float": "sasaw_segments::contract_kernel<float, 9, true, 32>",
         "double": "sasaw_segments::contract_kernel<double, 9, true, 64>",

@@ -34,6 +34,7 @@
 #include "sender_buckets.hpp"
 
 namespace mops::amd {
+namespace hpe { // a name of its own for this file's kernels: profilers print it
 namespace {
 
 constexpr size_t LDS_BUDGET = 60 * 1024;
@@ -1100,6 +1101,8 @@ int pick_rows(size_t n_rows, size_t bytes_per_row) {
 }
 
 } // namespace
+} // namespace hpe
+using namespace hpe;
 } // namespace mops::amd
 
 namespace mops::cuda {

@@ -30,6 +30,7 @@
 // order is fixed (ascending edge number in steps of four), so results are
 // bit-reproducible.
 #include <algorithm>
+#include <optional>
 #include <cstdlib>
 #include <memory>
 
@@ -49,6 +50,7 @@
 #include "sender_gather.hpp"
 
 namespace mops::amd {
+namespace opsa { // a name of its own for this file's kernels: profilers print it
 namespace {
 
 constexpr int CHUNK = 32;            // index positions per wavefront
@@ -1634,9 +1636,11 @@ void launch_vjp(
     SenderBuckets buckets{};
     EdgesBySender by_sender{};
     SenderSlots slots{};
+    std::optional<ScratchCounters> taken; // (until the end of this call, finish_call included)
     if (by_arrival) {
         // (places and counters of SenderArrivals: filled by the per-edge kernel, used by the sum)
-        slots = SenderSlots{reinterpret_cast<int32_t*>(workspace + edge_w_bytes), scratch_counters()};
+        taken.emplace();
+        slots = SenderSlots{reinterpret_cast<int32_t*>(workspace + edge_w_bytes), taken->data()};
     }
     const bool use_buckets = want_W && n_output > 0 && L > 0 && !gather_in_kernel && !by_arrival;
     std::unique_ptr<SideStream> beside;
@@ -1768,6 +1772,7 @@ void launch_vjp(
     }
 
     if (by_arrival) {
+        test_failure_point("opsaw_vjp_after_listing");
         const unsigned blocks = static_cast<unsigned>(ceil_div(static_cast<size_t>(n_output), LISTED_WAVES));
 #define MOPS_LAUNCH_ARRIVED(COLUMNS)                                                               \
     sum_slotted_rows_kernel<T, COLUMNS, true><<<blocks, LISTED_WAVES * WAVE, 0, stream>>>(         \
@@ -1865,6 +1870,8 @@ private:
 };
 
 } // namespace
+} // namespace opsa
+using namespace opsa;
 } // namespace mops::amd
 
 // ------------------------------------------------------------ C++ API ----

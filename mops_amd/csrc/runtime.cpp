@@ -3,12 +3,16 @@
 #include <algorithm>
 #include <atomic>
 #include <cstdlib>
+#include <exception>
 #include <limits>
 #include <mutex>
 #include <utility>
 #include <vector>
 
 namespace mops::amd {
+
+// (sender_buckets.hip: a launch that sets `count` integers to zero; usable while a stream is captured)
+void clear_counters(int32_t* counters, size_t count, hipStream_t stream);
 
 void check_hip(hipError_t status, const char* what) {
     if (status != hipSuccess) {
@@ -33,6 +37,11 @@ struct Resources {
     bool block_in_graph = false;        // handed out while a stream was being captured
     hipEvent_t last_use = nullptr;      // recorded behind the latest eager call that used the block
     bool last_use_recorded = false;
+    // The counters in front of the block were handed to a call that has not reached its end
+    // (finish_call) yet. Found set at the start of the next call, it means that a call failed
+    // between a launch that counts and the launch that reads and clears: the counters may hold
+    // anything and are cleared before they are handed out again.
+    bool counters_dirty = false;
     // blocks a captured graph may still name: kept until the process ends
     std::vector<void*> retired;
 
@@ -138,6 +147,16 @@ bool set_synchronous(bool value) {
     return previous;
 }
 
+namespace {
+void record_last_use(Resources& res, hipStream_t stream, const char* operation) {
+    if (res.last_use == nullptr) {
+        check_hip(hipEventCreateWithFlags(&res.last_use, hipEventDisableTiming), operation);
+    }
+    check_hip(hipEventRecord(res.last_use, stream), operation);
+    res.last_use_recorded = true;
+}
+} // namespace
+
 void finish_call(const char* operation) {
     check_hip(hipGetLastError(), operation);
     auto& st = state();
@@ -147,11 +166,7 @@ void finish_call(const char* operation) {
         st.used_scratch = false;
         Resources& res = st.res();
         if (!st.capturing) {
-            if (res.last_use == nullptr) {
-                check_hip(hipEventCreateWithFlags(&res.last_use, hipEventDisableTiming), operation);
-            }
-            check_hip(hipEventRecord(res.last_use, st.stream), operation);
-            res.last_use_recorded = true;
+            record_last_use(res, st.stream, operation);
         }
     }
     if (st.synchronous) {
@@ -298,6 +313,10 @@ void* scratch(size_t bytes) {
         MOPS_HIP_CHECK(hipMemsetAsync(res.block, 0, counter_bytes, st.stream));
         res.capacity = capacity;
         res.device = device;
+        res.counters_dirty = false;
+        // another stream that takes the block over waits for the clearing, also when this call
+        // fails before its end
+        record_last_use(res, st.stream, "scratch");
     } else if (res.block_stream != st.stream && res.last_use_recorded && !st.capturing) {
         // The previous user of the block ran on another stream: this stream
         // waits (on the device, not the host) for the event recorded behind
@@ -307,18 +326,52 @@ void* scratch(size_t bytes) {
         // ordering graph replays against eager calls is the caller's business.
         MOPS_HIP_CHECK(hipStreamWaitEvent(st.stream, res.last_use, 0));
     }
+    if (res.counters_dirty) {
+        // A call that had the counters did not reach its end: what it enqueued may have counted
+        // without the reader that clears. No event was recorded behind it, so when it ran on
+        // another stream the host waits for the device (this happens after a failure only).
+        if (!st.capturing && res.block_stream != st.stream) {
+            MOPS_HIP_CHECK(hipDeviceSynchronize());
+        }
+        clear_counters(static_cast<int32_t*>(res.block), SCRATCH_COUNTERS, st.stream);
+        // (a clearing that was only captured has not run: the next eager call still has to clear)
+        res.counters_dirty = st.capturing;
+    }
     res.block_stream = st.stream;
     res.block_in_graph = res.block_in_graph || st.capturing;
     st.used_scratch = true;
     return static_cast<char*>(res.block) + SCRATCH_COUNTERS * sizeof(int32_t);
 }
 
-int32_t* scratch_counters() {
+ScratchCounters::ScratchCounters() : exceptions_(std::uncaught_exceptions()) {
     auto& st = state();
     if (!st.used_scratch || st.resources == nullptr || st.resources->block == nullptr) {
-        throw std::runtime_error("mops: scratch_counters() without scratch() in the same call");
+        throw std::runtime_error("mops: ScratchCounters without scratch() in the same call");
     }
-    return static_cast<int32_t*>(st.resources->block);
+    resources_ = st.resources;
+    capturing_ = st.capturing;
+    before_ = st.resources->counters_dirty;
+    // until this object goes away in the ordinary way: a call that fails in between leaves the
+    // mark for the next one
+    st.resources->counters_dirty = true;
+}
+
+ScratchCounters::~ScratchCounters() {
+    if (std::uncaught_exceptions() > exceptions_) {
+        return; // the call is failing: what it enqueued may have counted without the reader
+    }
+    // Every launch of the call is enqueued, the readers that clear the counters included.
+    // (Captured launches have not run: the counters are as they were.)
+    static_cast<Resources*>(resources_)->counters_dirty = capturing_ ? before_ : false;
+}
+
+int32_t* ScratchCounters::data() const { return static_cast<int32_t*>(static_cast<Resources*>(resources_)->block); }
+
+void test_failure_point(const char* name) {
+    const char* wanted = std::getenv("MOPS_AMD_TEST_FAIL_AT");
+    if (wanted != nullptr && std::string(wanted) == name) {
+        throw std::runtime_error(std::string("mops: failure requested by MOPS_AMD_TEST_FAIL_AT at '") + name + "'");
+    }
 }
 
 size_t scratch_capacity() {

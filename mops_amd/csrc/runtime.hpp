@@ -54,8 +54,36 @@ size_t scratch_capacity();
 /// that counts in them sets what it has used back to zero before it ends, so
 /// that the next launch finds zeros without a launch that clears them (also
 /// the next replay of a graph the launches were captured into).
+/// A call that fails between a launch that counts and the launch that reads
+/// and clears would leave counts behind for the next call. The host keeps a
+/// mark per block for that: a call takes the counters by holding a
+/// ScratchCounters for as long as it enqueues work; the mark is set from the
+/// object's construction until its destruction in the ordinary way, and stays
+/// when the object is destroyed by an exception on its way out of the call.
+/// scratch() clears the counters with a launch of its own when it finds the
+/// mark. A graph that was captured earlier does not pass through scratch():
+/// after a failed call, make one eager call that succeeds
+/// (mops_amd_reserve_scratch(0) will do) before replaying it.
 constexpr size_t SCRATCH_COUNTERS = size_t(1) << 18;
-int32_t* scratch_counters();
+class ScratchCounters {
+public:
+    ScratchCounters();
+    ~ScratchCounters();
+    ScratchCounters(const ScratchCounters&) = delete;
+    ScratchCounters& operator=(const ScratchCounters&) = delete;
+    int32_t* data() const;
+
+private:
+    void* resources_ = nullptr;
+    int exceptions_;
+    bool capturing_ = false;
+    bool before_ = false;
+};
+
+/// Throws when the environment variable MOPS_AMD_TEST_FAIL_AT names `name`:
+/// lets a test make a call fail on the host between two of its launches (every
+/// kernel that was enqueued still runs to its end).
+void test_failure_point(const char* name);
 
 /// A second stream of the calling thread, for a kernel of a call that does not
 /// depend on the call's other kernels and leaves room on the device beside

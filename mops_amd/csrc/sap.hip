@@ -48,6 +48,7 @@
 #include "sap_mfma.hpp"
 
 namespace mops::amd {
+namespace sap { // a name of its own for this file's kernels: profilers print it
 namespace {
 
 constexpr int ROWS = WAVE;            // batch rows per workgroup (one per lane)
@@ -658,6 +659,8 @@ int pick_waves(size_t n_blocks, int32_t columns) {
 }
 
 } // namespace
+} // namespace sap
+using namespace sap;
 } // namespace mops::amd
 
 namespace mops::cuda {

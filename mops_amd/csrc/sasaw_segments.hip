@@ -1599,6 +1599,7 @@ void vjp(
             );
             args.slot_edges = lists.edges;
             args.slot_counts = lists.counts;
+            test_failure_point("sasaw_vjp_after_listing");
         } else {
             const SenderSlots slots = list_edges_in_slots(indices.W_1, s.n_edges, s.n_nodes, workspace, stream);
             args.slot_edges = slots.edges;

@@ -217,3 +217,29 @@ def test_a_block_that_a_graph_names_outlives_a_later_growth(device):
     for got, want in zip(captured, eager):
         assert torch.equal(got, want)
     del filler
+
+
+@pytest.mark.parametrize(
+    "op,point", [("opsaw_many_senders", "opsaw_vjp_after_listing"), ("sasaw_many_senders", "sasaw_vjp_after_listing")]
+)
+def test_a_call_that_fails_between_two_launches_does_not_spoil_the_next(device, monkeypatch, op, point):
+    """The senders' edges of large graphs are listed by a launch that counts in counters which the
+    launch that uses the lists sets back to zero. A call that fails on the host between the two
+    leaves counts behind; the library marks its counters on the host and clears them at the start
+    of the next call. The failure is requested from the host (MOPS_AMD_TEST_FAIL_AT): every
+    kernel that was enqueued runs to its end."""
+    from mops_amd.status import MopsError
+
+    case = support.to_device(CASES[op](np.float32), device)
+    good = [t.clone() for t in _call(op, case)]
+    torch.cuda.synchronize()
+    monkeypatch.setenv("MOPS_AMD_TEST_FAIL_AT", point)
+    with pytest.raises(MopsError, match="failure requested by MOPS_AMD_TEST_FAIL_AT"):
+        _call(op, case)
+    torch.cuda.synchronize()
+    monkeypatch.delenv("MOPS_AMD_TEST_FAIL_AT")
+    for attempt in range(2):
+        again = _call(op, case)
+        torch.cuda.synchronize()
+        for got, want in zip(again, good):
+            assert torch.equal(got, want), (op, attempt)
