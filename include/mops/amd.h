@@ -105,15 +105,24 @@ MOPS_EXPORT int64_t mops_amd_scratch_capacity(void);
  * temporaries of its kernels (the dense coupling table and the list of every
  * sender's edges) live in an array of 4 MiB that is part of the library's
  * device code, one copy per GPU, held until the process ends; the call makes
- * no hipMalloc / hipFree and creates no stream or event. Limits, reported as
- * status 1 with a message: A.shape[1], W.shape[1], output.shape[1] in 1..16;
- * temporaries within 4 MiB (about 7800 nodes); when grad_W is asked for
- * together with grad_A or grad_B, at most 48 edges per node on average and
- * W.shape[1], output.shape[1] in the same multiple of four; indices_output_1
- * sorted (mops_amd_accept_unsorted_indices does not apply). All calls on one
- * GPU share the array: calls that overlap on one GPU (two streams, two
+ * no hipMalloc / hipFree and creates no stream or event (kernel timing,
+ * mops_amd_kernel_timing, takes events from a pool that it fills on demand:
+ * it is off inside this call, whatever the thread's setting). Shapes whose
+ * sums are empty (no column, table entry, edge or node) give zero gradients,
+ * as there. Limits, reported as status 1 with a message: A.shape[1],
+ * W.shape[1], output.shape[1] at most 16; temporaries within 4 MiB (about
+ * 7800 nodes); when grad_W is asked for together with grad_A or grad_B, at
+ * most 48 edges per node on average and W.shape[1], output.shape[1] in the
+ * same multiple of four; no grad_W at all for graphs so large and dense that
+ * the edges are first sorted by sender; indices_output_1 sorted
+ * (mops_amd_accept_unsorted_indices does not apply). With
+ * MOPS_AMD_CHECK_INDICES=1 the indices are copied to the host and checked as
+ * in the existing entry point, which waits for the stream and allocates host
+ * memory: a debugging aid, not for a stream that is being captured. All calls
+ * on one GPU share the array: calls that overlap on one GPU (two streams, two
  * threads) race; the caller serialises them. Nothing in the array needs to be
- * zero at entry. Runs on the calling thread's stream (mops_amd_set_stream). */
+ * zero at entry. Runs on the calling thread's stream (mops_amd_set_stream);
+ * with mops_amd_set_synchronous(0) a call can be captured into a HIP graph. */
 MOPS_EXPORT int mops_amd_sparse_accumulation_scatter_add_with_weights_vjp_no_alloc_f32(
     mops_tensor_2d_f32_t grad_A,
     mops_tensor_2d_f32_t grad_B,

@@ -45,6 +45,7 @@
 // gradients) and, where those refuse (grad_W on graphs too dense for the
 // senders' slots, byte offsets beyond 32 bits), to sasaw_mfma.hip.
 #include <algorithm>
+#include <optional>
 #include <atomic>
 #include <stdexcept>
 #include <string>
@@ -57,12 +58,14 @@
 #include "index_validation.hpp"
 #include "no_alloc.hpp"
 #include "edge_order.hpp"
+#include "elementwise.hpp"
 #include "runtime.hpp"
 #include "sasaw_mfma.hpp"
 #include "sasaw_segments.hpp"
 #include "sender_buckets.hpp"
 
 namespace mops::amd {
+namespace sasaw { // a name of its own for this file's kernels: profilers print it
 namespace {
 
 constexpr int MAX_THREADS = 1024;
@@ -589,6 +592,8 @@ CouplingPlan<T> enqueue_plan(
 }
 
 } // namespace
+} // namespace sasaw
+using namespace sasaw;
 } // namespace mops::amd
 
 namespace mops::cuda {
@@ -756,7 +761,11 @@ void sparse_accumulation_scatter_add_with_weights_vjp(MOPS_SASAW_VJP_PARAMS(MOPS
         };
         const size_t bytes = sasaw_segments::vjp_workspace_bytes(shape, want_W);
         void* workspace = bytes > 0 ? scratch(bytes) : nullptr;
-        int32_t* counters = bytes > 0 ? scratch_counters() : nullptr;
+        std::optional<ScratchCounters> taken; // (until the end of this call, finish_call included)
+        if (bytes > 0) {
+            taken.emplace();
+        }
+        int32_t* counters = taken ? taken->data() : nullptr;
         sasaw_segments::vjp<scalar_t>(
             grad_A.data, grad_B.data, grad_W.data, grad_output.data, A.data, B.data, C.data, W.data, indices,
             shape, workspace, counters, true, stream
@@ -900,7 +909,36 @@ void sasaw_vjp_no_alloc(
     if (!want_edges && !want_W) {
         return;
     }
+    // (with MOPS_AMD_CHECK_INDICES=1 these copy the indices to the host and wait for the stream,
+    // as in the existing entry point: a debugging aid, not for a stream that is being captured)
+    validate_gather_index(indices_A, A.shape[1], "indices_A", operation);
+    validate_gather_index(indices_W_1, grad_output.shape[0], "indices_W_1", operation);
+    validate_gather_index(indices_W_2, W.shape[1], "indices_W_2", operation);
+    validate_scatter_index(indices_output_1, grad_output.shape[0], "indices_output_1", operation);
+    validate_gather_index(indices_output_2, grad_output.shape[1], "indices_output_2", operation);
+    // Kernel timing (mops_amd_kernel_timing) takes HIP events from a pool that it fills with
+    // hipEventCreate: not in a call that promises to create nothing. Off for the length of it.
+    struct TimingOff {
+        bool was = set_kernel_timing(false);
+        ~TimingOff() { set_kernel_timing(was); }
+    } timing_off;
     const Sizes s = sizes_of(grad_output, A, B, C, W);
+    hipStream_t stream = current_stream();
+    if (s.L == 0 || s.N == 0 || s.n_edges == 0 || s.n_nodes == 0 || s.nA == 0 || s.n2 == 0 || s.n3 == 0) {
+        // every sum is over nothing: the gradients that have elements are zero (as the existing
+        // entry point gives them)
+        if (grad_A.data != nullptr) {
+            fill_zero(grad_A.data, static_cast<size_t>(s.n_edges) * s.nA, stream);
+        }
+        if (grad_B.data != nullptr) {
+            fill_zero(grad_B.data, static_cast<size_t>(s.n_edges) * s.L, stream);
+        }
+        if (want_W) {
+            fill_zero(grad_W.data, static_cast<size_t>(s.n_nodes) * s.n2 * s.L, stream);
+        }
+        finish_call(operation);
+        return;
+    }
     const sasaw_mfma::Shape shape{s.n_nodes, s.n_edges, s.nA, s.L, s.N, s.n2, s.n3};
     const char* who = "mops_amd_sparse_accumulation_scatter_add_with_weights_vjp_no_alloc_f32: ";
     const sasaw_mfma::Indices indices{
@@ -923,7 +961,7 @@ void sasaw_vjp_no_alloc(
         char* const array = static_cast<char*>(no_alloc_scratch_of_current_device());
         sasaw_segments::vjp<float>(
             grad_A.data, grad_B.data, grad_W.data, grad_output.data, A.data, B.data, C.data, W.data, indices, shape,
-            array, reinterpret_cast<int32_t*>(array + places), false, current_stream()
+            array, reinterpret_cast<int32_t*>(array + places), false, stream
         );
         finish_call(operation);
         return;
@@ -933,6 +971,13 @@ void sasaw_vjp_no_alloc(
             std::string(who) + "only the shapes of the matrix-core kernels are served without allocation (at least "
             "one node, edge and table entry; A.shape[1], W.shape[1] and output.shape[1] between 1 and 16); use "
             "mops_cuda_sparse_accumulation_scatter_add_with_weights_vjp_f32"
+        );
+    }
+    if (want_W && sasaw_mfma::orders_edges_by_sender(shape, sizeof(float))) {
+        throw std::runtime_error(
+            std::string(who) + "for a graph of this size with more than 48 edges per node on average grad_W needs "
+            "the edges put in the order of their senders first, by a counting sort on a second stream, which this "
+            "entry point cannot create; use mops_cuda_sparse_accumulation_scatter_add_with_weights_vjp_f32"
         );
     }
     if (!sasaw_mfma::vjp_allocates_nothing(shape, sizeof(float), want_edges, want_W)) {
@@ -954,7 +999,7 @@ void sasaw_vjp_no_alloc(
     void* workspace = no_alloc_scratch_of_current_device();
     sasaw_mfma::vjp<float>(
         grad_A.data, grad_B.data, grad_W.data, grad_output.data, A.data, B.data, C.data, W.data, indices, shape,
-        workspace, current_stream()
+        workspace, stream
     );
     finish_call(operation);
 }

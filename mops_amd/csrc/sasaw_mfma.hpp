@@ -42,6 +42,11 @@ void forward(
     const Shape& shape, void* workspace, hipStream_t stream
 );
 
+/// Whether grad_W of this shape first puts the edges in the order of their
+/// senders by a counting sort (large graphs whose senders' edges overflow the
+/// slots).
+bool orders_edges_by_sender(const Shape& shape, size_t element_size);
+
 /// Whether vjp() for this shape and these wanted gradients only launches
 /// kernels on `stream` with `workspace` as their temporary memory: no second
 /// stream, no events, no allocation.
