@@ -59,6 +59,62 @@ def assert_close(actual, expected, dtype, what="", factor=1.0):
     assert error <= bound, f"{what}: relative error {error:.3e} above {bound:.1e}"
 
 
+def in_float64(case):
+    """The same (already rounded) inputs as float64 arrays."""
+    return {
+        key: value.astype(np.float64) if isinstance(value, np.ndarray) and value.dtype == np.float32 else value
+        for key, value in case.items()
+    }
+
+
+def magnitudes(case):
+    """``case`` in float64 with every floating-point value replaced by its absolute value: an
+    operation applied to it gives, element by element, the sum of the absolute values of the terms
+    whose signed sum the operation gives on ``case`` (every operation here is a sum of products)."""
+    return {
+        key: np.abs(value.astype(np.float64)) if isinstance(value, np.ndarray) and value.dtype.kind == "f" else value
+        for key, value in case.items()
+    }
+
+
+def calibrated_bar(dtype, exact, same_dtype=None, term_magnitudes=None):
+    """The bar a kernel's result is held to, and the reason as text.
+
+    The north star's bar (1e-5 / 1e-12, norm-wise) unless the sum itself is ill-conditioned, which
+    is MEASURED, never assumed:
+
+    * float32: ``same_dtype`` is the oracle run in float32 on the same inputs and ``exact`` the
+      oracle in float64. Where the oracle's own float32 error exceeds a quarter of 1e-5, no order
+      of summation does better than that error's scale, and the bar is four times it.
+    * float64: nothing more exact is at hand, so the conditioning is measured instead:
+      ``term_magnitudes`` is the operation applied to the absolute values (``magnitudes``), and
+      kappa = max(sum |terms|) / max|sum terms|. Rounding moves a sum by at least eps * sum|terms|
+      whatever the order, so the bar is max(1e-12, 8 eps kappa): 1e-12 up to kappa = 1100.
+    """
+    dtype = np.dtype(dtype)
+    base = TOLERANCE[dtype]
+    if dtype == np.float32 and same_dtype is not None:
+        own = relative_error(same_dtype, exact)
+        if 4.0 * own > base:
+            return 4.0 * own, f"4 x the float32 oracle's own error {own:.2e}"
+        return base, f"north star (float32 oracle's own error {own:.2e})"
+    if dtype == np.float64 and term_magnitudes is not None and np.size(exact):
+        scale = float(np.max(np.abs(exact)))
+        kappa = float(np.max(term_magnitudes)) / scale if scale > 0 else np.inf
+        widened = 8.0 * np.finfo(np.float64).eps * kappa
+        if widened > base:
+            return widened, f"8 eps kappa, kappa = {kappa:.3g}"
+        return base, f"north star (kappa = {kappa:.3g})"
+    return base, "north star"
+
+
+def assert_calibrated(actual, exact, dtype, what, same_dtype=None, term_magnitudes=None):
+    bar, reason = calibrated_bar(dtype, exact, same_dtype, term_magnitudes)
+    error = relative_error(actual, exact)
+    assert error <= bar, f"{what}: relative error {error:.3e} above {bar:.3e} ({reason})"
+    return error, bar, reason
+
+
 # --------------------------------------------------------------------------
 # input generators
 # --------------------------------------------------------------------------

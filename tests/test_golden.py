@@ -3,7 +3,8 @@
 The fixture's expected values come from dense float64 torch formulations and
 torch.autograd (tests/golden/make_golden.py), code that shares nothing with
 oracle/ or mops_amd/csrc. The inputs are exact in float32, so both precisions
-are checked against the same float64 answers.
+are checked against the same float64 answers, at the north star's bar (the
+oracle itself is within 0.02 of it on every fixture).
 """
 import os
 
@@ -57,15 +58,15 @@ def test_oracle_against_golden(oracle, name, dtype):
     op = name.split("/")[0]
     case = typed_case(name, dtype)
     expected = CASES[name]["out"]
-    assert_close(support.cpu_forward(oracle, op, case), expected["output"], dtype, f"{name} output", 4.0)
+    assert_close(support.cpu_forward(oracle, op, case), expected["output"], dtype, f"{name} output")
     gradients = support.cpu_vjp(oracle, op, case)
     for key in OPS[op].differentiable:
-        assert_close(gradients[key], expected["grad_" + key], dtype, f"{name} grad_{key}", 4.0)
+        assert_close(gradients[key], expected["grad_" + key], dtype, f"{name} grad_{key}")
     if op in support.SECOND_ORDER:
         second = support.cpu_vjp_vjp(oracle, op, case)
-        assert_close(second["grad_output"], expected["grad_grad_output"], dtype, f"{name} grad_grad_output", 8.0)
+        assert_close(second["grad_output"], expected["grad_grad_output"], dtype, f"{name} grad_grad_output")
         for key in OPS[op].differentiable:
-            assert_close(second[key], expected[f"grad_{key}_2"], dtype, f"{name} grad_{key}_2", 8.0)
+            assert_close(second[key], expected[f"grad_{key}_2"], dtype, f"{name} grad_{key}_2")
 
 
 @pytest.mark.gpu
@@ -76,14 +77,14 @@ def test_hip_against_golden(device, name, dtype):
     case = support.to_device(typed_case(name, dtype), device)
     expected = CASES[name]["out"]
     output = support.hip_forward(op, case).cpu().numpy()
-    assert_close(output, expected["output"], dtype, f"{name} output", 4.0)
+    assert_close(output, expected["output"], dtype, f"{name} output")
     gradients = support.hip_vjp(op, case)
     for key in OPS[op].differentiable:
-        assert_close(gradients[key].cpu().numpy(), expected["grad_" + key], dtype, f"{name} grad_{key}", 4.0)
+        assert_close(gradients[key].cpu().numpy(), expected["grad_" + key], dtype, f"{name} grad_{key}")
     if op in support.SECOND_ORDER:
         second = support.hip_vjp_vjp(op, case)
         assert_close(
-            second["grad_output"].cpu().numpy(), expected["grad_grad_output"], dtype, f"{name} grad_grad_output", 8.0
+            second["grad_output"].cpu().numpy(), expected["grad_grad_output"], dtype, f"{name} grad_grad_output"
         )
         for key in OPS[op].differentiable:
-            assert_close(second[key].cpu().numpy(), expected[f"grad_{key}_2"], dtype, f"{name} grad_{key}_2", 8.0)
+            assert_close(second[key].cpu().numpy(), expected[f"grad_{key}_2"], dtype, f"{name} grad_{key}_2")

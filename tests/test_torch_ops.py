@@ -129,7 +129,7 @@ def test_operator_second_derivatives(oracle, device, op):
     contracted = sum((on_device["grad_grad_" + n] * g).sum() for n, g in zip(spec.differentiable, gradients))
     second = torch.autograd.grad(contracted, [on_device["grad_output"]] + wanted)
     for name, value in zip(["grad_output"] + spec.differentiable, second):
-        support.assert_close(value.cpu().numpy(), expected[name], np.float64, f"{op} second order {name}", 2.0)
+        support.assert_close(value.cpu().numpy(), expected[name], np.float64, f"{op} second order {name}")
     assert torch.autograd.gradgradcheck(operator, arguments(op, on_device), fast_mode=True)
 
 
