@@ -640,7 +640,7 @@ void sparse_accumulation_scatter_add_with_weights(MOPS_SASAW_PARAMS(MOPS_CXX_FIR
     hipStream_t stream = current_stream();
 
     const sasaw_mfma::Shape shape{s.n_nodes, s.n_edges, s.nA, s.L, s.N, s.n2, s.n3};
-    if (sasaw_segments::supports(shape, sizeof(scalar_t))) {
+    if (sasaw_segments::supports_forward(shape, sizeof(scalar_t))) {
         const sasaw_mfma::Indices indices{
             indices_A.data, indices_W_1.data, indices_W_2.data, indices_output_1.data, indices_output_2.data
         };

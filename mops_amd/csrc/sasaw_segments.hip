@@ -111,6 +111,11 @@ struct Table {
     int32_t registers; // ceil(nA / 4)
     Layout layout;
     int32_t bucket; // BETA: accumulator tiles of the kernel (>= n_red)
+    // The part of the coupling table this launch works with: components m1_begin .. m1_begin + nA
+    // of A, block rows red_begin .. red_begin + n_red, rows out_begin .. out_begin + n_out of the
+    // result (all zero and the whole ranges for shapes that one launch covers). RESULT only:
+    // n_out may exceed 16; the rows of the result then come in blocks of 16.
+    int32_t m1_begin, red_begin, out_begin;
 
     __host__ __device__ int32_t steps3() const { return (n_out + 3) / 4; }
     __host__ __device__ int32_t slots() const {
@@ -120,9 +125,10 @@ struct Table {
         case Layout::BETA:
             return (registers * bucket + 3) / 4 * steps3() * WAVE;
         default:
-            return registers * n_red * WAVE;
+            return out_blocks() * registers * n_red * WAVE;
         }
     }
+    __host__ __device__ int32_t out_blocks() const { return (n_out + 15) / 16; }
 };
 
 /// Where D[o, c, m1] goes (all three inside their ranges).
@@ -139,7 +145,7 @@ template <typename T> __device__ __forceinline__ int32_t slot_in(const Table& t,
     default: {
         int q, r;
         place_of_component<T>(m1, t.registers, q, r);
-        return (r * t.n_red + c) * WAVE + 16 * q + o;
+        return (((o >> 4) * t.registers + r) * t.n_red + c) * WAVE + 16 * q + (o & 15);
     }
     }
 }
@@ -200,9 +206,9 @@ __device__ __forceinline__ void build_table(
 #pragma unroll
         for (int k = 0; k < ENTRIES_PER_LANE; k++) {
             const int32_t n = first + lane + k * WAVE;
-            const bool inside = n < t.N && in_bounds(mine.m1[k], t.nA) && in_bounds(mine.c[k], t.n_red) &&
-                                in_bounds(mine.o[k], t.n_out);
-            slot[k] = inside ? slot_in<T>(t, mine.m1[k], mine.c[k], mine.o[k]) : -1;
+            const int32_t m1 = mine.m1[k] - t.m1_begin, c = mine.c[k] - t.red_begin, o = mine.o[k] - t.out_begin;
+            const bool inside = n < t.N && in_bounds(m1, t.nA) && in_bounds(c, t.n_red) && in_bounds(o, t.n_out);
+            slot[k] = inside ? slot_in<T>(t, m1, c, o) : -1;
             pending |= inside ? 1u << k : 0u;
         }
         // Every round the smallest pending entry of each slot is added to it: the
@@ -248,6 +254,12 @@ template <typename T> struct Contraction {
     T* result;                   // [n_blocks][n_out][ld]
     int32_t n_edges, n_blocks, nA, L, ld, n_red, n_out;
     int32_t column_tiles; // ceil(L / 16): wavefronts per node
+    // A launch that works on a part of the tensors (NodeSum<.., GENERAL>): `A`, `rows` and `result`
+    // point to the first component / block row / row of the part, nA, n_red and n_out count the
+    // part, and these are the full extents the rows are apart by. `accumulate`: the launch adds
+    // to what `result` holds (another part of the sums over m1 and the block rows is there already).
+    int32_t lda, rows_stride, out_stride;
+    bool accumulate;
 };
 
 /// Edges whose operands a wavefront asks for together: STEPS steps of four.
@@ -341,7 +353,7 @@ __device__ __forceinline__ void load_four(
 
 /// What a wavefront keeps for one node. NB = accumulator tiles: the block rows
 /// n_red, or (EXACT false) a bucket above them.
-template <typename T, int NB, bool EXACT, bool COMPACT = false> struct NodeSum {
+template <typename T, int NB, bool EXACT, bool COMPACT = false, bool GENERAL = false> struct NodeSum {
     using M = Mfma<T>;
     static constexpr int STEPS = steps_in_flight<T>();
 
@@ -369,8 +381,10 @@ template <typename T, int NB, bool EXACT, bool COMPACT = false> struct NodeSum {
         : p(contraction), registers_of_A(registers) {
         set_column_tile(0);
         row_bytes = static_cast<uint32_t>(p.ld) * sizeof(T);
-        block_bytes = static_cast<uint32_t>(p.n_red) * row_bytes;
-        a_row_bytes = static_cast<uint32_t>(p.nA) * sizeof(T);
+        block_bytes = static_cast<uint32_t>(GENERAL ? p.rows_stride : p.n_red) * row_bytes;
+        a_row_bytes = static_cast<uint32_t>(GENERAL ? p.lda : p.nA) * sizeof(T);
+        // (GENERAL: the tensors begin up to a row before `A` and `rows`, so these limits lie up to a
+        // row behind their ends; no lane that is not masked asks for anything there)
         A.set(p.A, static_cast<uint32_t>(p.n_edges) * a_row_bytes);
         B.set(p.B, static_cast<uint32_t>(p.n_edges) * row_bytes);
         rows.set(p.rows, static_cast<uint32_t>(p.n_blocks) * block_bytes);
@@ -515,6 +529,21 @@ template <typename T, int NB, bool EXACT, bool COMPACT = false> struct NodeSum {
 
     /// result[node] = D * (the sums so far), this wavefront's 16 columns.
     __device__ __forceinline__ void finish(const T* __restrict__ table, int32_t registers, int32_t node) {
+        if constexpr (GENERAL) {
+            // the rows of the result in blocks of 16, each with its own part of the table
+            const int32_t blocks = (p.n_out + 15) / 16;
+            for (int32_t block = 0; block < blocks; block++) {
+                finish_block(table + static_cast<size_t>(block) * registers * p.n_red * WAVE, registers, node, 16 * block);
+            }
+        } else {
+            finish_block(table, registers, node, 0);
+        }
+    }
+
+    /// Rows first_row .. first_row + 16 of result[node].
+    __device__ __forceinline__ void finish_block(
+        const T* __restrict__ table, int32_t registers, int32_t node, int32_t first_row
+    ) {
         // result = D * sums, one block of NB table operands per register r of the
         // sums; four sums (double: two) take the products in turn, so that
         // consecutive matrix instructions do not wait for each other.
@@ -565,16 +594,23 @@ template <typename T, int NB, bool EXACT, bool COMPACT = false> struct NodeSum {
                 }
             }
         }
-        T* target = p.result + static_cast<size_t>(node) * p.n_out * p.ld + column;
+        T* target = p.result + static_cast<size_t>(node) * (GENERAL ? p.out_stride : p.n_out) * p.ld + column;
 #pragma unroll
         for (int r = 0; r < 4; r++) {
-            const int32_t row = M::row(lane, r);
+            const int32_t row = first_row + M::row(lane, r);
             if (row < p.n_out && column_inside) {
+                T value;
                 if constexpr (sizeof(T) == 4) {
-                    target[static_cast<size_t>(row) * p.ld] = (out[0][r] + out[1][r]) + (out[2][r] + out[3][r]);
+                    value = (out[0][r] + out[1][r]) + (out[2][r] + out[3][r]);
                 } else {
-                    target[static_cast<size_t>(row) * p.ld] = out[0][r] + out[1][r];
+                    value = out[0][r] + out[1][r];
                 }
+                if constexpr (GENERAL) {
+                    if (p.accumulate) { // (uniform)
+                        value += target[static_cast<size_t>(row) * p.ld];
+                    }
+                }
+                target[static_cast<size_t>(row) * p.ld] = value;
             }
         }
     }
@@ -582,6 +618,17 @@ template <typename T, int NB, bool EXACT, bool COMPACT = false> struct NodeSum {
     /// Rows of the result that no edge names.
     __device__ __forceinline__ void clear_rows(int32_t begin, int32_t end) const {
         if (!column_inside) {
+            return;
+        }
+        if constexpr (GENERAL) {
+            if (!p.accumulate) { // (the launch that adds finds the zeros of the one before it)
+                for (int32_t node = begin; node < end; node++) {
+                    T* target = p.result + static_cast<size_t>(node) * p.out_stride * p.ld + column;
+                    for (int32_t row = q; row < p.n_out; row += 4) {
+                        target[static_cast<size_t>(row) * p.ld] = T(0);
+                    }
+                }
+            }
             return;
         }
         const int32_t rows = (end - begin) * p.n_out;
@@ -723,7 +770,7 @@ struct UnitAhead {
 // global memory has to be cleared, and every wavefront leaves when the
 // counter has passed the workgroup's last unit. While a wavefront works on a
 // unit, the index values of its next unit are on their way.
-template <typename T, int NB, bool EXACT, int CHUNK>
+template <typename T, int NB, bool EXACT, int CHUNK, bool GENERAL = false>
 __global__ __launch_bounds__((group_threads<T, NB>())) void contract_kernel(const ContractArgs<T> args) {
     constexpr int THREADS = group_threads<T, NB>();
     constexpr int GROUP_WAVES = THREADS / WAVE;
@@ -739,7 +786,7 @@ __global__ __launch_bounds__((group_threads<T, NB>())) void contract_kernel(cons
     const int32_t wave = threadIdx.x >> 6;
     const int32_t group = static_cast<int32_t>(blockIdx.x);
     const int32_t n_groups = static_cast<int32_t>(gridDim.x);
-    NodeSum<T, NB, EXACT> sum(p, registers);
+    NodeSum<T, NB, EXACT, false, GENERAL> sum(p, registers);
     // Unit u is column tile u mod column_tiles of chunk u / column_tiles. The
     // column tiles of a chunk are consecutive turns of ONE workgroup (chunks
     // group, group + n_groups, ...): its wavefronts then ask for the same rows at
@@ -1207,6 +1254,10 @@ __global__ __launch_bounds__((gradient_group_threads<T, NB>())) void gradients_k
     contraction.n_red = args.n3;
     contraction.n_out = args.n2;
     contraction.column_tiles = args.column_tiles;
+    contraction.lda = args.nA;
+    contraction.rows_stride = args.n3;
+    contraction.out_stride = args.n2;
+    contraction.accumulate = false;
     NodeSum<T, NB, EXACT, true> sum(contraction, args.table_W.registers);
     EdgeGradients<T, NB, EXACT, VECTORS> edges(args);
 
@@ -1382,6 +1433,9 @@ Table table_of(const Shape& s, const int32_t* PA, const int32_t* Pred, const int
     t.registers = (s.nA + 3) / 4;
     t.layout = Layout::RESULT;
     t.bucket = n_red;
+    t.m1_begin = 0;
+    t.red_begin = 0;
+    t.out_begin = 0;
     return t;
 }
 
@@ -1431,14 +1485,14 @@ int32_t chunk_for(int32_t n_edges, int32_t column_tiles, int64_t resident_waves)
     return 64;
 }
 
-template <typename T> void launch_contract(ContractArgs<T> args, hipStream_t stream) {
+template <typename T> void launch_contract(ContractArgs<T> args, hipStream_t stream, bool general = false) {
     const Contraction<T>& p = args.contraction;
     const size_t lds = table_lds(args.table, sizeof(T));
     with_block_rows(p.n_red, [&](auto block_rows, auto exact) {
         constexpr int NB = decltype(block_rows)::value;
         constexpr bool EXACT = decltype(exact)::value;
         constexpr int64_t GROUP_WAVES = group_threads<T, NB>() / WAVE;
-        auto go = [&](auto chunk_constant) {
+        auto go = [&](auto chunk_constant, auto general_constant) {
             constexpr int CHUNK = decltype(chunk_constant)::value;
             const int64_t units = (static_cast<int64_t>(p.n_edges) + CHUNK - 1) / CHUNK * p.column_tiles;
             args.n_units = narrow_i32(static_cast<size_t>(units), "units of work");
@@ -1449,19 +1503,24 @@ template <typename T> void launch_contract(ContractArgs<T> args, hipStream_t str
             const unsigned grid = static_cast<unsigned>(
                 std::min<int64_t>(compute_units(), (chunks + chunks_per_round - 1) / chunks_per_round)
             );
-            auto kernel = contract_kernel<T, NB, EXACT, CHUNK>;
+            auto kernel = contract_kernel<T, NB, EXACT, CHUNK, decltype(general_constant)::value>;
             allow_lds(kernel, lds);
             kernel<<<grid, group_threads<T, NB>(), lds, stream>>>(args);
         };
+        if (general) {
+            // (parts of larger tensors: one size of chunk, the one of the shapes the kernel was tuned on)
+            go(std::integral_constant<int, 32>{}, std::true_type{});
+            return;
+        }
         switch (chunk_for(p.n_edges, p.column_tiles, GROUP_WAVES * compute_units())) {
         case 16:
-            go(std::integral_constant<int, 16>{});
+            go(std::integral_constant<int, 16>{}, std::false_type{});
             break;
         case 32:
-            go(std::integral_constant<int, 32>{});
+            go(std::integral_constant<int, 32>{}, std::false_type{});
             break;
         default:
-            go(std::integral_constant<int, 64>{});
+            go(std::integral_constant<int, 64>{}, std::false_type{});
             break;
         }
     });
@@ -1487,10 +1546,22 @@ Contraction<T> contraction_of(
     c.n_red = n_red;
     c.n_out = n_out;
     c.column_tiles = (s.L + 15) / 16;
+    c.lda = s.nA;
+    c.rows_stride = n_red;
+    c.out_stride = n_out;
+    c.accumulate = false;
     return c;
 }
 
 } // namespace
+
+static bool offsets_fit(const Shape& s, size_t element_size) {
+    // 32-bit byte offsets into every tensor
+    const uint64_t limit = uint64_t(1) << 32;
+    const uint64_t widest = static_cast<uint64_t>(std::max(std::max(s.n2, s.n3), 1)) * s.L * element_size;
+    return static_cast<uint64_t>(s.n_nodes) * widest < limit &&
+           static_cast<uint64_t>(s.n_edges) * std::max(s.nA, s.L) * element_size < limit;
+}
 
 bool supports(const Shape& s, size_t element_size) {
     if (s.n_nodes < 1 || s.n_edges < 1 || s.N < 1 || s.N > MAX_TABLE || s.L < 1) {
@@ -1499,11 +1570,35 @@ bool supports(const Shape& s, size_t element_size) {
     if (s.nA < 1 || s.nA > MAX_INDEX || s.n2 < 1 || s.n2 > MAX_INDEX || s.n3 < 1 || s.n3 > MAX_INDEX) {
         return false;
     }
-    // 32-bit byte offsets into every tensor
-    const uint64_t limit = uint64_t(1) << 32;
-    const uint64_t widest = static_cast<uint64_t>(std::max(std::max(s.n2, s.n3), 1)) * s.L * element_size;
-    return static_cast<uint64_t>(s.n_nodes) * widest < limit &&
-           static_cast<uint64_t>(s.n_edges) * std::max(s.nA, s.L) * element_size < limit;
+    return offsets_fit(s, element_size);
+}
+
+// More than 16 values of a component index (forward pass): the sums over m1 and over the block
+// rows are taken in parts of 16 each, a launch per pair of parts that adds to what the one before
+// left, and the rows of the result in blocks of 16 inside a launch, as many as the table in LDS
+// has room for (then the next launches). Every launch walks all edges again, so the parts are
+// limited: MAX_PARTS launches.
+constexpr int32_t MAX_PARTS = 64;
+constexpr size_t GENERAL_TABLE_LDS = 144 * 1024; // of the 160 KB of a compute unit
+
+/// Rows of the result per launch: whole blocks of 16, as many as fit the LDS with a table of
+/// 4 registers x 16 block rows per block.
+static int32_t result_rows_per_launch(const Shape& s, size_t element_size) {
+    const size_t per_block = static_cast<size_t>(4) * std::min(s.n2, MAX_INDEX) * WAVE * (element_size + sizeof(int32_t));
+    const int32_t blocks = static_cast<int32_t>(std::max<size_t>(1, (GENERAL_TABLE_LDS - 64) / per_block));
+    return 16 * std::min(blocks, (s.n3 + 15) / 16);
+}
+
+bool supports_forward(const Shape& s, size_t element_size) {
+    if (sasaw_segments::supports(s, element_size)) {
+        return true;
+    }
+    if (s.n_nodes < 1 || s.n_edges < 1 || s.N < 1 || s.N > MAX_TABLE || s.L < 1 || s.nA < 1 || s.n2 < 1 || s.n3 < 1) {
+        return false;
+    }
+    const int64_t parts = static_cast<int64_t>((s.nA + MAX_INDEX - 1) / MAX_INDEX) * ((s.n2 + MAX_INDEX - 1) / MAX_INDEX) *
+                          ((s.n3 + result_rows_per_launch(s, element_size) - 1) / result_rows_per_launch(s, element_size));
+    return parts <= MAX_PARTS && offsets_fit(s, element_size);
 }
 
 template <typename T>
@@ -1511,13 +1606,46 @@ void forward(
     T* output, const T* A, const T* B, const T* C, const T* W, const Indices& indices, const Shape& s,
     hipStream_t stream
 ) {
-    ContractArgs<T> args{};
-    args.contraction = contraction_of<T>(s, A, B, W, indices.W_1, output, s.n2, s.n3);
-    args.table = table_of(s, indices.A, indices.W_2, indices.output_2, s.n2, s.n3);
-    args.C = C;
-    args.sorted_index = indices.output_1;
     MainKernelTimer timer(stream);
-    launch_contract<T>(args, stream);
+    if (sasaw_segments::supports(s, sizeof(T))) {
+        ContractArgs<T> args{};
+        args.contraction = contraction_of<T>(s, A, B, W, indices.W_1, output, s.n2, s.n3);
+        args.table = table_of(s, indices.A, indices.W_2, indices.output_2, s.n2, s.n3);
+        args.C = C;
+        args.sorted_index = indices.output_1;
+        launch_contract<T>(args, stream);
+        return;
+    }
+    const int32_t rows_per_launch = result_rows_per_launch(s, sizeof(T));
+    for (int32_t out_begin = 0; out_begin < s.n3; out_begin += rows_per_launch) {
+        const int32_t n_out = std::min(rows_per_launch, s.n3 - out_begin);
+        bool first = true;
+        for (int32_t m1_begin = 0; m1_begin < s.nA; m1_begin += MAX_INDEX) {
+            const int32_t nA = std::min(MAX_INDEX, s.nA - m1_begin);
+            for (int32_t red_begin = 0; red_begin < s.n2; red_begin += MAX_INDEX) {
+                const int32_t n_red = std::min(MAX_INDEX, s.n2 - red_begin);
+                ContractArgs<T> args{};
+                Contraction<T>& c = args.contraction;
+                c = contraction_of<T>(s, A + m1_begin, B, W + static_cast<size_t>(red_begin) * s.L, indices.W_1,
+                                      output + static_cast<size_t>(out_begin) * s.L, n_red, n_out);
+                c.nA = nA;
+                c.lda = s.nA;
+                c.rows_stride = s.n2;
+                c.out_stride = s.n3;
+                c.accumulate = !first;
+                args.table = table_of(s, indices.A, indices.W_2, indices.output_2, n_red, n_out);
+                args.table.nA = nA;
+                args.table.registers = (nA + 3) / 4;
+                args.table.m1_begin = m1_begin;
+                args.table.red_begin = red_begin;
+                args.table.out_begin = out_begin;
+                args.C = C;
+                args.sorted_index = indices.output_1;
+                launch_contract<T>(args, stream, true);
+                first = false;
+            }
+        }
+    }
 }
 
 /// Whether the persistent gradient kernel serves this vjp: the senders' edges

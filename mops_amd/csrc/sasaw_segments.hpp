@@ -17,8 +17,12 @@ namespace mops::amd::sasaw_segments {
 using sasaw_mfma::Indices;
 using sasaw_mfma::Shape;
 
-/// Whether these kernels cover the shape for elements of `element_size` bytes.
+/// Whether these kernels cover the shape for elements of `element_size` bytes
+/// with one launch (at most 16 values of each component index).
 bool supports(const Shape& shape, size_t element_size);
+/// Whether forward() covers the shape: also more values of a component index,
+/// in several launches that take the index ranges in parts of 16.
+bool supports_forward(const Shape& shape, size_t element_size);
 
 template <typename T>
 void forward(

@@ -101,6 +101,12 @@ CASES = {
         "many_columns": lambda s, d: support.sasaw_case(s, d, E=500, nA=9, L=128, n_nodes=21, n2=9, n3=9, N=120, allow_empty=True),
         "ragged_columns": lambda s, d: support.sasaw_case(s, d, E=400, nA=4, L=70, n_nodes=17, n2=6, n3=11, N=80, allow_empty=True),
         "three_blocks": lambda s, d: support.sasaw_case(s, d, E=300, nA=16, L=164, n_nodes=40, n2=16, n3=16, N=300, allow_empty=True),
+        # more than 16 values of a component index: the forward pass takes the index ranges in parts.
+        # The shape of the reference's own benchmark (mops/benchmarks/sasaw.cpp:10-51: 13 x 7 x 100
+        # components, 900 entries, 60 edges per node), and 25 components each (spherical harmonics up to l = 4)
+        "hundred_output_rows": lambda s, d: support.sasaw_case(s, d, E=3000, nA=13, L=32, n_nodes=50, n2=7, n3=100, N=900),
+        "twenty_five_components": lambda s, d: support.sasaw_case(s, d, E=1500, nA=25, L=32, n_nodes=60, n2=25, n3=25, N=2000, allow_empty=True),
+        "ragged_parts": lambda s, d: support.sasaw_case(s, d, E=700, nA=17, L=20, n_nodes=31, n2=33, n3=40, N=700, allow_empty=True),
     },
 }  # fmt: skip
 
