@@ -55,7 +55,7 @@ constexpr int MAX_INNER_GROUPS_FORWARD = 4; // nB <= 16
 constexpr int MAX_INNER_GROUPS_VJP = 16;    // nO <= 64
 constexpr int MAX_OUTER = 16;
 constexpr int MAX_ENTRIES = 2048;
-constexpr size_t LDS_BUDGET = 128 * 1024; // of the 160 KB of a compute unit
+constexpr size_t LDS_BUDGET = 156 * 1024; // of the 160 KB of a compute unit (16 values of every index in double need 153 KB for the vjp)
 constexpr size_t LDS_WITHOUT_ASKING = 64 * 1024;
 
 __host__ __device__ constexpr size_t align16(size_t bytes) { return (bytes + 15) & ~static_cast<size_t>(15); }

@@ -932,9 +932,15 @@ template <typename T> struct GradientArgs {
     const int32_t* slot_edges;
     int32_t* slot_counts;
     bool by_arrival;
+    // A launch that works on a part of the index ranges (gradients_kernel<.., GENERAL>): A, W, G,
+    // grad_A and grad_W point to the first component / row of the part, nA, n2 and n3 count the
+    // part, and these are the full extents; a gradient whose flag is set is added to (another part
+    // of its sum is there already).
+    int32_t lda, w_stride_rows, g_stride_rows;
+    bool add_to_A, add_to_B, add_to_W;
 };
 
-template <typename T, int NB, bool EXACT, bool VECTORS> struct EdgeGradients {
+template <typename T, int NB, bool EXACT, bool VECTORS, bool GENERAL = false> struct EdgeGradients {
     using M = Mfma<T>;
     static constexpr uint32_t ELEMENT = sizeof(T);
 
@@ -951,9 +957,10 @@ template <typename T, int NB, bool EXACT, bool VECTORS> struct EdgeGradients {
         steps1 = (p.nA + 3) / 4;
         steps3_of_shape = (p.n3 + 3) / 4;
         row_bytes = static_cast<uint32_t>(p.L) * ELEMENT;
-        w_block_bytes = static_cast<uint32_t>(p.n2) * row_bytes;
-        g_block_bytes = static_cast<uint32_t>(p.n3) * row_bytes;
-        a_row_bytes = static_cast<uint32_t>(p.nA) * ELEMENT;
+        w_block_bytes = static_cast<uint32_t>(GENERAL ? p.w_stride_rows : p.n2) * row_bytes;
+        g_block_bytes = static_cast<uint32_t>(GENERAL ? p.g_stride_rows : p.n3) * row_bytes;
+        a_row_bytes = static_cast<uint32_t>(GENERAL ? p.lda : p.nA) * ELEMENT;
+        // (GENERAL: the limits lie up to a row behind the ends of the tensors, see NodeSum)
         A.set(p.A, static_cast<uint32_t>(p.n_edges) * a_row_bytes);
         B.set(p.B, static_cast<uint32_t>(p.n_edges) * row_bytes);
         W.set(p.W, static_cast<uint32_t>(p.n_nodes) * w_block_bytes);
@@ -1074,7 +1081,13 @@ template <typename T, int NB, bool EXACT, bool VECTORS> struct EdgeGradients {
 #pragma unroll
             for (int r = 0; r < 4; r++) {
                 if (row_edge[r] >= 0 && column_inside) {
-                    p.grad_B[static_cast<size_t>(row_edge[r]) * p.L + column] = result[r];
+                    T* target = p.grad_B + static_cast<size_t>(row_edge[r]) * p.L + column;
+                    if constexpr (GENERAL) {
+                        if (p.add_to_B) { // (uniform)
+                            result[r] += *target;
+                        }
+                    }
+                    *target = result[r];
                 }
             }
         }
@@ -1193,7 +1206,14 @@ template <typename T, int NB, bool EXACT, bool VECTORS> struct EdgeGradients {
                     for (int r = 0; r < 4; r++) {
                         const int32_t m1 = M::row(lane, r);
                         if (m1 < p.nA) {
-                            p.grad_A[static_cast<size_t>(my_edge[t]) * p.nA + m1] = sums[t][r];
+                            T* target = p.grad_A + static_cast<size_t>(my_edge[t]) * (GENERAL ? p.lda : p.nA) + m1;
+                            T value = sums[t][r];
+                            if constexpr (GENERAL) {
+                                if (p.add_to_A) { // (uniform)
+                                    value += *target;
+                                }
+                            }
+                            *target = value;
                         }
                     }
                 }
@@ -1217,7 +1237,7 @@ template <typename T, int NB> constexpr int gradient_group_threads() {
 
 /// EXACT: n2 = n3 = NB, no row of a block is padding (otherwise the block rows are
 /// compared with n2 / n3 as the loops go).
-template <typename T, int NB, bool EXACT, bool VECTORS, bool ARRIVALS>
+template <typename T, int NB, bool EXACT, bool VECTORS, bool ARRIVALS, bool GENERAL = false>
 __global__ __launch_bounds__((gradient_group_threads<T, NB>())) void gradients_kernel(const GradientArgs<T> args) {
     constexpr int THREADS = gradient_group_threads<T, NB>();
     constexpr int GROUP_WAVES = THREADS / WAVE;
@@ -1254,12 +1274,12 @@ __global__ __launch_bounds__((gradient_group_threads<T, NB>())) void gradients_k
     contraction.n_red = args.n3;
     contraction.n_out = args.n2;
     contraction.column_tiles = args.column_tiles;
-    contraction.lda = args.nA;
-    contraction.rows_stride = args.n3;
-    contraction.out_stride = args.n2;
-    contraction.accumulate = false;
-    NodeSum<T, NB, EXACT, true> sum(contraction, args.table_W.registers);
-    EdgeGradients<T, NB, EXACT, VECTORS> edges(args);
+    contraction.lda = GENERAL ? args.lda : args.nA;
+    contraction.rows_stride = GENERAL ? args.g_stride_rows : args.n3;
+    contraction.out_stride = GENERAL ? args.w_stride_rows : args.n2;
+    contraction.accumulate = GENERAL && args.add_to_W;
+    NodeSum<T, NB, EXACT, true, GENERAL> sum(contraction, args.table_W.registers);
+    EdgeGradients<T, NB, EXACT, VECTORS, GENERAL> edges(args);
 
     // Turn k of this workgroup is unit group + k * n_groups: the roles of a chunk
     // go to neighbouring workgroups. (Giving them to the wavefronts of one
@@ -1661,10 +1681,20 @@ static bool lists_by_arrival(const Shape& s) {
 }
 
 bool vjp_supported(const Shape& s, size_t element_size, bool want_grad_W) {
-    if (!sasaw_segments::supports(s, element_size)) {
+    if (sasaw_segments::supports(s, element_size)) {
+        return !want_grad_W || static_cast<size_t>(s.n_edges) <= static_cast<size_t>(s.n_nodes) * 48;
+    }
+    // more than 16 values of a component index: in parts (see vjp), every launch with the lists in
+    // slots (a sender with more than 32 edges in a quarter of the index is served by a wavefront
+    // that reads the whole index: rare up to 64 edges per node on average)
+    if (s.n_nodes < 1 || s.n_edges < 1 || s.N < 1 || s.N > MAX_TABLE || s.L < 1 || s.nA < 1 || s.n2 < 1 || s.n3 < 1) {
         return false;
     }
-    return !want_grad_W || static_cast<size_t>(s.n_edges) <= static_cast<size_t>(s.n_nodes) * 48;
+    constexpr int32_t ROWS = 9; // (GRADIENT_PART_ROWS)
+    const int64_t parts =
+        static_cast<int64_t>((s.nA + MAX_INDEX - 1) / MAX_INDEX) * ((s.n2 + ROWS - 1) / ROWS) * ((s.n3 + ROWS - 1) / ROWS);
+    return parts <= MAX_PARTS && offsets_fit(s, element_size) &&
+           (!want_grad_W || static_cast<size_t>(s.n_edges) <= static_cast<size_t>(s.n_nodes) * 64);
 }
 
 size_t vjp_workspace_bytes(const Shape& s, bool want_grad_W) {
@@ -1691,62 +1721,57 @@ int32_t edge_chunk_for(int32_t n_edges, int32_t edge_roles, int64_t wanted_units
     return 16;
 }
 
+/// Block rows (of W and of grad_output) per launch of the gradient kernel when the index ranges
+/// are taken in parts: the kernel with 9 accumulator tiles does a row in less than half the time
+/// of the one with 16 (measured on 13 x 7 x 100 components, 60 000 edges, float: 16 rows 222 us,
+/// 9 rows 60 us per launch; in double the 16-tile kernel spills and is four times slower still).
+constexpr int32_t GRADIENT_PART_ROWS = 9;
+
+/// The index ranges one launch of the gradient kernel works on.
+struct Part {
+    int32_t m1_begin, nA, m2_begin, n2, m3_begin, n3;
+};
+
+/// One launch of gradients_kernel for `part` of the shape `s`. `args` holds the tensors (already
+/// pointing to the part), the lists of the senders' edges and the flags; `general`: the part is
+/// not the whole shape (strides and offsets apply).
 template <typename T>
-void vjp(
-    T* grad_A, T* grad_B, T* grad_W, const T* grad_output, const T* A, const T* B, const T* C, const T* W,
-    const Indices& indices, const Shape& s, void* workspace, int32_t* counters, bool counters_are_zero,
-    hipStream_t stream
+void launch_gradients(
+    GradientArgs<T> args, const Shape& s, const Part& part, const Indices& indices, bool general, hipStream_t stream
 ) {
-    GradientArgs<T> args{};
-    args.A = A;
-    args.B = B;
-    args.W = W;
-    args.G = grad_output;
-    args.C = C;
-    args.grad_A = grad_A;
-    args.grad_B = grad_B;
-    args.grad_W = grad_W;
-    args.receivers = indices.output_1;
-    args.senders = indices.W_1;
     args.n_edges = s.n_edges;
     args.n_nodes = s.n_nodes;
-    args.nA = s.nA;
+    args.nA = part.nA;
     args.L = s.L;
-    args.n2 = s.n2;
-    args.n3 = s.n3;
+    args.n2 = part.n2;
+    args.n3 = part.n3;
     args.column_tiles = (s.L + 15) / 16;
-    if (grad_W != nullptr) {
-        // the edges of every sender, listed by a launch of its own in front
-        args.by_arrival = lists_by_arrival(s);
-        if (args.by_arrival) {
-            if (!counters_are_zero) {
-                clear_counters(counters, vjp_counters(s, true), stream);
-            }
-            const SenderArrivals lists = list_edges_by_arrival(
-                indices.W_1, s.n_edges, s.n_nodes, args.column_tiles, workspace, counters, stream
-            );
-            args.slot_edges = lists.edges;
-            args.slot_counts = lists.counts;
-            test_failure_point("sasaw_vjp_after_listing");
-        } else {
-            const SenderSlots slots = list_edges_in_slots(indices.W_1, s.n_edges, s.n_nodes, workspace, stream);
-            args.slot_edges = slots.edges;
-            args.slot_counts = const_cast<int32_t*>(slots.counts);
-        }
-    }
-    args.edge_roles = (grad_A != nullptr ? 1 : 0) + (grad_B != nullptr ? args.column_tiles : 0);
-    const int64_t W_units = grad_W != nullptr ? static_cast<int64_t>(s.n_nodes) * args.column_tiles : 0;
+    args.edge_roles = (args.grad_A != nullptr ? 1 : 0) + (args.grad_B != nullptr ? args.column_tiles : 0);
+    const int64_t W_units = args.grad_W != nullptr ? static_cast<int64_t>(s.n_nodes) * args.column_tiles : 0;
     args.n_W_units = narrow_i32(static_cast<size_t>(W_units), "units of work");
     // (rows of B and W are read 16 bytes at a time where their alignment allows)
-    const bool vectors =
-        s.L % 4 == 0 && reinterpret_cast<uintptr_t>(B) % 16 == 0 && reinterpret_cast<uintptr_t>(W) % 16 == 0;
-    MainKernelTimer timer(stream);
+    const bool vectors = s.L % 4 == 0 && reinterpret_cast<uintptr_t>(args.B) % 16 == 0 &&
+                         reinterpret_cast<uintptr_t>(args.W) % 16 == 0;
+    Shape of_part = s;
+    of_part.nA = part.nA;
+    of_part.n2 = part.n2;
+    of_part.n3 = part.n3;
+    auto with_offsets = [&](Table table, int32_t red_begin, int32_t out_begin) {
+        table.m1_begin = part.m1_begin;
+        table.red_begin = red_begin;
+        table.out_begin = out_begin;
+        return table;
+    };
 
-    with_block_rows(std::max(s.n2, s.n3), [&](auto block_rows, auto fits) {
+    with_block_rows(std::max(part.n2, part.n3), [&](auto block_rows, auto fits) {
         constexpr int NB = decltype(block_rows)::value;
         // grad_W sums over the rows of grad_output (n3 of them), the others over those of W (n2)
-        args.table_W = table_of(s, indices.A, indices.output_2, indices.W_2, s.n3, s.n2);
-        args.table_alpha = table_of(s, indices.A, indices.W_2, indices.output_2, s.n2, s.n3);
+        args.table_W = with_offsets(
+            table_of(of_part, indices.A, indices.output_2, indices.W_2, part.n3, part.n2), part.m3_begin, part.m2_begin
+        );
+        args.table_alpha = with_offsets(
+            table_of(of_part, indices.A, indices.W_2, indices.output_2, part.n2, part.n3), part.m2_begin, part.m3_begin
+        );
         args.table_alpha.layout = Layout::ALPHA;
         args.table_beta = args.table_alpha;
         args.table_beta.layout = Layout::BETA;
@@ -1765,25 +1790,111 @@ void vjp(
         const unsigned grid =
             static_cast<unsigned>(std::min<int64_t>(compute_units(), (units + GROUP_WAVES - 1) / GROUP_WAVES));
         (void)fits;
-        auto launch = [&](auto exact, auto with_vectors) {
-            auto kernel = args.by_arrival
-                              ? gradients_kernel<T, NB, decltype(exact)::value, decltype(with_vectors)::value, true>
-                              : gradients_kernel<T, NB, decltype(exact)::value, decltype(with_vectors)::value, false>;
+        auto launch = [&](auto exact, auto with_vectors, auto arrivals, auto is_general) {
+            auto kernel = gradients_kernel<
+                T, NB, decltype(exact)::value, decltype(with_vectors)::value, decltype(arrivals)::value,
+                decltype(is_general)::value>;
             allow_lds(kernel, lds);
             kernel<<<grid, gradient_group_threads<T, NB>(), lds, stream>>>(args);
         };
-        const bool exact = s.n2 == NB && s.n3 == NB;
+        const bool exact = part.n2 == NB && part.n3 == NB;
+        if (general) {
+            // (parts of larger index ranges: lists in slots only, one variant for rows with and without padding)
+            if (vectors) {
+                launch(std::false_type{}, std::true_type{}, std::false_type{}, std::true_type{});
+            } else {
+                launch(std::false_type{}, std::false_type{}, std::false_type{}, std::true_type{});
+            }
+            return;
+        }
+        auto with_lists = [&](auto is_exact, auto with_vectors) {
+            if (args.by_arrival) {
+                launch(is_exact, with_vectors, std::true_type{}, std::false_type{});
+            } else {
+                launch(is_exact, with_vectors, std::false_type{}, std::false_type{});
+            }
+        };
         if (exact && vectors) {
-            launch(std::true_type{}, std::true_type{});
+            with_lists(std::true_type{}, std::true_type{});
         } else if (exact) {
-            launch(std::true_type{}, std::false_type{});
+            with_lists(std::true_type{}, std::false_type{});
         } else if (vectors) {
-            launch(std::false_type{}, std::true_type{});
+            with_lists(std::false_type{}, std::true_type{});
         } else {
-            launch(std::false_type{}, std::false_type{});
+            with_lists(std::false_type{}, std::false_type{});
         }
     });
     MOPS_HIP_CHECK(hipGetLastError());
+}
+
+template <typename T>
+void vjp(
+    T* grad_A, T* grad_B, T* grad_W, const T* grad_output, const T* A, const T* B, const T* C, const T* W,
+    const Indices& indices, const Shape& s, void* workspace, int32_t* counters, bool counters_are_zero,
+    hipStream_t stream
+) {
+    GradientArgs<T> args{};
+    args.A = A;
+    args.B = B;
+    args.W = W;
+    args.G = grad_output;
+    args.C = C;
+    args.grad_A = grad_A;
+    args.grad_B = grad_B;
+    args.grad_W = grad_W;
+    args.receivers = indices.output_1;
+    args.senders = indices.W_1;
+    args.lda = s.nA;
+    args.w_stride_rows = s.n2;
+    args.g_stride_rows = s.n3;
+    const bool whole = sasaw_segments::supports(s, sizeof(T));
+    if (grad_W != nullptr) {
+        // the edges of every sender, listed by a launch of its own in front
+        args.by_arrival = whole && lists_by_arrival(s);
+        if (args.by_arrival) {
+            if (!counters_are_zero) {
+                clear_counters(counters, vjp_counters(s, true), stream);
+            }
+            const SenderArrivals lists = list_edges_by_arrival(
+                indices.W_1, s.n_edges, s.n_nodes, (s.L + 15) / 16, workspace, counters, stream
+            );
+            args.slot_edges = lists.edges;
+            args.slot_counts = lists.counts;
+            test_failure_point("sasaw_vjp_after_listing");
+        } else {
+            const SenderSlots slots = list_edges_in_slots(indices.W_1, s.n_edges, s.n_nodes, workspace, stream);
+            args.slot_edges = slots.edges;
+            args.slot_counts = const_cast<int32_t*>(slots.counts);
+        }
+    }
+    MainKernelTimer timer(stream);
+    if (whole) {
+        launch_gradients<T>(args, s, Part{0, s.nA, 0, s.n2, 0, s.n3}, indices, false, stream);
+        return;
+    }
+    // More than 16 values of a component index: the ranges in parts, a launch per triple of
+    // parts; a gradient is a sum over the parts of the two ranges it does not have as an index
+    // (grad_B: of all three), so all launches but the first of such a sum add to what is there.
+    for (int32_t m1_begin = 0; m1_begin < s.nA; m1_begin += MAX_INDEX) {
+        for (int32_t m2_begin = 0; m2_begin < s.n2; m2_begin += GRADIENT_PART_ROWS) {
+            for (int32_t m3_begin = 0; m3_begin < s.n3; m3_begin += GRADIENT_PART_ROWS) {
+                const Part part{
+                    m1_begin, std::min(MAX_INDEX, s.nA - m1_begin), m2_begin,
+                    std::min(GRADIENT_PART_ROWS, s.n2 - m2_begin), m3_begin,
+                    std::min(GRADIENT_PART_ROWS, s.n3 - m3_begin)};
+                GradientArgs<T> of_part = args;
+                of_part.A = A + m1_begin;
+                of_part.W = W + static_cast<size_t>(m2_begin) * s.L;
+                of_part.G = grad_output + static_cast<size_t>(m3_begin) * s.L;
+                of_part.grad_A = grad_A != nullptr ? grad_A + m1_begin : nullptr;
+                of_part.grad_W = grad_W != nullptr ? grad_W + static_cast<size_t>(m2_begin) * s.L : nullptr;
+                of_part.add_to_A = m2_begin > 0 || m3_begin > 0;
+                of_part.add_to_B = m1_begin > 0 || m2_begin > 0 || m3_begin > 0;
+                of_part.add_to_W = m1_begin > 0 || m3_begin > 0;
+                launch_gradients<T>(of_part, s, part, indices, true, stream);
+            }
+        }
+    }
 }
 
 template void forward<float>(

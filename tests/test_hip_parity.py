@@ -281,6 +281,20 @@ def test_vjp_subsets_of_gradients(oracle, device, op):
                     assert partial[key] is None
 
 
+def test_sasaw_in_parts_subsets_of_gradients(device):
+    """The same where the index ranges are taken in parts (launches that add to each other's results)."""
+    case = CASES["sasaw"]["ragged_parts"](304, np.float64)
+    on_device = to_device(case, device)
+    full = hip_vjp("sasaw", on_device)
+    for wanted in (["A"], ["B"], ["W"], ["A", "W"], ["B", "W"]):
+        partial = hip_vjp("sasaw", on_device, wanted=wanted)
+        for key in ("A", "B", "W"):
+            if key in wanted:
+                assert np.array_equal(partial[key].cpu().numpy(), full[key].cpu().numpy()), (wanted, key)
+            else:
+                assert partial[key] is None
+
+
 @pytest.mark.parametrize("dtype", DTYPES, ids=["f32", "f64"])
 def test_sap_many_rows_subsets_of_gradients(device, dtype):
     """The same for the SAP kernels whose wavefronts walk over the rows (300 000 rows and more)."""
