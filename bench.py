@@ -79,12 +79,12 @@ MAIN_KERNELS = {
     ("opsaw", "forward"): "opsa::forward_kernel<{T}, 2, true, true>",
     ("opsaw", "vjp"): "opsa::edge_rows_vjp_kernel<{T}, 1, 2, true, true, false, true>",
     ("sasaw", "forward"): {
-        "float": "sasaw_segments::contract_kernel<float, 9, true, 32>",
-        "double": "sasaw_segments::contract_kernel<double, 9, true, 64>",
+        "float": "sasaw_segments::contract_kernel<float, 9, true, 32, false>",
+        "double": "sasaw_segments::contract_kernel<double, 9, true, 64, false>",
     },
     ("sasaw", "vjp"): {
-        "float": "sasaw_segments::gradients_kernel<float, 9, true, true, false>",
-        "double": "sasaw_segments::gradients_kernel<double, 9, true, true, false>",
+        "float": "sasaw_segments::gradients_kernel<float, 9, true, true, false, false>",
+        "double": "sasaw_segments::gradients_kernel<double, 9, true, true, false, false>",
     },
 }
 
@@ -506,8 +506,8 @@ def main():
     )
     parser.add_argument(
         "--profile-scaled", action="store_true",
-        help="with --profile: also 10 eager forward+vjp calls at the scaled shapes (per_op_scaled), each followed "
-        "by the flat copy of the same number of bytes",
+        help="with --profile: the scaled shapes (per_op_scaled) instead of the BASELINE ones, 10 eager forward+vjp "
+        "calls each, every call followed by the flat copy of the same number of bytes",
     )  # fmt: skip
     parser.add_argument("--repetitions", type=int, default=25, help="how often the region of --steps steps is timed")
     parser.add_argument("--no-scaled", action="store_true", help="leave per_op_scaled out")
@@ -537,7 +537,7 @@ def main():
     baseline = [c for c in configs if c[0].startswith("c")]
 
     if args.profile:
-        for config, op_name, _, op_case in baseline:
+        for config, op_name, _, op_case in [] if args.profile_scaled else baseline:
             if args.profile in (op_name, "all"):
                 w = DeviceWorkload(op_name, op_case, device)
                 for _ in range(50):
