@@ -1675,14 +1675,24 @@ void forward(
 /// index, which costs edges x nodes). Measured at 30 edges per node, whole vjp
 /// in float, by arrival / in slots: 2000 nodes 66.7 / 60.7 us, 3000: 93.8 /
 /// 92.8, 4000: 113.7 / 114.0, 6000: 170 / 179, 8000: 233 / 255, 20 000: 682 /
-/// 820 (double alike).
+/// 820 (double alike). Graphs with 48 to 64 edges per node on average overflow the
+/// slots (32 places per quarter of the index) but not the 128 places of a
+/// sender's list by arrival: 1000 nodes with 60 edges each, whole vjp by arrival
+/// against the older kernels of sasaw_mfma.hip: 76.6 / 87.6 us (float), 115.3 /
+/// 143.8 (double); with 100 edges each the lists overflow too (375 / 101 us).
+static bool dense_for_slots(const Shape& s) {
+    return static_cast<size_t>(s.n_edges) > static_cast<size_t>(s.n_nodes) * 48;
+}
 static bool lists_by_arrival(const Shape& s) {
-    return s.n_nodes > 4000 && static_cast<size_t>(s.n_nodes) * ((s.L + 15) / 16) <= SCRATCH_COUNTERS;
+    return (s.n_nodes > 4000 || dense_for_slots(s)) &&
+           static_cast<size_t>(s.n_nodes) * ((s.L + 15) / 16) <= SCRATCH_COUNTERS;
 }
 
 bool vjp_supported(const Shape& s, size_t element_size, bool want_grad_W) {
     if (sasaw_segments::supports(s, element_size)) {
-        return !want_grad_W || static_cast<size_t>(s.n_edges) <= static_cast<size_t>(s.n_nodes) * 48;
+        // (more than 48 edges per node on average: only by arrival, see lists_by_arrival)
+        return !want_grad_W || !dense_for_slots(s) ||
+               (static_cast<size_t>(s.n_edges) <= static_cast<size_t>(s.n_nodes) * 64 && lists_by_arrival(s));
     }
     // more than 16 values of a component index: in parts (see vjp), every launch with the lists in
     // slots (a sender with more than 32 edges in a quarter of the index is served by a wavefront

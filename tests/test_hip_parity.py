@@ -98,6 +98,8 @@ CASES = {
             "indices_W_1", SENDER_COUNTS
         ),
         "forty_five_per_sender": lambda s, d: support.sasaw_case(s, d, E=2250, nA=4, L=16, n_nodes=50, n2=4, n3=3, N=30),
+        # (48 to 64 edges per sender on average: too many for the slots, listed by arrival)
+        "sixty_per_sender": lambda s, d: support.sasaw_case(s, d, E=3000, nA=4, L=16, n_nodes=50, n2=4, n3=3, N=30),
         "many_columns": lambda s, d: support.sasaw_case(s, d, E=500, nA=9, L=128, n_nodes=21, n2=9, n3=9, N=120, allow_empty=True),
         "ragged_columns": lambda s, d: support.sasaw_case(s, d, E=400, nA=4, L=70, n_nodes=17, n2=6, n3=11, N=80, allow_empty=True),
         "three_blocks": lambda s, d: support.sasaw_case(s, d, E=300, nA=16, L=164, n_nodes=40, n2=16, n3=16, N=300, allow_empty=True),
