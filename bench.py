@@ -32,6 +32,9 @@ factored count, see ``useful_flops``) with ``flop_frac`` = flops / device time
 or edges of the BASELINE shapes: sizes at which a launch lasts long enough to
 be bound by bandwidth or arithmetic rather than by latency.
 
+``per_op_second_order`` times the vjp_vjp functions (HPE, SAP, OPSA) at the
+BASELINE shapes; they are not part of a step.
+
 ``roofline`` is the kernel with the most time in a step; ``roofline_per_op``
 lists the main kernel of every call. Their durations come from pairs of HIP
 events that the library puts around that kernel on the stream it launches it on
@@ -701,6 +704,48 @@ def main():
             del w, op_case
             torch.cuda.empty_cache()
 
+    # ---------------- second-order functions (not part of the step; not tuned) ----------------
+    per_op_second_order = []
+    if not args.no_per_op:
+        for config, op_name, op_dtype, op_case in baseline:
+            if op_name not in support.SECOND_ORDER:
+                continue
+            case = support.add_cotangents(dict(op_case), op_name)
+            on_device = support.to_device(case, device)
+            spec = support.OPS[op_name]
+            outputs, arguments = support._vjp_vjp_arguments(
+                spec, on_device, None, None, lambda x: torch.empty_like(x)
+            )
+
+            def second_order(arguments=arguments, spec=spec):
+                library.call(spec.function + "_vjp_vjp", *arguments)
+
+            # (eager: these functions take a temporary from the stream's memory pool, which a
+            # capture would turn into nodes of the graph)
+            for _ in range(3):
+                second_order()
+            torch.cuda.synchronize()
+            start = torch.cuda.Event(enable_timing=True)
+            stop = torch.cuda.Event(enable_timing=True)
+            start.record()
+            for _ in range(50):
+                second_order()
+            stop.record()
+            torch.cuda.synchronize()
+            seconds, captured = start.elapsed_time(stop) * 1e-3 / 50, False
+            per_op_second_order.append(
+                {
+                    "config": config,
+                    "op": op_name,
+                    "dtype": np.dtype(op_dtype).name,
+                    "function": "vjp_vjp",
+                    "device_us": round(seconds * 1e6, 3),
+                    "timed": ("hip-graph replay" if captured else "eager launches") + ", HIP events, the same buffers every call",
+                }
+            )
+            del on_device, outputs, arguments
+        torch.cuda.empty_cache()
+
     # ---------------- roofline of the kernel with the most time in a step -------------------
     if roofline_per_op:
         dominant = max(roofline_per_op, key=lambda e: e["avg_us"])
@@ -813,6 +858,7 @@ def main():
         "roofline_per_op": roofline_per_op,
         "per_op": per_op,
         "per_op_scaled": per_op_scaled,
+        "per_op_second_order": per_op_second_order,
         "device": torch.cuda.get_device_name(0),
     }
     print(json.dumps(result))
