@@ -1021,6 +1021,239 @@ __global__ __launch_bounds__(WAVE) void vjp_vjp_kernel(
     }
 }
 
+// ---------------------------------------------------------------------------
+// Second order with the order known at compile time. Layout and division of
+// labour of vjp_ordered_kernel (the first wavefront walks the monomials, the
+// others help to stage, clear and add up), with a tile of grad_grad_A beside
+// the tile of A. A monomial costs O(K) instead of O(K^3): with a = A[i, P[j, .]]
+// and g = grad_grad_A[i, P[j, .]], the sums above are the derivative of the
+// product of the a's along g and that derivative's gradient,
+//
+//   S      = sum_f g[f] prod_{k != f} a[k]              (into grad_grad_output)
+//   D[f2]  = sum_{f != f2} g[f] prod_{k != f, f2} a[k]   (into grad_A_2, times gO)
+//
+// and both come from products of the factors before and after a position that
+// carry their own derivative along g:  p' = p a,  dp' = dp a + p g.
+// Then D[f2] = dp[f2] s[f2] + p[f2] ds[f2] and S = dp[K].
+// LDS: a[nA + 1][R] gg[nA + 1][R] accumulator[G][nA + 1][R]
+// ---------------------------------------------------------------------------
+template <typename T, int ORDER>
+__global__ __launch_bounds__(ORDERED_VJP_THREADS) void vjp_vjp_ordered_kernel(
+    T* __restrict__ grad_grad_output,
+    T* __restrict__ grad_A_2,
+    const T* __restrict__ grad_grad_A,
+    const T* __restrict__ grad_output,
+    const T* __restrict__ A,
+    const T* __restrict__ C,
+    const int32_t* __restrict__ P,
+    int32_t n_rows,
+    int32_t nA,
+    int32_t n_monomials,
+    int32_t log2_R
+) {
+    extern __shared__ __align__(16) unsigned char lds_bytes[];
+    const int32_t R = 1 << log2_R;
+    T* a_stage = reinterpret_cast<T*>(lds_bytes);
+    T* gg_stage = a_stage + static_cast<size_t>(nA + 1) * R;
+    T* accumulator = gg_stage + static_cast<size_t>(nA + 1) * R;
+    const bool want_O = grad_grad_output != nullptr;
+    const bool want_A = grad_A_2 != nullptr;
+
+    const int tid = threadIdx.x;
+    const bool walks = tid < WAVE;
+    const int G = WAVE >> log2_R;
+    const int r = tid & (R - 1);
+    const int g = (tid & (WAVE - 1)) >> log2_R;
+    const int32_t row0 = blockIdx.x * R;
+    const int32_t rows = min(R, n_rows - row0);
+
+    struct Monomial {
+        int32_t factor[ORDER];
+        T coefficient;
+    };
+    auto fetch = [&](Monomial& to, int32_t j) {
+        const int32_t safe = min(j, n_monomials - 1);
+        const int32_t* factors = P + static_cast<size_t>(safe) * ORDER;
+#pragma unroll
+        for (int k = 0; k < ORDER; k++) {
+            to.factor[k] = factors[k];
+        }
+        to.coefficient = C[safe];
+    };
+    constexpr int BATCH = 4;
+    Monomial queue[BATCH];
+    T upstream = T(0);
+    if (walks) {
+#pragma unroll
+        for (int d = 0; d < BATCH; d++) {
+            fetch(queue[d], g + d * G);
+        }
+        upstream = grad_output[min(row0 + r, n_rows - 1)];
+    }
+
+    // the rows of A and of grad_grad_A, STAGE values of each per lane asked for together
+    const T* a_src = A + static_cast<size_t>(row0) * nA;
+    const T* gg_src = grad_grad_A + static_cast<size_t>(row0) * nA;
+    constexpr int STAGE = 4;
+    for (int32_t base = 0; base < rows * nA; base += STAGE * ORDERED_VJP_THREADS) {
+        T staged[2][STAGE];
+#pragma unroll
+        for (int u = 0; u < STAGE; u++) {
+            const int32_t i = min(base + u * ORDERED_VJP_THREADS + tid, rows * nA - 1);
+            staged[0][u] = a_src[i];
+            staged[1][u] = gg_src[i];
+        }
+#pragma unroll
+        for (int u = 0; u < STAGE; u++) {
+            const int32_t i = base + u * ORDERED_VJP_THREADS + tid;
+            if (i < rows * nA) {
+                const int32_t row = i / nA;
+                const int32_t at = ((i - row * nA) << log2_R) + row;
+                a_stage[at] = staged[0][u];
+                gg_stage[at] = staged[1][u];
+            }
+        }
+    }
+    if (tid < R) {
+        a_stage[nA * R + tid] = T(0);
+        gg_stage[nA * R + tid] = T(0);
+    }
+    if (want_A) {
+        constexpr int HELPERS = ORDERED_VJP_THREADS / WAVE;
+        T* clear = accumulator + (tid & (WAVE - 1));
+        int32_t k = tid >> 6;
+        for (; k + 7 * HELPERS < nA + 1; k += 8 * HELPERS) {
+#pragma unroll
+            for (int u = 0; u < 8; u++) {
+                clear[(k + u * HELPERS) * WAVE] = T(0);
+            }
+        }
+        for (; k < nA + 1; k += HELPERS) {
+            clear[k * WAVE] = T(0);
+        }
+    }
+    __syncthreads();
+
+    T sum = T(0);
+    if (walks && r < rows) {
+        T* mine = accumulator + static_cast<size_t>(g) * (nA + 1) * R + r;
+        const int32_t byte_shift = log2_R + (sizeof(T) == 8 ? 3 : 2);
+        auto at = [&](auto* base, uint32_t feature) {
+            using Pointer = decltype(base);
+            using Bytes = std::conditional_t<std::is_const_v<std::remove_pointer_t<Pointer>>, const char*, char*>;
+            return reinterpret_cast<Pointer>(reinterpret_cast<Bytes>(base) + (feature << byte_shift));
+        };
+        const T* my_a = a_stage + r;
+        const T* my_gg = gg_stage + r;
+        const uint32_t features = static_cast<uint32_t>(nA);
+        auto batch = [&](int32_t j0, auto whole) {
+            constexpr bool WHOLE = decltype(whole)::value;
+            Monomial now[BATCH];
+            T a[BATCH][ORDER];
+            T gg[BATCH][ORDER];
+#pragma unroll
+            for (int d = 0; d < BATCH; d++) {
+                now[d] = queue[d];
+#pragma unroll
+                for (int k = 0; k < ORDER; k++) {
+                    // (as unsigned, a negative factor is a large one)
+                    const uint32_t feature = min(static_cast<uint32_t>(now[d].factor[k]), features);
+                    a[d][k] = *at(my_a, feature);
+                    gg[d][k] = *at(my_gg, feature);
+                }
+            }
+            if constexpr (WHOLE) {
+#pragma unroll
+                for (int d = 0; d < BATCH; d++) {
+                    fetch(queue[d], j0 + (d + BATCH) * G);
+                }
+            }
+            T term[BATCH][ORDER];
+#pragma unroll
+            for (int d = 0; d < BATCH; d++) {
+                const bool exists = WHOLE || j0 + d * G < n_monomials;
+                // products of the factors before a position, and their derivative along gg
+                T before[ORDER + 1];
+                T d_before[ORDER + 1];
+                before[0] = exists ? now[d].coefficient : T(0);
+                d_before[0] = T(0);
+#pragma unroll
+                for (int k = 0; k < ORDER; k++) {
+                    before[k + 1] = before[k] * a[d][k];
+                    d_before[k + 1] = d_before[k] * a[d][k] + before[k] * gg[d][k];
+                }
+                sum += d_before[ORDER];
+                // the same from the other end, and the two put together
+                T after = T(1);
+                T d_after = T(0);
+#pragma unroll
+                for (int f = ORDER - 1; f >= 0; f--) {
+                    term[d][f] = upstream * (d_before[f] * after + before[f] * d_after);
+                    d_after = d_after * a[d][f] + after * gg[d][f];
+                    after *= a[d][f];
+                }
+            }
+            if (want_A) {
+#pragma unroll
+                for (int d = 0; d < BATCH; d++) {
+#pragma unroll
+                    for (int f = ORDER - 1; f >= 0; f--) {
+                        // (a factor outside [0, nA) and a monomial beyond the last, whose terms
+                        // are zero, go to the row that is never read)
+                        T* to = at(mine, min(static_cast<uint32_t>(now[d].factor[f]), features));
+                        if constexpr (sizeof(T) == 8) {
+                            unsafeAtomicAdd(to, term[d][f]);
+                        } else {
+                            *to += term[d][f];
+                        }
+                    }
+                }
+            }
+        };
+        int32_t j0 = g;
+        for (; j0 + (BATCH - 1) * G < n_monomials; j0 += BATCH * G) {
+            batch(j0, std::true_type{});
+        }
+        if (j0 < n_monomials) {
+            batch(j0, std::false_type{});
+        }
+    }
+    // grad_grad_output: the lanes of the first wavefront that share a row, by a fixed tree
+    if (walks && want_O) {
+        for (int offset = WAVE / 2; offset >= R; offset >>= 1) {
+            sum += __shfl_xor(sum, offset);
+        }
+        if (tid < rows) {
+            grad_grad_output[row0 + tid] = sum;
+        }
+    }
+    __syncthreads();
+
+    if (want_A) {
+        T* dst = grad_A_2 + static_cast<size_t>(row0) * nA;
+        const int32_t copy_stride = (nA + 1) * R;
+        for (int32_t entry = tid; entry < nA * R; entry += ORDERED_VJP_THREADS) {
+            const int32_t row = entry & (R - 1);
+            const int32_t feature = entry >> log2_R;
+            const T* from = accumulator + entry;
+            T partial[4] = {T(0), T(0), T(0), T(0)};
+            int group = 0;
+            for (; group + 4 <= G; group += 4) {
+#pragma unroll
+                for (int u = 0; u < 4; u++) {
+                    partial[u] += from[(group + u) * copy_stride];
+                }
+            }
+            for (; group < G; group++) {
+                partial[group & 3] += from[group * copy_stride];
+            }
+            if (row < rows) {
+                dst[static_cast<size_t>(row) * nA + feature] = (partial[0] + partial[1]) + (partial[2] + partial[3]);
+            }
+        }
+    }
+}
+
 // The same with everything in global memory, one thread per batch row, for
 // feature counts whose tiles do not fit in LDS.
 template <typename T>
@@ -1436,6 +1669,54 @@ void homogeneous_polynomial_evaluation_vjp_vjp(MOPS_HPE_VJP_VJP_PARAMS(MOPS_CXX_
         }
         finish_call(operation);
         return;
+    }
+    // order known at compile time: the tiles of vjp_ordered_kernel and one more of grad_grad_A;
+    // rows per workgroup as there (the fewest for which all workgroups are on the device at once)
+    if (order >= 1 && order <= 6 && n_monomials > 0) {
+        const size_t accumulator_bytes = (static_cast<size_t>(nA) + 1) * WAVE * sizeof(scalar_t);
+        auto ordered_lds = [&](int rows) {
+            return accumulator_bytes + 2 * (static_cast<size_t>(nA) + 1) * rows * sizeof(scalar_t);
+        };
+        int log2_R = -1;
+        for (int log2_rows = 0; log2_rows <= 6 && ordered_lds(1 << log2_rows) <= LDS_BUDGET; log2_rows++) {
+            log2_R = log2_rows;
+            const size_t resident = 256 * std::max<size_t>(1, (160 * 1024) / ordered_lds(1 << log2_rows));
+            if (ceil_div(static_cast<size_t>(n_rows), size_t(1) << log2_rows) <= resident) {
+                break;
+            }
+        }
+        if (log2_R >= 0) {
+            const unsigned blocks = static_cast<unsigned>(ceil_div(static_cast<size_t>(n_rows), size_t(1) << log2_R));
+            const size_t lds = ordered_lds(1 << log2_R);
+#define MOPS_LAUNCH_ORDERED(ORDER)                                                                  \
+    vjp_vjp_ordered_kernel<scalar_t, ORDER><<<blocks, ORDERED_VJP_THREADS, lds, stream>>>(         \
+        grad_grad_output.data, grad_A_2.data, grad_grad_A.data, grad_output.data, A.data, C.data,  \
+        indices_A.data, n_rows, nA, n_monomials, log2_R                                            \
+    )
+            switch (order) {
+            case 1:
+                MOPS_LAUNCH_ORDERED(1);
+                break;
+            case 2:
+                MOPS_LAUNCH_ORDERED(2);
+                break;
+            case 3:
+                MOPS_LAUNCH_ORDERED(3);
+                break;
+            case 4:
+                MOPS_LAUNCH_ORDERED(4);
+                break;
+            case 5:
+                MOPS_LAUNCH_ORDERED(5);
+                break;
+            default:
+                MOPS_LAUNCH_ORDERED(6);
+                break;
+            }
+#undef MOPS_LAUNCH_ORDERED
+            finish_call(operation);
+            return;
+        }
     }
     // LDS: 2 R rows (A and grad_grad_A), WAVE accumulator rows, WAVE partial sums
     const size_t fixed_bytes = (static_cast<size_t>(nA) + 1) * WAVE * sizeof(scalar_t);

@@ -192,7 +192,9 @@ template <typename T> struct RowBuffer {
 /// All ones unless `wanted`.
 __device__ __forceinline__ uint32_t unless(bool wanted) { return static_cast<uint32_t>(wanted) - 1u; }
 
-template <typename T, int NT, bool WEIGHTED, bool NARROW>
+/// PAIRS = 2: the sum over the edges of A (x) B and of A2 (x) B2 in the same accumulators
+/// (NARROW only).
+template <typename T, int NT, bool WEIGHTED, bool NARROW, int PAIRS = 1>
 __device__ __forceinline__ void forward_segment(
     T* __restrict__ out_row,
     const T* __restrict__ A,
@@ -203,8 +205,11 @@ __device__ __forceinline__ void forward_segment(
     int32_t first,
     int32_t last,
     int32_t K,
-    int32_t L
+    int32_t L,
+    const T* __restrict__ A2 = nullptr,
+    const T* __restrict__ B2 = nullptr
 ) {
+    static_assert(PAIRS == 1 || NARROW, "two pairs: offsets of 32 bits only");
     if constexpr (!NARROW) {
         forward_segment_wide<T, NT, WEIGHTED>(out_row, A, B, W, indices_W, n_weights, first, last, K, L);
         return;
@@ -215,7 +220,9 @@ __device__ __forceinline__ void forward_segment(
     const int lane = threadIdx.x & (WAVE - 1);
     const int sub = lane & 15;
     const int quarter = lane >> 4;
-    const RowBuffer<T> rows_A(A), rows_B(B), rows_W(W);
+    const RowBuffer<T> rows_W(W);
+    const RowBuffer<T> pair_A[2] = {RowBuffer<T>(A), RowBuffer<T>(PAIRS > 1 ? A2 : A)};
+    const RowBuffer<T> pair_B[2] = {RowBuffer<T>(B), RowBuffer<T>(PAIRS > 1 ? B2 : B)};
     const RowBuffer<int32_t> rows_of_W(indices_W);
     const uint32_t a_row_bytes = static_cast<uint32_t>(K) * ES;
     const uint32_t b_row_bytes = static_cast<uint32_t>(L) * ES;
@@ -237,6 +244,10 @@ __device__ __forceinline__ void forward_segment(
             for (int t = 0; t < NT; t++) {
                 acc[t] = M::zero();
             }
+#pragma unroll
+            for (int pair = 0; pair < PAIRS; pair++) {
+            const RowBuffer<T>& rows_A = pair_A[pair];
+            const RowBuffer<T>& rows_B = pair_B[pair];
             for (int32_t e0 = first; e0 < last; e0 += 4 * UNROLL) {
                 T a[UNROLL];
                 T b[UNROLL][NT];
@@ -291,6 +302,7 @@ __device__ __forceinline__ void forward_segment(
                     }
                 }
             }
+            }
 #pragma unroll
             for (int t = 0; t < NT; t++) {
                 const int32_t col = l0 + 16 * t + sub;
@@ -332,6 +344,45 @@ __global__ __launch_bounds__(BLOCK) void forward_kernel(
         [&](int32_t row, int32_t first, int32_t last) {
             forward_segment<T, NT, WEIGHTED, NARROW>(
                 output + row * row_elements, A, B, W, indices_W, n_output, first, last, K, L
+            );
+        },
+        [&](int32_t begin, int32_t end) {
+            T* base = output + begin * row_elements;
+            const size_t count = (end - begin) * row_elements;
+            for (size_t i = lane; i < count; i += WAVE) {
+                base[i] = T(0);
+            }
+        }
+    );
+}
+
+/// output = opsa(A, B) + opsa(A2, B2) in one launch: what the second-order function needs
+/// (the forward with grad_grad_A for A plus the forward with grad_grad_B for B).
+template <typename T, int NT>
+__global__ __launch_bounds__(BLOCK) void forward_two_pairs_kernel(
+    T* __restrict__ output,
+    const T* __restrict__ A,
+    const T* __restrict__ B,
+    const T* __restrict__ A2,
+    const T* __restrict__ B2,
+    const int32_t* __restrict__ indices_output,
+    int32_t n_edges,
+    int32_t n_output,
+    int32_t K,
+    int32_t L
+) {
+    const int32_t wave_index =
+        __builtin_amdgcn_readfirstlane(blockIdx.x * WAVES_PER_BLOCK + (threadIdx.x >> 6));
+    const int lane = threadIdx.x & (WAVE - 1);
+    const size_t row_elements = static_cast<size_t>(K) * L;
+    walk_owned_segments<CHUNK>(
+        indices_output,
+        n_edges,
+        n_output,
+        wave_index,
+        [&](int32_t row, int32_t first, int32_t last) {
+            forward_segment<T, NT, false, true, 2>(
+                output + row * row_elements, A, B, nullptr, nullptr, n_output, first, last, K, L, A2, B2
             );
         },
         [&](int32_t begin, int32_t end) {
@@ -1571,6 +1622,45 @@ void launch_forward(
     finish_call(operation);
 }
 
+/// output = opsa(A, B) + opsa(A2, B2); false (and nothing launched) for shapes that
+/// launch_forward gives to other kernels than forward_kernel with offsets of 32 bits.
+template <typename T>
+bool launch_forward_of_two_pairs(
+    Tensor<T, 3> output, Tensor<T, 2> A, Tensor<T, 2> B, const T* A2, const T* B2, Tensor<int32_t, 1> indices_output
+) {
+    const int32_t n_output = narrow_i32(output.shape[0], "output.shape[0]");
+    const int32_t n_edges = narrow_i32(A.shape[0], "A.shape[0]");
+    const int32_t K = narrow_i32(A.shape[1], "A.shape[1]");
+    const int32_t L = narrow_i32(B.shape[1], "B.shape[1]");
+    narrow_i32(A.shape[1] * B.shape[1], "size_A * size_B");
+    if (n_output == 0 || K == 0 || L == 0 || n_edges == 0) {
+        return false;
+    }
+    const uint64_t widest_row = static_cast<uint64_t>(std::max(K, L)) * sizeof(T);
+    const bool narrow = !wide_offsets_forced() &&
+                        (static_cast<uint64_t>(n_edges) + 64) * std::max<uint64_t>(widest_row, 4) < (uint64_t(1) << 32) - 64 &&
+                        (static_cast<uint64_t>(n_output) + 1) * widest_row < (uint64_t(1) << 32) - 64;
+    const bool split = static_cast<size_t>(n_edges) >= static_cast<size_t>(n_output) * 2 * SPLIT && n_edges > SPLIT;
+    if (!narrow || split) {
+        return false;
+    }
+    hipStream_t stream = current_stream();
+    const unsigned blocks = blocks_for(n_edges);
+#define MOPS_LAUNCH_TWO(NT)                                                                        \
+    forward_two_pairs_kernel<T, NT><<<blocks, BLOCK, 0, stream>>>(                                 \
+        output.data, A.data, B.data, A2, B2, indices_output.data, n_edges, n_output, K, L          \
+    )
+    if (L <= 16) {
+        MOPS_LAUNCH_TWO(1);
+    } else if (L <= 32) {
+        MOPS_LAUNCH_TWO(2);
+    } else {
+        MOPS_LAUNCH_TWO(4);
+    }
+#undef MOPS_LAUNCH_TWO
+    return true;
+}
+
 template <typename T, bool WEIGHTED>
 void launch_vjp(
     Tensor<T, 2> grad_A,
@@ -1941,10 +2031,12 @@ void outer_product_scatter_add_vjp_vjp(MOPS_OPSA_VJP_VJP_PARAMS(MOPS_CXX_FIRST, 
     const size_t output_count = grad_output.shape[0] * grad_output.shape[1] * grad_output.shape[2];
 
     if (grad_grad_output.data != nullptr) {
-        if (have_A) {
+        // (callers that may pass unsorted indices: the calls below put the edges in order)
+        if (have_A && have_B && !accept_unsorted() &&
+            launch_forward_of_two_pairs<scalar_t>(grad_grad_output, grad_grad_A, B, A.data, grad_grad_B.data, indices_output)) {
+            // both terms in the sums of one launch
+        } else if (have_A && have_B) {
             ::mops::cuda::outer_product_scatter_add<scalar_t>(grad_grad_output, grad_grad_A, B, indices_output);
-        }
-        if (have_A && have_B) {
             StreamTemporary<scalar_t> second(output_count, stream);
             ::mops::cuda::outer_product_scatter_add<scalar_t>(
                 Tensor<scalar_t, 3>{second.data(), {grad_output.shape[0], grad_output.shape[1], grad_output.shape[2]}},
@@ -1953,9 +2045,20 @@ void outer_product_scatter_add_vjp_vjp(MOPS_OPSA_VJP_VJP_PARAMS(MOPS_CXX_FIRST, 
             add_in_place<scalar_t>(grad_grad_output.data, second.data(), output_count, stream);
         } else if (have_B) {
             ::mops::cuda::outer_product_scatter_add<scalar_t>(grad_grad_output, A, grad_grad_B, indices_output);
-        } else if (!have_A) {
+        } else if (have_A) {
+            ::mops::cuda::outer_product_scatter_add<scalar_t>(grad_grad_output, grad_grad_A, B, indices_output);
+        } else {
             fill_zero<scalar_t>(grad_grad_output.data, output_count, stream);
         }
+    }
+    if (grad_A_2.data != nullptr && grad_B_2.data != nullptr && have_A && have_B) {
+        // grad_A_2 is the vjp's grad_A with grad_grad_B for B, grad_B_2 its grad_B with
+        // grad_grad_A for A, and neither gradient of the vjp reads its own tensor: one call
+        ::mops::cuda::outer_product_scatter_add_vjp<scalar_t>(
+            grad_A_2, grad_B_2, grad_output, grad_grad_A, grad_grad_B, indices_output
+        );
+        finish_call(operation);
+        return;
     }
     if (grad_A_2.data != nullptr) {
         if (have_B) {

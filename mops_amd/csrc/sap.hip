@@ -845,12 +845,21 @@ void sparse_accumulation_of_products_vjp_vjp(MOPS_SAP_VJP_VJP_PARAMS(MOPS_CXX_FI
     const size_t output_count = grad_output.shape[0] * grad_output.shape[1];
 
     if (grad_grad_output.data != nullptr) {
-        if (have_A) {
+        const sap_mfma::Shape dense_shape{
+            narrow_i32(A.shape[0], "A.shape[0]"), narrow_i32(A.shape[1], "A.shape[1]"),
+            narrow_i32(B.shape[1], "B.shape[1]"), narrow_i32(grad_output.shape[1], "grad_output.shape[1]"),
+            narrow_i32(C.shape[0], "C.shape[0]")};
+        if (have_A && have_B && sap_mfma::supports_forward_of_two_pairs(dense_shape, sizeof(scalar_t))) {
+            // both terms in the sums of one launch
+            const sap_mfma::Table dense_table{C.data, indices_A.data, indices_B.data, indices_output.data};
+            sap_mfma::forward_of_two_pairs<scalar_t>(
+                grad_grad_output.data, grad_grad_A.data, B.data, A.data, grad_grad_B.data, dense_table,
+                dense_shape, stream
+            );
+        } else if (have_A && have_B) {
             ::mops::cuda::sparse_accumulation_of_products<scalar_t>(
                 grad_grad_output, grad_grad_A, B, C, indices_A, indices_B, indices_output
             );
-        }
-        if (have_A && have_B) {
             StreamTemporary<scalar_t> second(output_count, stream);
             ::mops::cuda::sparse_accumulation_of_products<scalar_t>(
                 Tensor<scalar_t, 2>{second.data(), {grad_output.shape[0], grad_output.shape[1]}}, A,
@@ -861,9 +870,22 @@ void sparse_accumulation_of_products_vjp_vjp(MOPS_SAP_VJP_VJP_PARAMS(MOPS_CXX_FI
             ::mops::cuda::sparse_accumulation_of_products<scalar_t>(
                 grad_grad_output, A, grad_grad_B, C, indices_A, indices_B, indices_output
             );
-        } else if (!have_A) {
+        } else if (have_A) {
+            ::mops::cuda::sparse_accumulation_of_products<scalar_t>(
+                grad_grad_output, grad_grad_A, B, C, indices_A, indices_B, indices_output
+            );
+        } else {
             fill_zero<scalar_t>(grad_grad_output.data, output_count, stream);
         }
+    }
+    if (grad_A_2.data != nullptr && grad_B_2.data != nullptr && have_A && have_B) {
+        // grad_A_2 is the vjp's grad_A with grad_grad_B for B, grad_B_2 its grad_B with
+        // grad_grad_A for A, and neither gradient of the vjp reads its own tensor: one call
+        ::mops::cuda::sparse_accumulation_of_products_vjp<scalar_t>(
+            grad_A_2, grad_B_2, grad_output, grad_grad_A, grad_grad_B, C, indices_A, indices_B, indices_output
+        );
+        finish_call(operation);
+        return;
     }
     if (grad_A_2.data != nullptr) {
         if (have_B) {

@@ -511,6 +511,8 @@ template <typename T> struct Arguments {
     const T* A;
     const T* B;
     const T* G; // grad_output (vjp)
+    const T* A2; // forward of two pairs: O = sap(A, B) + sap(A2, B2)
+    const T* B2;
     const T* C;
     const int32_t* PA;
     const int32_t* PB;
@@ -540,7 +542,7 @@ size_t build_areas_bytes(const Shape& s, size_t element_size) {
 /// Two wavefronts per tile of 16 rows, as in vjp_kernel below: with an even
 /// number of column tiles each takes half of them (otherwise the second one
 /// only helps with loading and storing).
-template <typename T, int NT, int GROUPS>
+template <typename T, int NT, int GROUPS, bool TWO_PAIRS = false>
 __global__ __launch_bounds__(THREADS) void forward_kernel(const Arguments<T> p) {
     using M = Mfma<T>;
     constexpr bool SPLIT = NT % 2 == 0;
@@ -595,6 +597,27 @@ __global__ __launch_bounds__(THREADS) void forward_kernel(const Arguments<T> p) 
     const bool computes = SPLIT || !second_half;
     if (computes) {
         pair_products<T, MY_TILES, GROUPS, NT>(acc, a_tile + i * p.nA, 16 * p.nA, p.nA, inner, operand, lane, first_tile);
+    }
+    if constexpr (TWO_PAIRS) {
+        // the second pair of rows through the same tiles, its products added to the same sums
+        __syncthreads();
+        if (second_half) {
+            stage_rows<T>(b_tile, p.B2 + static_cast<size_t>(safe_first) * p.nB, p.nB, valid_rows, ROWS_PER_WAVE, lane);
+        } else {
+            stage_rows<T>(a_tile, p.A2 + static_cast<size_t>(safe_first) * p.nA, p.nA, valid_rows, ROWS_PER_WAVE, lane);
+        }
+        __syncthreads();
+#pragma unroll
+        for (int r = 0; r < ROW_TILES; r++) {
+#pragma unroll
+            for (int g = 0; g < GROUPS; g++) {
+                const int32_t b = 4 * g + q;
+                inner[r][g] = load_or_zero(b_tile, (16 * r + i) * p.nB + b, b < p.nB);
+            }
+        }
+        if (computes) {
+            pair_products<T, MY_TILES, GROUPS, NT>(acc, a_tile + i * p.nA, 16 * p.nA, p.nA, inner, operand, lane, first_tile);
+        }
     }
     __syncthreads(); // nobody reads the tiles any more: they become the staging area of the store
     if (computes) {
@@ -1043,6 +1066,30 @@ void forward(T* output, const T* A, const T* B, const Table& table, const Shape&
     MOPS_HIP_CHECK(hipGetLastError());
 }
 
+bool supports_forward_of_two_pairs(const Shape& s, size_t element_size) {
+    return supports_forward(s, element_size) && !walks(s, s.nA, forward_walk_lds(s, element_size), 1);
+}
+
+template <typename T>
+void forward_of_two_pairs(
+    T* output, const T* A, const T* B, const T* A2, const T* B2, const Table& table, const Shape& s,
+    hipStream_t stream
+) {
+    Arguments<T> p = arguments<T>(A, B, table, s);
+    p.A2 = A2;
+    p.B2 = B2;
+    p.output = output;
+    p.first = operand_shape(s.nA, s.nB, s.nO);
+    const unsigned grid = static_cast<unsigned>((s.n_rows + ROWS_PER_GROUP - 1) / ROWS_PER_GROUP);
+    const size_t lds = forward_lds(s, sizeof(T));
+    with_constants<4, 4>(p.first.n_tiles, p.first.n_groups, [&](auto tiles, auto groups) {
+        auto kernel = forward_kernel<T, decltype(tiles)::value, decltype(groups)::value, true>;
+        allow_lds(kernel, lds);
+        hipLaunchKernelGGL(kernel, dim3(grid), dim3(THREADS), lds, stream, p);
+    });
+    MOPS_HIP_CHECK(hipGetLastError());
+}
+
 template <typename T>
 void vjp(
     T* grad_A, T* grad_B, const T* grad_output, const T* A, const T* B, const Table& table,
@@ -1070,6 +1117,12 @@ void vjp(
 
 template void forward<float>(float*, const float*, const float*, const Table&, const Shape&, hipStream_t);
 template void forward<double>(double*, const double*, const double*, const Table&, const Shape&, hipStream_t);
+template void forward_of_two_pairs<float>(
+    float*, const float*, const float*, const float*, const float*, const Table&, const Shape&, hipStream_t
+);
+template void forward_of_two_pairs<double>(
+    double*, const double*, const double*, const double*, const double*, const Table&, const Shape&, hipStream_t
+);
 template void vjp<float>(float*, float*, const float*, const float*, const float*, const Table&, const Shape&, hipStream_t);
 template void vjp<double>(double*, double*, const double*, const double*, const double*, const Table&, const Shape&, hipStream_t);
 

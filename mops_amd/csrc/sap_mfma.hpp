@@ -32,6 +32,17 @@ bool supports_vjp(const Shape& shape, size_t element_size);
 template <typename T>
 void forward(T* output, const T* A, const T* B, const Table& table, const Shape& shape, hipStream_t stream);
 
+/// output = sap(A, B) + sap(A2, B2) in one launch (what the second-order
+/// function needs: the sum of the forward with grad_grad_A for A and of the
+/// forward with grad_grad_B for B). Shapes of `supports_forward` whose launch
+/// has a workgroup for every 128 rows.
+bool supports_forward_of_two_pairs(const Shape& shape, size_t element_size);
+template <typename T>
+void forward_of_two_pairs(
+    T* output, const T* A, const T* B, const T* A2, const T* B2, const Table& table, const Shape& shape,
+    hipStream_t stream
+);
+
 /// grad_A or grad_B may be null.
 template <typename T>
 void vjp(
