@@ -1688,8 +1688,23 @@ static bool lists_by_arrival(const Shape& s) {
            static_cast<size_t>(s.n_nodes) * ((s.L + 15) / 16) <= SCRATCH_COUNTERS;
 }
 
+/// Block rows (of W and of grad_output) per launch of the gradient kernel when the index ranges
+/// are taken in parts: the kernel with 9 accumulator tiles does a row in less than half the time
+/// of the one with 16 (measured on 13 x 7 x 100 components, 60 000 edges, float: 16 rows 222 us,
+/// 9 rows 60 us per launch; in double the 16-tile kernel spills and is four times slower still).
+constexpr int32_t GRADIENT_PART_ROWS = 9;
+
+/// Whether the vjp is one launch on the whole index ranges. In double, also a shape with at most
+/// 16 values of every index goes in parts when W or grad_output have more than 9 rows: the
+/// 16-tile kernel spills its accumulators, and four launches on 9 and 7 rows take 0.83 of its
+/// time (16 x 16 x 16 components, 64 columns, 60 000 edges: 784 against 950 us).
+static bool vjp_in_one_launch(const Shape& s, size_t element_size) {
+    return sasaw_segments::supports(s, element_size) &&
+           !(element_size == 8 && std::max(s.n2, s.n3) > GRADIENT_PART_ROWS);
+}
+
 bool vjp_supported(const Shape& s, size_t element_size, bool want_grad_W) {
-    if (sasaw_segments::supports(s, element_size)) {
+    if (vjp_in_one_launch(s, element_size)) {
         // (more than 48 edges per node on average: only by arrival, see lists_by_arrival)
         return !want_grad_W || !dense_for_slots(s) ||
                (static_cast<size_t>(s.n_edges) <= static_cast<size_t>(s.n_nodes) * 64 && lists_by_arrival(s));
@@ -1700,7 +1715,7 @@ bool vjp_supported(const Shape& s, size_t element_size, bool want_grad_W) {
     if (s.n_nodes < 1 || s.n_edges < 1 || s.N < 1 || s.N > MAX_TABLE || s.L < 1 || s.nA < 1 || s.n2 < 1 || s.n3 < 1) {
         return false;
     }
-    constexpr int32_t ROWS = 9; // (GRADIENT_PART_ROWS)
+    constexpr int32_t ROWS = GRADIENT_PART_ROWS;
     const int64_t parts =
         static_cast<int64_t>((s.nA + MAX_INDEX - 1) / MAX_INDEX) * ((s.n2 + ROWS - 1) / ROWS) * ((s.n3 + ROWS - 1) / ROWS);
     return parts <= MAX_PARTS && offsets_fit(s, element_size) &&
@@ -1730,12 +1745,6 @@ int32_t edge_chunk_for(int32_t n_edges, int32_t edge_roles, int64_t wanted_units
     }
     return 16;
 }
-
-/// Block rows (of W and of grad_output) per launch of the gradient kernel when the index ranges
-/// are taken in parts: the kernel with 9 accumulator tiles does a row in less than half the time
-/// of the one with 16 (measured on 13 x 7 x 100 components, 60 000 edges, float: 16 rows 222 us,
-/// 9 rows 60 us per launch; in double the 16-tile kernel spills and is four times slower still).
-constexpr int32_t GRADIENT_PART_ROWS = 9;
 
 /// The index ranges one launch of the gradient kernel works on.
 struct Part {
@@ -1775,6 +1784,10 @@ void launch_gradients(
 
     with_block_rows(std::max(part.n2, part.n3), [&](auto block_rows, auto fits) {
         constexpr int NB = decltype(block_rows)::value;
+        // (more than GRADIENT_PART_ROWS rows: whole shapes in float only, see vjp_in_one_launch)
+        if constexpr (NB > GRADIENT_PART_ROWS && sizeof(T) == 8) {
+            throw std::logic_error("sasaw_segments: a launch on more than 9 rows in double");
+        } else {
         // grad_W sums over the rows of grad_output (n3 of them), the others over those of W (n2)
         args.table_W = with_offsets(
             table_of(of_part, indices.A, indices.output_2, indices.W_2, part.n3, part.n2), part.m3_begin, part.m2_begin
@@ -1810,12 +1823,16 @@ void launch_gradients(
         const bool exact = part.n2 == NB && part.n3 == NB;
         if (general) {
             // (parts of larger index ranges: lists in slots only, one variant for rows with and without padding)
-            if (vectors) {
-                launch(std::false_type{}, std::true_type{}, std::false_type{}, std::true_type{});
+            if constexpr (NB > GRADIENT_PART_ROWS) {
+                throw std::logic_error("sasaw_segments: a part of more than 9 rows");
             } else {
-                launch(std::false_type{}, std::false_type{}, std::false_type{}, std::true_type{});
+                if (vectors) {
+                    launch(std::false_type{}, std::true_type{}, std::false_type{}, std::true_type{});
+                } else {
+                    launch(std::false_type{}, std::false_type{}, std::false_type{}, std::true_type{});
+                }
+                return;
             }
-            return;
         }
         auto with_lists = [&](auto is_exact, auto with_vectors) {
             if (args.by_arrival) {
@@ -1832,6 +1849,7 @@ void launch_gradients(
             with_lists(std::false_type{}, std::true_type{});
         } else {
             with_lists(std::false_type{}, std::false_type{});
+        }
         }
     });
     MOPS_HIP_CHECK(hipGetLastError());
@@ -1857,7 +1875,7 @@ void vjp(
     args.lda = s.nA;
     args.w_stride_rows = s.n2;
     args.g_stride_rows = s.n3;
-    const bool whole = sasaw_segments::supports(s, sizeof(T));
+    const bool whole = vjp_in_one_launch(s, sizeof(T));
     if (grad_W != nullptr) {
         // the edges of every sender, listed by a launch of its own in front
         args.by_arrival = whole && lists_by_arrival(s);
