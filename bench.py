@@ -704,7 +704,7 @@ def main():
             del w, op_case
             torch.cuda.empty_cache()
 
-    # ---------------- second-order functions (not part of the step; not tuned) ----------------
+    # ---------------- second-order functions (not part of the step) ----------------
     per_op_second_order = []
     if not args.no_per_op:
         for config, op_name, op_dtype, op_case in baseline:
@@ -720,19 +720,12 @@ def main():
             def second_order(arguments=arguments, spec=spec):
                 library.call(spec.function + "_vjp_vjp", *arguments)
 
-            # (eager: these functions take a temporary from the stream's memory pool, which a
-            # capture would turn into nodes of the graph)
+            # (at these shapes the functions take no temporary, so they can be captured like the
+            # first-order calls; device_time_per_call falls back to eager calls where a capture fails)
             for _ in range(3):
                 second_order()
             torch.cuda.synchronize()
-            start = torch.cuda.Event(enable_timing=True)
-            stop = torch.cuda.Event(enable_timing=True)
-            start.record()
-            for _ in range(50):
-                second_order()
-            stop.record()
-            torch.cuda.synchronize()
-            seconds, captured = start.elapsed_time(stop) * 1e-3 / 50, False
+            seconds, captured = device_time_per_call(second_order, 20, 10, device)
             per_op_second_order.append(
                 {
                     "config": config,

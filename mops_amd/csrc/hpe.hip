@@ -28,6 +28,7 @@
 
 #include "checks.hpp"
 #include "device_common.hpp"
+#include "dispatch_thresholds.hpp"
 #include "index_validation.hpp"
 #include "elementwise.hpp"
 #include "runtime.hpp"
@@ -38,8 +39,8 @@ namespace hpe { // a name of its own for this file's kernels: profilers print it
 namespace {
 
 constexpr size_t LDS_BUDGET = 60 * 1024;
-constexpr int32_t MANY_ROWS = 4096;                     // from here on the vjp goes by feature (at 1000 rows it is the slower way)
-constexpr int32_t FORWARD_MANY_ROWS = 200 * 64;            // from here on the forward pass has a lane per row
+constexpr int32_t MANY_ROWS = thresholds::HPE_VJP_BY_FEATURE_ROWS;            // from here on the vjp goes by feature
+constexpr int32_t FORWARD_MANY_ROWS = thresholds::HPE_FORWARD_LANE_PER_ROW_ROWS; // from here on the forward pass has a lane per row
 constexpr size_t BY_FEATURE_LDS_BUDGET = 140 * 1024;    // its two tiles, of the 160 KB of a compute unit
 
 // ---------------------------------------------------------------------------

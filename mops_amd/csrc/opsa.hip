@@ -39,6 +39,7 @@
 
 #include "checks.hpp"
 #include "device_common.hpp"
+#include "dispatch_thresholds.hpp"
 #include "first_occurrences.hpp"
 #include "index_validation.hpp"
 #include "mfma.hpp"
@@ -406,7 +407,7 @@ __global__ __launch_bounds__(BLOCK) void forward_two_pairs_kernel(
 // combine_pieces_kernel adds tail[b] + head[b + 1] + head[b + 2] + ... in that
 // order for every cut segment: no atomics, one fixed order.
 // ---------------------------------------------------------------------------
-constexpr int SPLIT = 256;
+constexpr int SPLIT = thresholds::OPSA_SPLIT_POSITIONS;
 
 template <typename T, int NT, bool WEIGHTED, bool NARROW>
 __global__ __launch_bounds__(BLOCK) void forward_split_kernel(
@@ -1171,7 +1172,7 @@ __global__ __launch_bounds__((LISTS ? LISTING_WAVES : 1) * WAVE) void edge_rows_
 // flight. Used when a row of W fits one value per lane and register.
 constexpr int GATHER_SENDERS = 8;
 constexpr int GATHER_COLUMNS = 4; // values of a row per lane
-constexpr size_t SENDER_SCAN_LIMIT = 100u * 1000 * 1000; // index reads of the in-kernel gather, all workgroups together
+constexpr size_t SENDER_SCAN_LIMIT = thresholds::SENDER_SCAN_LIMIT; // index reads of the in-kernel gather, all workgroups together
 
 template <typename T>
 __global__ __launch_bounds__(GATHER_SENDERS* WAVE) void sum_by_sender_kernel(
@@ -1242,7 +1243,7 @@ __global__ __launch_bounds__(GATHER_SENDERS* WAVE) void sum_by_sender_kernel(
 // run beside the kernel that writes them (sender_buckets.hpp:
 // list_edges_in_slots): used while a sender has SLOT_MEAN_LIMIT edges or fewer
 // on average.
-constexpr int SLOT_MEAN_LIMIT = 48;
+constexpr int SLOT_MEAN_LIMIT = thresholds::SLOT_MEAN_EDGES;
 
 // The sum over the slots: one wavefront per sender, ascending edge order, as
 // many rows in flight as 32 registers hold (COLUMNS values of a row per lane).
@@ -1706,8 +1707,8 @@ void launch_vjp(
     // 33.4 / 29.6, 4000: 37.6 / 39.3, 6000: 48 / 75, 20 000: 156 / 212
     // (with no edges at all gather_in_kernel is false too: the per-edge kernel that would fill the
     // places is not launched then, so this way needs edges)
-    const bool by_arrival = want_W && narrow_rows && sparse && n_edges > 0 && K > 0 && K <= 32 &&
-                            (n_output > 4000 || !gather_in_kernel) &&
+    const bool by_arrival = want_W && narrow_rows && sparse && n_edges > 0 && K > 0 && K <= thresholds::OPSA_VJP_ROWS_IN_REGISTERS &&
+                            (n_output > thresholds::ARRIVAL_NODES || !gather_in_kernel) &&
                             static_cast<size_t>(n_output) <= SCRATCH_COUNTERS;
     // small sparse graphs: the pass over the sender index is done by workgroups of the
     // per-edge kernel's launch and leaves every sender's edges in places of its own
@@ -1776,13 +1777,13 @@ void launch_vjp(
             return shift;
         };
         const unsigned waves = static_cast<unsigned>(ceil_div(static_cast<size_t>(n_edges), CHUNK));
-        if (lds > 64 * 1024 && K > 32) {
+        if (lds > 64 * 1024 && K > thresholds::OPSA_VJP_ROWS_IN_REGISTERS) {
             const unsigned blocks = static_cast<unsigned>(ceil_div(static_cast<size_t>(n_edges), WIDE_WAVES));
             vjp_wide_kernel<T, WEIGHTED><<<blocks, WIDE_WAVES * WAVE, 0, stream>>>(
                 grad_A.data, grad_B.data, edge_W, grad_output.data, A.data, B.data, W, indices_W,
                 indices_output.data, n_edges, n_output, K, L
             );
-        } else if (K <= 32) {
+        } else if (K <= thresholds::OPSA_VJP_ROWS_IN_REGISTERS) {
             const unsigned groups = static_cast<unsigned>(ceil_div(static_cast<size_t>(n_edges), 16));
             MainKernelTimer timer(stream);
             const bool vectors = L % (16 / static_cast<int32_t>(sizeof(T))) == 0 &&

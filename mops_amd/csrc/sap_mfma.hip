@@ -40,6 +40,7 @@
 #include <hip/hip_ext.h>
 
 #include "device_common.hpp"
+#include "dispatch_thresholds.hpp"
 #include "mfma.hpp"
 #include "runtime.hpp"
 
@@ -1052,7 +1053,7 @@ void forward(T* output, const T* A, const T* B, const Table& table, const Shape&
     p.output = output;
     p.first = operand_shape(s.nA, s.nB, s.nO);
     const size_t walk_lds = forward_walk_lds(s, sizeof(T));
-    const bool walk = walks(s, s.nA, walk_lds, 1);
+    const bool walk = walks(s, s.nA, walk_lds, thresholds::SAP_FORWARD_WALK_TILES_PER_WAVE);
     const unsigned grid =
         walk ? walking_workgroups(walk_lds) : static_cast<unsigned>((s.n_rows + ROWS_PER_GROUP - 1) / ROWS_PER_GROUP);
     const size_t lds = walk ? walk_lds : forward_lds(s, sizeof(T));
@@ -1067,7 +1068,7 @@ void forward(T* output, const T* A, const T* B, const Table& table, const Shape&
 }
 
 bool supports_forward_of_two_pairs(const Shape& s, size_t element_size) {
-    return supports_forward(s, element_size) && !walks(s, s.nA, forward_walk_lds(s, element_size), 1);
+    return supports_forward(s, element_size) && !walks(s, s.nA, forward_walk_lds(s, element_size), thresholds::SAP_FORWARD_WALK_TILES_PER_WAVE);
 }
 
 template <typename T>
@@ -1102,7 +1103,7 @@ void vjp(
     p.first = operand_shape(s.nB, s.nO, s.nA);
     p.second = operand_shape(s.nA, s.nO, s.nB);
     const size_t walk_lds = vjp_walk_lds(s, sizeof(T), grad_A != nullptr, grad_B != nullptr);
-    const bool walk = walks(s, std::max(s.nA, s.nB), walk_lds, 2);
+    const bool walk = walks(s, std::max(s.nA, s.nB), walk_lds, thresholds::SAP_VJP_WALK_TILES_PER_WAVE);
     const unsigned grid =
         walk ? walking_workgroups(walk_lds) : static_cast<unsigned>((s.n_rows + ROWS_PER_GROUP - 1) / ROWS_PER_GROUP);
     const size_t lds = walk ? walk_lds : vjp_lds(s, sizeof(T), grad_A != nullptr, grad_B != nullptr);

@@ -48,6 +48,7 @@
 #include <type_traits>
 
 #include "device_common.hpp"
+#include "dispatch_thresholds.hpp"
 #include "mfma.hpp"
 #include "runtime.hpp"
 #include "segment_walk.hpp"
@@ -68,7 +69,7 @@ constexpr int TILE_GROUP = 3;    // tiles of 16 cells handled together
 constexpr int STEP_GROUP = 8;    // steps of 4 cells handled together
 constexpr size_t LDS_BUDGET = 150 * 1024; // of the 160 KB of a compute unit (beyond 64 KB a kernel has to ask)
 constexpr size_t WEIGHT_LDS_BUDGET = 96 * 1024; // the weight-gradient kernel asks for more than 64 KB
-constexpr size_t SENDER_SCAN_LIMIT = 100u * 1000 * 1000; // index reads of the in-kernel gather, all workgroups together
+constexpr size_t SENDER_SCAN_LIMIT = thresholds::SENDER_SCAN_LIMIT; // index reads of the in-kernel gather, all workgroups together
 
 template <typename T>
 __device__ __forceinline__ T load_at(const T* __restrict__ base, uint32_t byte_offset) {
@@ -1345,7 +1346,7 @@ bool orders_edges_by_sender(const Shape& s, size_t element_size) {
 /// Sparse graphs that take the in-kernel path: the edges of every sender are
 /// listed in slots (sender_buckets.hpp) beside the dense table, and the
 /// weight-gradient kernel reads the lists instead of the whole index.
-constexpr int32_t SLOT_MEAN_LIMIT = 48; // edges per sender on average (a part of the index then holds 12 of them, 32 fit)
+constexpr int32_t SLOT_MEAN_LIMIT = thresholds::SLOT_MEAN_EDGES; // edges per sender on average (a part of the index then holds 12 of them, 32 fit)
 bool lists_edges_in_slots(const Shape& s) {
     return s.n_nodes > 0 && static_cast<size_t>(s.n_edges) <= static_cast<size_t>(s.n_nodes) * SLOT_MEAN_LIMIT;
 }

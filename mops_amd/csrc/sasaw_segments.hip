@@ -37,6 +37,7 @@
 #include <type_traits>
 
 #include "device_common.hpp"
+#include "dispatch_thresholds.hpp"
 #include "mfma.hpp"
 #include "runtime.hpp"
 #include "segment_walk.hpp"
@@ -45,7 +46,7 @@
 namespace mops::amd::sasaw_segments {
 namespace {
 
-constexpr int MAX_INDEX = 16;          // values of a component index
+constexpr int MAX_INDEX = thresholds::SASAW_INDEX_VALUES; // values of a component index
 constexpr int ENTRIES_PER_LANE = 4;    // table entries a lane of the building wavefront handles at a time
 constexpr int MAX_TABLE = 1 << 16;     // entries (more: the general kernels)
 
@@ -1598,7 +1599,7 @@ bool supports(const Shape& s, size_t element_size) {
 // left, and the rows of the result in blocks of 16 inside a launch, as many as the table in LDS
 // has room for (then the next launches). Every launch walks all edges again, so the parts are
 // limited: MAX_PARTS launches.
-constexpr int32_t MAX_PARTS = 64;
+constexpr int32_t MAX_PARTS = thresholds::SASAW_MAX_PARTS;
 constexpr size_t GENERAL_TABLE_LDS = 144 * 1024; // of the 160 KB of a compute unit
 
 /// Rows of the result per launch: whole blocks of 16, as many as fit the LDS with a table of
@@ -1681,10 +1682,10 @@ void forward(
 /// against the older kernels of sasaw_mfma.hip: 76.6 / 87.6 us (float), 115.3 /
 /// 143.8 (double); with 100 edges each the lists overflow too (375 / 101 us).
 static bool dense_for_slots(const Shape& s) {
-    return static_cast<size_t>(s.n_edges) > static_cast<size_t>(s.n_nodes) * 48;
+    return static_cast<size_t>(s.n_edges) > static_cast<size_t>(s.n_nodes) * thresholds::SLOT_MEAN_EDGES;
 }
 static bool lists_by_arrival(const Shape& s) {
-    return (s.n_nodes > 4000 || dense_for_slots(s)) &&
+    return (s.n_nodes > thresholds::ARRIVAL_NODES || dense_for_slots(s)) &&
            static_cast<size_t>(s.n_nodes) * ((s.L + 15) / 16) <= SCRATCH_COUNTERS;
 }
 
@@ -1692,7 +1693,7 @@ static bool lists_by_arrival(const Shape& s) {
 /// are taken in parts: the kernel with 9 accumulator tiles does a row in less than half the time
 /// of the one with 16 (measured on 13 x 7 x 100 components, 60 000 edges, float: 16 rows 222 us,
 /// 9 rows 60 us per launch; in double the 16-tile kernel spills and is four times slower still).
-constexpr int32_t GRADIENT_PART_ROWS = 9;
+constexpr int32_t GRADIENT_PART_ROWS = thresholds::SASAW_GRADIENT_PART_ROWS;
 
 /// Whether the vjp is one launch on the whole index ranges. In double, also a shape with at most
 /// 16 values of every index goes in parts when W or grad_output have more than 9 rows: the
@@ -1707,7 +1708,7 @@ bool vjp_supported(const Shape& s, size_t element_size, bool want_grad_W) {
     if (vjp_in_one_launch(s, element_size)) {
         // (more than 48 edges per node on average: only by arrival, see lists_by_arrival)
         return !want_grad_W || !dense_for_slots(s) ||
-               (static_cast<size_t>(s.n_edges) <= static_cast<size_t>(s.n_nodes) * 64 && lists_by_arrival(s));
+               (static_cast<size_t>(s.n_edges) <= static_cast<size_t>(s.n_nodes) * thresholds::ARRIVAL_MEAN_EDGES && lists_by_arrival(s));
     }
     // more than 16 values of a component index: in parts (see vjp), every launch with the lists in
     // slots (a sender with more than 32 edges in a quarter of the index is served by a wavefront
@@ -1719,7 +1720,7 @@ bool vjp_supported(const Shape& s, size_t element_size, bool want_grad_W) {
     const int64_t parts =
         static_cast<int64_t>((s.nA + MAX_INDEX - 1) / MAX_INDEX) * ((s.n2 + ROWS - 1) / ROWS) * ((s.n3 + ROWS - 1) / ROWS);
     return parts <= MAX_PARTS && offsets_fit(s, element_size) &&
-           (!want_grad_W || static_cast<size_t>(s.n_edges) <= static_cast<size_t>(s.n_nodes) * 64);
+           (!want_grad_W || static_cast<size_t>(s.n_edges) <= static_cast<size_t>(s.n_nodes) * thresholds::ARRIVAL_MEAN_EDGES);
 }
 
 size_t vjp_workspace_bytes(const Shape& s, bool want_grad_W) {
