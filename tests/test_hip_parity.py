@@ -150,6 +150,9 @@ LARGE = {
             _one_receiver(support.sasaw_case(s, d, E=60000, nA=9, L=32, n_nodes=40), "indices_output_1"), "indices_W_1"
         ),
         "sixteen": lambda s, d: support.sasaw_case(s, d, E=30000, nA=16, L=64, n_nodes=900, n2=16, n3=16, N=700),
+        # (a hundred edges per node on a graph too large for every workgroup to read the whole sender index: the
+        # edges put in the order of their senders by a counting sort, grad_W by the forward kernel of sasaw_mfma.hip)
+        "dense_large_graph": lambda s, d: support.sasaw_case(s, d, E=400000, nA=4, L=16, n_nodes=4000, n2=3, n3=4, N=30),
         "beyond_the_matrix_path": lambda s, d: support.sasaw_case(
             s, d, E=8000, nA=20, L=100, n_nodes=300, n2=18, n3=25, N=900, allow_empty=True
         ),
