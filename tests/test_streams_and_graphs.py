@@ -82,6 +82,51 @@ def test_graph_replays_match_eager_calls(device, op):
             assert torch.equal(again, want), (op, replay)
 
 
+@pytest.mark.parametrize("op", sorted(support.SECOND_ORDER))
+def test_second_order_calls_replayed_from_a_graph(device, op):
+    """With both cotangents given, the second-order functions of these shapes launch kernels only (no
+    temporary from the stream's memory pool), so they can be captured; replays against eager calls."""
+    from mops_amd._c_lib import device_library
+
+    library = device_library()
+    spec = OPS[op]
+    case = support.to_device(support.add_cotangents(CASES[op](np.float64), op), device)
+
+    def call():
+        library.cdll.mops_amd_set_stream(torch.cuda.current_stream(device).cuda_stream)
+        library.cdll.mops_amd_set_synchronous(0)
+        outputs, arguments = support._vjp_vjp_arguments(
+            spec, case, None, None, lambda x: torch.full_like(x, float("nan"))
+        )
+        library.call(spec.function + "_vjp_vjp", *arguments)
+        return outputs
+
+    try:
+        eager = {key: value.clone() for key, value in call().items()}
+        torch.cuda.synchronize()
+        stream = torch.cuda.Stream(device=device)
+        stream.wait_stream(torch.cuda.current_stream(device))
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.stream(stream):
+            call()
+            torch.cuda.synchronize()
+            with torch.cuda.graph(graph, stream=stream):
+                captured = call()
+        torch.cuda.synchronize()
+        for replay in range(2):
+            for tensor in captured.values():
+                tensor.fill_(float("nan"))
+            other = call()  # eager work between the replays
+            torch.cuda.synchronize()
+            graph.replay()
+            torch.cuda.synchronize()
+            for key in eager:
+                assert torch.equal(captured[key], eager[key]), (op, key, replay)
+                assert torch.equal(other[key], eager[key]), (op, key, replay)
+    finally:
+        support._bind_stream(library, device)
+
+
 def test_two_host_threads_on_their_own_streams(oracle, device):
     """Two host threads, each on a stream of its own, call different operations at the same time:
     the per-thread state (stream, scratch block, error message) keeps them apart, and both get
