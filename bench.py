@@ -77,9 +77,9 @@ MAIN_KERNELS = {
     ("hpe", "vjp"): "hpe::vjp_ordered_kernel<{T}, 4, true>",
     ("sap", "forward"): "sap_mfma::forward_kernel<{T}, 2, 2>",
     ("sap", "vjp"): "sap_mfma::vjp_kernel<{T}, 5>",
-    ("opsa", "forward"): "opsa::forward_kernel<{T}, 2, false, true>",
+    ("opsa", "forward"): "opsa::forward_kernel<{T}, 2, false, true, true>",
     ("opsa", "vjp"): "opsa::edge_rows_vjp_kernel<{T}, 1, 2, false, true, false, false>",
-    ("opsaw", "forward"): "opsa::forward_kernel<{T}, 2, true, true>",
+    ("opsaw", "forward"): "opsa::forward_kernel<{T}, 2, true, true, true>",
     ("opsaw", "vjp"): "opsa::edge_rows_vjp_kernel<{T}, 1, 2, true, true, false, true>",
     ("sasaw", "forward"): {
         "float": "sasaw_segments::contract_kernel<float, 9, true, 32, false>",

@@ -189,13 +189,60 @@ template <typename T> struct RowBuffer {
             return __builtin_bit_cast(T, __builtin_amdgcn_raw_buffer_load_b64(descriptor, lane_bytes, uniform_bytes, 0));
         }
     }
+    /// N consecutive elements (N = 2 or 4) by loads of 8 or 16 bytes.
+    template <int N> __device__ __forceinline__ void load_vector(T (&to)[N], uint32_t lane_bytes, uint32_t uniform_bytes) const {
+        static_assert(N == 2 || N == 4, "two or four elements");
+        typedef uint32_t Two __attribute__((ext_vector_type(2)));
+        if constexpr (sizeof(T) == 4 && N == 2) {
+            const auto raw = __builtin_amdgcn_raw_buffer_load_b64(descriptor, lane_bytes, uniform_bytes, 0);
+            to[0] = __builtin_bit_cast(T, static_cast<uint32_t>(raw[0]));
+            to[1] = __builtin_bit_cast(T, static_cast<uint32_t>(raw[1]));
+        } else if constexpr (sizeof(T) == 4) {
+            const auto raw = __builtin_amdgcn_raw_buffer_load_b128(descriptor, lane_bytes, uniform_bytes, 0);
+#pragma unroll
+            for (int v = 0; v < 4; v++) {
+                to[v] = __builtin_bit_cast(T, static_cast<uint32_t>(raw[v]));
+            }
+        } else {
+#pragma unroll
+            for (int half = 0; half < N / 2; half++) {
+                // (the second half through the uniform offset: the lane's may be all ones)
+                const auto raw = __builtin_amdgcn_raw_buffer_load_b128(descriptor, lane_bytes, uniform_bytes + 16 * half, 0);
+                to[2 * half] = __builtin_bit_cast(T, Two{raw[0], raw[1]});
+                to[2 * half + 1] = __builtin_bit_cast(T, Two{raw[2], raw[3]});
+            }
+        }
+    }
 };
+/// N consecutive elements to memory by stores of 8 or 16 bytes (`to` aligned to them).
+template <typename T, int N> __device__ __forceinline__ void store_vector(T* to, const T (&from)[N]) {
+    static_assert(N == 2 || N == 4, "two or four elements");
+    if constexpr (sizeof(T) == 4 && N == 2) {
+        typedef T Pair __attribute__((ext_vector_type(2)));
+        *reinterpret_cast<Pair*>(to) = Pair{from[0], from[1]};
+    } else if constexpr (sizeof(T) == 4) {
+        typedef T Four __attribute__((ext_vector_type(4)));
+        *reinterpret_cast<Four*>(to) = Four{from[0], from[1], from[2], from[3]};
+    } else {
+        typedef T Pair __attribute__((ext_vector_type(2)));
+#pragma unroll
+        for (int half = 0; half < N / 2; half++) {
+            reinterpret_cast<Pair*>(to)[half] = Pair{from[2 * half], from[2 * half + 1]};
+        }
+    }
+}
 /// All ones unless `wanted`.
 __device__ __forceinline__ uint32_t unless(bool wanted) { return static_cast<uint32_t>(wanted) - 1u; }
 
 /// PAIRS = 2: the sum over the edges of A (x) B and of A2 (x) B2 in the same accumulators
 /// (NARROW only).
-template <typename T, int NT, bool WEIGHTED, bool NARROW, int PAIRS = 1>
+/// PACKED (NARROW, NT = 2 or 4, L a multiple of NT, B, W and the output aligned to NT elements):
+/// a lane holds NT CONSECUTIVE columns of a block of 16 NT (tile t of lane `sub` is column
+/// NT sub + t, not 16 t + sub), so that a row of B or W is one load of NT elements per lane and
+/// a row of the output one store, not NT of each: the kernel is bound by the number of its
+/// load instructions (half of them were loads of B), and which column a tile's lane stands
+/// for is free.
+template <typename T, int NT, bool WEIGHTED, bool NARROW, int PAIRS = 1, bool PACKED = false>
 __device__ __forceinline__ void forward_segment(
     T* __restrict__ out_row,
     const T* __restrict__ A,
@@ -211,6 +258,7 @@ __device__ __forceinline__ void forward_segment(
     const T* __restrict__ B2 = nullptr
 ) {
     static_assert(PAIRS == 1 || NARROW, "two pairs: offsets of 32 bits only");
+    static_assert(!PACKED || (NARROW && NT > 1), "packed columns: offsets of 32 bits, more than one tile");
     if constexpr (!NARROW) {
         forward_segment_wide<T, NT, WEIGHTED>(out_row, A, B, W, indices_W, n_weights, first, last, K, L);
         return;
@@ -235,11 +283,12 @@ __device__ __forceinline__ void forward_segment(
             uint32_t b_lane[NT], w_column[NT], no_column[NT];
 #pragma unroll
             for (int t = 0; t < NT; t++) {
-                const int32_t col = l0 + 16 * t + sub;
+                const int32_t col = PACKED ? l0 + NT * sub + t : l0 + 16 * t + sub;
                 no_column[t] = unless(col < L);
                 w_column[t] = static_cast<uint32_t>(col) * ES;
                 b_lane[t] = (static_cast<uint32_t>(quarter) * b_row_bytes + w_column[t]) | no_column[t];
             }
+            // (PACKED: the lane's NT columns are all inside a row or all outside: index 0 stands for them)
             typename M::Acc acc[NT];
 #pragma unroll
             for (int t = 0; t < NT; t++) {
@@ -266,9 +315,13 @@ __device__ __forceinline__ void forward_segment(
                 for (int u = 0; u < UNROLL; u++) {
                     const uint32_t row = static_cast<uint32_t>(e0 + 4 * u); // (uniform)
                     a[u] = rows_A.load(a_lane | beyond[u], row * a_row_bytes);
+                    if constexpr (PACKED) {
+                        rows_B.template load_vector<NT>(b[u], b_lane[0] | beyond[u], row * b_row_bytes);
+                    } else {
 #pragma unroll
-                    for (int t = 0; t < NT; t++) {
-                        b[u][t] = rows_B.load(b_lane[t] | beyond[u], row * b_row_bytes);
+                        for (int t = 0; t < NT; t++) {
+                            b[u][t] = rows_B.load(b_lane[t] | beyond[u], row * b_row_bytes);
+                        }
                     }
                 }
                 if (WEIGHTED) {
@@ -276,9 +329,13 @@ __device__ __forceinline__ void forward_segment(
                     for (int u = 0; u < UNROLL; u++) {
                         const uint32_t from = static_cast<uint32_t>(w_row[u]) * b_row_bytes;
                         const uint32_t nothing = unless(in_bounds(w_row[u], n_weights)) | beyond[u];
+                        if constexpr (PACKED) {
+                            rows_W.template load_vector<NT>(w[u], (from + w_column[0]) | nothing | no_column[0], 0);
+                        } else {
 #pragma unroll
-                        for (int t = 0; t < NT; t++) {
-                            w[u][t] = rows_W.load((from + w_column[t]) | nothing | no_column[t], 0);
+                            for (int t = 0; t < NT; t++) {
+                                w[u][t] = rows_W.load((from + w_column[t]) | nothing | no_column[t], 0);
+                            }
                         }
                     }
                     if (NT >= 4) {
@@ -304,14 +361,30 @@ __device__ __forceinline__ void forward_segment(
                 }
             }
             }
-#pragma unroll
-            for (int t = 0; t < NT; t++) {
-                const int32_t col = l0 + 16 * t + sub;
+            if constexpr (PACKED) {
+                const int32_t col = l0 + NT * sub;
 #pragma unroll
                 for (int r = 0; r < 4; r++) {
                     const int32_t row_k = k0 + M::row(lane, r);
                     if (row_k < K && col < L) {
-                        out_row[static_cast<size_t>(row_k) * L + col] = acc[t][r];
+                        T values[NT];
+#pragma unroll
+                        for (int t = 0; t < NT; t++) {
+                            values[t] = acc[t][r];
+                        }
+                        store_vector<T, NT>(out_row + static_cast<size_t>(row_k) * L + col, values);
+                    }
+                }
+            } else {
+#pragma unroll
+                for (int t = 0; t < NT; t++) {
+                    const int32_t col = l0 + 16 * t + sub;
+#pragma unroll
+                    for (int r = 0; r < 4; r++) {
+                        const int32_t row_k = k0 + M::row(lane, r);
+                        if (row_k < K && col < L) {
+                            out_row[static_cast<size_t>(row_k) * L + col] = acc[t][r];
+                        }
                     }
                 }
             }
@@ -320,7 +393,7 @@ __device__ __forceinline__ void forward_segment(
 }
 
 /// NARROW: every tensor is smaller than 4 GB, byte offsets of 32 bits (see RowBuffer).
-template <typename T, int NT, bool WEIGHTED, bool NARROW>
+template <typename T, int NT, bool WEIGHTED, bool NARROW, bool PACKED = false>
 __global__ __launch_bounds__(BLOCK) void forward_kernel(
     T* __restrict__ output,
     const T* __restrict__ A,
@@ -343,7 +416,7 @@ __global__ __launch_bounds__(BLOCK) void forward_kernel(
         n_output,
         wave_index,
         [&](int32_t row, int32_t first, int32_t last) {
-            forward_segment<T, NT, WEIGHTED, NARROW>(
+            forward_segment<T, NT, WEIGHTED, NARROW, 1, PACKED>(
                 output + row * row_elements, A, B, W, indices_W, n_output, first, last, K, L
             );
         },
@@ -1599,8 +1672,19 @@ void launch_forward(
     }
     {
     MainKernelTimer timer(stream);
+    // NT consecutive columns per lane (forward_segment, PACKED) where rows and pointers allow
+    const int tiles = L <= 16 ? 1 : L <= 32 ? 2 : 4;
+    const size_t vector_bytes = tiles * sizeof(T);
+    const bool packed = tiles > 1 && L % tiles == 0 && reinterpret_cast<uintptr_t>(B.data) % vector_bytes == 0 &&
+                        reinterpret_cast<uintptr_t>(output.data) % vector_bytes == 0 &&
+                        (!WEIGHTED || reinterpret_cast<uintptr_t>(W) % vector_bytes == 0);
 #define MOPS_LAUNCH_FORWARD(NT)                                                                    \
-    if (narrow) {                                                                                  \
+    if (narrow && packed) {                                                                        \
+        forward_kernel<T, NT, WEIGHTED, true, (NT > 1)><<<blocks, BLOCK, 0, stream>>>(             \
+            output.data, A.data, B.data, W, indices_W, indices_output.data, n_edges, n_output, K,  \
+            L                                                                                      \
+        );                                                                                         \
+    } else if (narrow) {                                                                           \
         forward_kernel<T, NT, WEIGHTED, true><<<blocks, BLOCK, 0, stream>>>(                       \
             output.data, A.data, B.data, W, indices_W, indices_output.data, n_edges, n_output, K,  \
             L                                                                                      \
