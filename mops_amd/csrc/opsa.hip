@@ -944,7 +944,13 @@ __global__ __launch_bounds__(256) void gather_weights_kernel(
 constexpr int LISTING_WAVES = 2;
 
 template <typename T, int KT, int NT, bool WEIGHTED, bool VECTORS, bool BLOCKS, bool LISTS>
-__global__ __launch_bounds__((LISTS ? LISTING_WAVES : 1) * WAVE) void edge_rows_vjp_kernel(
+// (LISTS: at most three wavefronts per SIMD. The workgroups that list run beside the ones that
+// work on edges, and more of the latter at a time make the launch longer, not shorter: OPSAW
+// vjp, 60 000 edges over 2000 nodes, with 5 / 4 / 3 / 2 wavefronts per SIMD 23.5 / 22.4 / 21.8 /
+// 25.7 us. Without the listing workgroups the kernel wants all it can get: 1M edges, 82 us
+// uncapped, 102 with four, 120 with three.)
+__global__ __launch_bounds__((LISTS ? LISTING_WAVES : 1) * WAVE)
+__attribute__((amdgpu_waves_per_eu(1, LISTS ? 3 : 8))) void edge_rows_vjp_kernel(
     T* __restrict__ grad_A,
     T* __restrict__ grad_B,
     T* __restrict__ edge_W,
@@ -1008,6 +1014,60 @@ __global__ __launch_bounds__((LISTS ? LISTING_WAVES : 1) * WAVE) void edge_rows_
     constexpr int VL = 16 / sizeof(T); // elements of a 16-byte vector
     typedef T Wide __attribute__((ext_vector_type(VL)));
     constexpr int L_VECTORS = L_STEPS / VL;
+    // VECTORS also decides which columns the accumulators of grad_B stand for: tile t of lane i
+    // is column 16 t + i otherwise, and with VECTORS the tiles come in groups of PW whose lanes
+    // hold PW CONSECUTIVE columns (group g, lane i: columns 16 PW g + PW i ...), so that the
+    // rows of grad_output, W and B that meet these accumulators are read, and grad_B and the
+    // per-edge rows of grad_W written, PW columns per instruction: the matrix instruction does
+    // not care which column a lane stands for, and the kernel pays per instruction.
+    constexpr int PW = VECTORS ? (NT < VL ? NT : VL) : 1;
+    // the NT values of a row at this lane's columns (`row_start`: index of the row's column l_base)
+    auto load_columns = [&](T (&to)[NT], const T* base, size_t row_start, int32_t l_base, bool row_ok) {
+        if constexpr (PW > 1) {
+            typedef T Columns __attribute__((ext_vector_type(PW)));
+#pragma unroll
+            for (int g = 0; g < NT / PW; g++) {
+                const int32_t l = 16 * PW * g + PW * i;
+                const bool ok = row_ok && l_base + l < L;
+                const Columns values = *reinterpret_cast<const Columns*>(base + (ok ? row_start + l : 0));
+#pragma unroll
+                for (int c = 0; c < PW; c++) {
+                    to[PW * g + c] = ok ? values[c] : T(0);
+                }
+            }
+        } else {
+#pragma unroll
+            for (int t = 0; t < NT; t++) {
+                const int32_t l = 16 * t + i;
+                to[t] = load_or_zero(base, row_start + l, row_ok && l_base + l < L);
+            }
+        }
+    };
+    auto store_columns = [&](T* base, size_t row_start, int32_t l_base, const T (&from)[NT]) {
+        if constexpr (PW > 1) {
+            typedef T Columns __attribute__((ext_vector_type(PW)));
+#pragma unroll
+            for (int g = 0; g < NT / PW; g++) {
+                const int32_t l = 16 * PW * g + PW * i;
+                if (l_base + l < L) {
+                    Columns values;
+#pragma unroll
+                    for (int c = 0; c < PW; c++) {
+                        values[c] = from[PW * g + c];
+                    }
+                    *reinterpret_cast<Columns*>(base + row_start + l) = values;
+                }
+            }
+        } else {
+#pragma unroll
+            for (int t = 0; t < NT; t++) {
+                const int32_t l = 16 * t + i;
+                if (l_base + l < L) {
+                    base[row_start + l] = from[t];
+                }
+            }
+        }
+    };
     auto wide_or_zero = [](const T* pointer, size_t index, bool ok) {
         const Wide value = *reinterpret_cast<const Wide*>(pointer + (ok ? index : 0));
         Wide zero;
@@ -1089,24 +1149,20 @@ __global__ __launch_bounds__((LISTS ? LISTING_WAVES : 1) * WAVE) void edge_rows_
 
     for (int32_t next_base = 0;;) {
     const int32_t l_base = BLOCKS ? next_base : 0;
-    // factors of the results, per accumulator element (row = edge, column l = 16 t + i):
+    // factors of the results, per accumulator element (row = edge, column of the tile):
     // asked for now, needed after the matrix products
-    T weight_out[NT][4];
-    T b_out[NT][4];
+    T weight_out[4][NT];
+    T b_out[4][NT];
     if constexpr (WEIGHTED) {
 #pragma unroll
-        for (int t = 0; t < NT; t++) {
-#pragma unroll
-            for (int r = 0; r < 4; r++) {
-                const int32_t row = M::row(lane, r);
-                const int32_t l = l_base + 16 * t + i;
-                const bool ok = row < n && l < L;
-                const int32_t sender = __shfl(my_sender, row);
-                weight_out[t][r] = load_or_zero(
-                    W, static_cast<size_t>(sender) * L + l, ok && want_B && in_bounds(sender, n_output)
-                );
-                b_out[t][r] = load_or_zero(B, static_cast<size_t>(first_edge + row) * L + l, ok && want_W);
-            }
+        for (int r = 0; r < 4; r++) {
+            const int32_t row = M::row(lane, r);
+            const int32_t sender = __shfl(my_sender, row);
+            load_columns(
+                weight_out[r], W, static_cast<size_t>(sender) * L + l_base, l_base,
+                row < n && want_B && in_bounds(sender, n_output)
+            );
+            load_columns(b_out[r], B, static_cast<size_t>(first_edge + row) * L + l_base, l_base, row < n && want_W);
         }
     }
 
@@ -1165,16 +1221,12 @@ __global__ __launch_bounds__((LISTS ? LISTING_WAVES : 1) * WAVE) void edge_rows_
                 }
             }
             if (want_B || want_W) {
-                // right operand: lane (column l = 16 t + i, reduction index k = 4 s + q)
+                // right operand: lane (column of tile t, reduction index k = 4 s + q)
                 T right[K_STEPS][NT];
 #pragma unroll
                 for (int s = 0; s < K_STEPS; s++) {
                     const int32_t k = 4 * s + q;
-#pragma unroll
-                    for (int t = 0; t < NT; t++) {
-                        const int32_t l = l_base + 16 * t + i;
-                        right[s][t] = load_or_zero(block, k * L + l, k < K && l < L);
-                    }
+                    load_columns(right[s], block, static_cast<size_t>(k) * L + l_base, l_base, k < K);
                 }
 #pragma unroll
                 for (int s = 0; s < K_STEPS; s++) {
@@ -1192,25 +1244,35 @@ __global__ __launch_bounds__((LISTS ? LISTING_WAVES : 1) * WAVE) void edge_rows_
         node = later == 0 ? -1 : __builtin_amdgcn_readlane(my_node, __ffsll(static_cast<long long>(later)) - 1);
     }
 
-    // accumulators: lane (column = 16 t + i, rows = edges M::row(lane, r))
+    // accumulators: lane (column of tile t, rows = edges M::row(lane, r))
     if (want_B || want_W) {
 #pragma unroll
-        for (int t = 0; t < NT; t++) {
-#pragma unroll
-            for (int r = 0; r < 4; r++) {
-                const int32_t row = M::row(lane, r);
-                const int32_t l = l_base + 16 * t + i;
-                const bool ok = row < n && l < L;
-                const size_t at = static_cast<size_t>(first_edge + row) * L + l;
+        for (int r = 0; r < 4; r++) {
+            const int32_t row = M::row(lane, r);
+            if (row < n) {
+                const size_t row_start = static_cast<size_t>(first_edge + row) * L + l_base;
+                T values[NT];
                 if constexpr (WEIGHTED) {
-                    if (want_B && ok) {
-                        grad_B[at] = acc_B[t][r] * weight_out[t][r];
+                    if (want_B) {
+#pragma unroll
+                        for (int t = 0; t < NT; t++) {
+                            values[t] = acc_B[t][r] * weight_out[r][t];
+                        }
+                        store_columns(grad_B, row_start, l_base, values);
                     }
-                    if (want_W && ok) {
-                        edge_W[at] = acc_B[t][r] * b_out[t][r];
+                    if (want_W) {
+#pragma unroll
+                        for (int t = 0; t < NT; t++) {
+                            values[t] = acc_B[t][r] * b_out[r][t];
+                        }
+                        store_columns(edge_W, row_start, l_base, values);
                     }
-                } else if (ok) {
-                    grad_B[at] = acc_B[t][r];
+                } else {
+#pragma unroll
+                    for (int t = 0; t < NT; t++) {
+                        values[t] = acc_B[t][r];
+                    }
+                    store_columns(grad_B, row_start, l_base, values);
                 }
             }
         }
@@ -1873,6 +1935,8 @@ void launch_vjp(
             const bool vectors = L % (16 / static_cast<int32_t>(sizeof(T))) == 0 &&
                                  reinterpret_cast<uintptr_t>(B.data) % 16 == 0 &&
                                  reinterpret_cast<uintptr_t>(grad_output.data) % 16 == 0 &&
+                                 reinterpret_cast<uintptr_t>(grad_B.data) % 16 == 0 &&
+                                 reinterpret_cast<uintptr_t>(edge_W) % 16 == 0 &&
                                  (!WEIGHTED || reinterpret_cast<uintptr_t>(W) % 16 == 0);
 #define MOPS_LAUNCH_ROWS_WITH(KT, NT, VECTORS, BLOCKS, LISTS, GRID, WAVES)                          \
     edge_rows_vjp_kernel<T, KT, NT, WEIGHTED, VECTORS, BLOCKS, LISTS><<<GRID, (WAVES) * WAVE, 0, stream>>>( \
