@@ -392,6 +392,57 @@ def test_large_inputs(oracle, device, op, name, dtype):
         check(gradients[key].cpu().numpy(), expected[key], same.get(key), sums.get(key), f"{op}/{name} grad_{key}")
 
 
+# ---- pointers that are aligned to an element and no more -------------------
+OFF_BOUNDARY = {
+    "hpe": lambda d: support.hpe_case(31, d, I=300, nA=20, J=150, K=3),
+    "sap": lambda d: support.sap_case(32, d, I=700, nA=13, nB=7, K=300, nO=20),
+    "opsa": lambda d: support.opsa_case(33, d, J=3000, K=13, L=20, n_out=90, allow_empty=True),
+    "opsa_wide": lambda d: support.opsa_case(34, d, J=2000, K=20, L=64, n_out=60, allow_empty=True),
+    "opsaw": lambda d: support.opsaw_case(35, d, E=3000, K=13, L=32, n_nodes=90, allow_empty=True),
+    "opsaw_many_senders": lambda d: support.opsaw_case(36, d, E=20000, K=4, L=16, n_nodes=5000, allow_empty=True),
+    "sasaw": lambda d: support.sasaw_case(37, d, E=3000, nA=9, L=32, n_nodes=90, allow_empty=True),
+    "sasaw_parts": lambda d: support.sasaw_case(38, d, E=900, nA=17, L=20, n_nodes=31, n2=20, n3=18, N=500, allow_empty=True),
+}
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=["f32", "f64"])
+@pytest.mark.parametrize("name", list(OFF_BOUNDARY))
+def test_pointers_one_element_off_the_vector_boundaries(oracle, device, name, dtype):
+    """Every tensor (inputs, indices, outputs) starts one element behind a 256-byte boundary, so no
+    pointer is aligned to 8 or 16 bytes: the kernels that move 8 or 16 bytes per lane must step aside
+    for the ones that move single elements."""
+    import torch
+
+    from mops_amd._c_lib import device_library
+
+    op = name.split("_")[0]
+    spec = OPS[op]
+    case = OFF_BOUNDARY[name](dtype)
+
+    def shifted(tensor):
+        room = torch.empty(tensor.numel() + 1, dtype=tensor.dtype, device=device)
+        view = room[1:].view(tensor.shape)
+        view.copy_(tensor)
+        assert view.data_ptr() % 256 == tensor.element_size()
+        return view
+
+    on_device = {
+        key: shifted(value) if isinstance(value, torch.Tensor) else value
+        for key, value in to_device(case, device).items()
+    }
+    library = device_library()
+    support._bind_stream(library, device)
+    inputs = [on_device[key] for key in spec.inputs]
+    output = shifted(torch.full(spec.output_shape(on_device), float("nan"), dtype=on_device["A"].dtype, device=device))
+    library.call(spec.function, output, *inputs)
+    assert_close(output.cpu().numpy(), cpu_forward(oracle, op, case), dtype, f"{name} forward")
+    gradients = [shifted(torch.full_like(on_device[key], float("nan"))) for key in spec.differentiable]
+    library.call(spec.function + "_vjp", *gradients, on_device["grad_output"], *inputs)
+    expected = cpu_vjp(oracle, op, case)
+    for key, got in zip(spec.differentiable, gradients):
+        assert_close(got.cpu().numpy(), expected[key], dtype, f"{name} grad_{key}")
+
+
 # ---- BASELINE configurations at full size ---------------------------------
 BASELINE = [
     ("hpe", 0, np.float64, lambda d: support.hpe_case(0, d)),
