@@ -57,6 +57,9 @@ CASES = {
         ),
         "many_columns": lambda s, d: support.opsa_case(s, d, J=700, K=16, L=128, n_out=31, allow_empty=True),
         "ragged_columns": lambda s, d: support.opsa_case(s, d, J=500, K=20, L=70, n_out=23, allow_empty=True),
+        # (rows of B that end inside a block of 64 or 32 columns whose lanes hold 4 or 2 consecutive ones)
+        "columns_in_fours": lambda s, d: support.opsa_case(s, d, J=600, K=7, L=72, n_out=29, allow_empty=True),
+        "columns_in_twos": lambda s, d: support.opsa_case(s, d, J=600, K=18, L=18, n_out=29, allow_empty=True),
     },
     "opsaw": {
         "tiny": lambda s, d: support.opsaw_case(s, d, E=6, K=2, L=3, n_nodes=4, allow_empty=True),
@@ -79,6 +82,8 @@ CASES = {
         ),
         "many_columns": lambda s, d: support.opsaw_case(s, d, E=700, K=32, L=192, n_nodes=31, allow_empty=True),
         "ragged_columns": lambda s, d: support.opsaw_case(s, d, E=500, K=9, L=131, n_nodes=23, allow_empty=True),
+        "columns_in_fours": lambda s, d: support.opsaw_case(s, d, E=600, K=7, L=72, n_nodes=29, allow_empty=True),
+        "columns_in_twos": lambda s, d: support.opsaw_case(s, d, E=600, K=18, L=18, n_nodes=29, allow_empty=True),
     },
     "sasaw": {
         "tiny": lambda s, d: support.sasaw_case(s, d, E=6, nA=2, L=3, n_nodes=4, n2=2, n3=2, N=5, allow_empty=True),
