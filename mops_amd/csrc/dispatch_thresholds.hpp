@@ -41,9 +41,12 @@ constexpr int64_t SAP_VJP_WALK_TILES_PER_WAVE = 2;
 /// leave the device idle). 50 rows of 2400 edges: 94 -> 21 us in f32.
 constexpr int OPSA_SPLIT_POSITIONS = 256;
 /// vjp: columns of A up to which the per-edge kernel keeps a receiver's rows
-/// of grad_output as matrix operands in registers; beyond, the LDS-staged
-/// kernels (K = L = 48: 82 us against about 30 at K = 32).
-constexpr int32_t OPSA_VJP_ROWS_IN_REGISTERS = 32;
+/// of grad_output as matrix operands in registers (one to four tiles of 16);
+/// beyond, the LDS-staged kernels. 60 000 edges, K = L = 48: 34 us against 82
+/// (f32), 61 against 150 (f64); K = L = 64: 58 against 140, 107 against 552;
+/// K = 56, L = 128: 118 against 507, 177 against 994; OPSAW K = L = 64: 97
+/// against 220, 133 against 566.
+constexpr int32_t OPSA_VJP_ROWS_IN_REGISTERS = 64;
 
 // ---- the edges of every sender (grad_W of OPSAW and SASAW) -------------------
 /// Index reads (edges x workgroups) up to which every workgroup finds its

@@ -1986,7 +1986,7 @@ void launch_vjp(
                 } else {
                     MOPS_LAUNCH_ROW_PASSES(1);
                 }
-            } else {
+            } else if (K <= 32) {
                 if (L <= 16) {
                     MOPS_LAUNCH_ROWS(2, 1);
                 } else if (L <= 32) {
@@ -1995,6 +1995,26 @@ void launch_vjp(
                     MOPS_LAUNCH_ROWS(2, 4);
                 } else {
                     MOPS_LAUNCH_ROW_PASSES(2);
+                }
+            } else if (K <= 48) {
+                if (L <= 16) {
+                    MOPS_LAUNCH_ROWS(3, 1);
+                } else if (L <= 32) {
+                    MOPS_LAUNCH_ROWS(3, 2);
+                } else if (L <= 64) {
+                    MOPS_LAUNCH_ROWS(3, 4);
+                } else {
+                    MOPS_LAUNCH_ROW_PASSES(3);
+                }
+            } else {
+                if (L <= 16) {
+                    MOPS_LAUNCH_ROWS(4, 1);
+                } else if (L <= 32) {
+                    MOPS_LAUNCH_ROWS(4, 2);
+                } else if (L <= 64) {
+                    MOPS_LAUNCH_ROWS(4, 4);
+                } else {
+                    MOPS_LAUNCH_ROW_PASSES(4);
                 }
             }
 #undef MOPS_LAUNCH_ROW_PASSES

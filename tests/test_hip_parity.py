@@ -50,6 +50,9 @@ CASES = {
         "ragged": lambda s, d: support.opsa_case(s, d, J=1000, K=13, L=20, n_out=37, allow_empty=True),
         "long_segments": lambda s, d: support.opsa_case(s, d, J=3000, K=5, L=7, n_out=6),
         "wide": lambda s, d: support.opsa_case(s, d, J=400, K=40, L=33, n_out=21, allow_empty=True),
+        # (more than 64 columns of A: the vjp whose rows of grad_output are staged in LDS)
+        "tall": lambda s, d: support.opsa_case(s, d, J=400, K=70, L=33, n_out=21, allow_empty=True),
+        "sixty_four_by_sixty_four": lambda s, d: support.opsa_case(s, d, J=500, K=64, L=64, n_out=25, allow_empty=True),
         "mostly_empty": lambda s, d: support.opsa_case(s, d, J=20, K=4, L=4, n_out=300, allow_empty=True),
         "pooling": lambda s, d: support.opsa_case(s, d, J=5000, K=13, L=20, n_out=7),
         "pooling_mixed_lengths": lambda s, d: _with_lengths(
@@ -76,6 +79,8 @@ CASES = {
         ),
         "forty_five_per_sender": lambda s, d: support.opsaw_case(s, d, E=4500, K=6, L=32, n_nodes=100),
         "sparse_tall": lambda s, d: support.opsaw_case(s, d, E=700, K=40, L=24, n_nodes=60, allow_empty=True),
+        "sparse_taller": lambda s, d: support.opsaw_case(s, d, E=700, K=70, L=24, n_nodes=60, allow_empty=True),
+        "fifty_seven_by_eighty": lambda s, d: support.opsaw_case(s, d, E=700, K=57, L=80, n_nodes=40, allow_empty=True),
         "pooling": lambda s, d: support.opsaw_case(s, d, E=5000, K=13, L=32, n_nodes=7),
         "pooling_mixed_lengths": lambda s, d: _with_lengths(
             support.opsaw_case(s, d, E=sum(MIXED_LENGTHS), K=3, L=17, n_nodes=len(MIXED_LENGTHS)), "indices_output", MIXED_LENGTHS
@@ -141,6 +146,8 @@ LARGE = {
         "many_edges": lambda s, d: support.opsa_case(s, d, J=1000003, K=13, L=20, n_out=30000, allow_empty=True),
         "one_receiver": lambda s, d: _one_receiver(support.opsa_case(s, d, J=120000, K=13, L=20, n_out=50), "indices_output"),
         "wide_rows": lambda s, d: support.opsa_case(s, d, J=20000, K=50, L=200, n_out=300, allow_empty=True),
+        # (more than 64 columns of A and rows of grad_output beyond 64 KB: the vjp that keeps them in global memory)
+        "tall_wide_rows": lambda s, d: support.opsa_case(s, d, J=8000, K=70, L=300, n_out=100, allow_empty=True),
     },
     "opsaw": {
         "many_edges": lambda s, d: support.opsaw_case(s, d, E=500001, K=16, L=64, n_nodes=20000, allow_empty=True),
@@ -148,6 +155,7 @@ LARGE = {
             _one_receiver(support.opsaw_case(s, d, E=120000, K=13, L=32, n_nodes=50), "indices_output"), "indices_W"
         ),
         "wide_rows": lambda s, d: support.opsaw_case(s, d, E=20000, K=40, L=300, n_nodes=300, allow_empty=True),
+        "tall_wide_rows": lambda s, d: support.opsaw_case(s, d, E=8000, K=70, L=300, n_nodes=100, allow_empty=True),
     },
     "sasaw": {
         "many_edges": lambda s, d: support.sasaw_case(s, d, E=300001, nA=9, L=32, n_nodes=10000, allow_empty=True),
