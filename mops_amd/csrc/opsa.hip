@@ -1960,11 +1960,28 @@ void launch_vjp(
     } else {                                                                                       \
         MOPS_LAUNCH_ROWS_AS(KT, NT, false, false);                                                 \
     }
-#define MOPS_LAUNCH_ROW_PASSES(KT)                                                                 \
+#define MOPS_LAUNCH_ROW_PASSES_OF(KT, NT)                                                          \
     if (vectors) {                                                                                 \
-        MOPS_LAUNCH_ROWS_AS(KT, 4, true, true);                                                    \
+        MOPS_LAUNCH_ROWS_AS(KT, NT, true, true);                                                   \
     } else {                                                                                       \
-        MOPS_LAUNCH_ROWS_AS(KT, 4, false, true);                                                   \
+        MOPS_LAUNCH_ROWS_AS(KT, NT, false, true);                                                  \
+    }
+// More than 32 columns: one pass over 64 (four column tiles), or passes of 64 each beyond that.
+// In double the kernel with four column tiles has room for one wavefront per SIMD where the
+// rows of W come with it (OPSAW) or A has more than 16 columns; passes of 32 columns (two
+// tiles, three wavefronts per SIMD) are then the faster way, although grad_output is read once
+// per pass (60 000 edges, f64, 64 / 32 columns per pass: OPSAW K = 13, L = 64: 67.8 / 57.3 us;
+// K = 13, L = 128: 139 / 104; K = 25, L = 64: 84.9 / 71.0; OPSA K = 25, L = 64: 54.1 / 45.3;
+// K = 25, L = 128: 102 / 89), but not with three or four tiles of columns of A (K = L = 48:
+// 61.5 / 78.3; OPSAW K = L = 64: 132 / 158) nor for OPSA with up to 16 columns of A
+// (K = 13, L = 64: 27.4 / 29.0).
+#define MOPS_LAUNCH_BEYOND_32(KT, SINGLE_PASS)                                                     \
+    if constexpr (sizeof(T) == 8 && (WEIGHTED ? KT <= 2 : KT == 2)) {                              \
+        MOPS_LAUNCH_ROW_PASSES_OF(KT, 2);                                                          \
+    } else if (SINGLE_PASS) {                                                                      \
+        MOPS_LAUNCH_ROWS(KT, 4);                                                                   \
+    } else {                                                                                       \
+        MOPS_LAUNCH_ROW_PASSES_OF(KT, 4);                                                          \
     }
             // the listing of the senders' edges rides along in this launch
             const unsigned list_blocks = slotted ? sender_slots_blocks(n_output) : 0;
@@ -1981,43 +1998,36 @@ void launch_vjp(
                     MOPS_LAUNCH_ROWS(1, 1);
                 } else if (L <= 32) {
                     MOPS_LAUNCH_ROWS(1, 2);
-                } else if (L <= 64) {
-                    MOPS_LAUNCH_ROWS(1, 4);
                 } else {
-                    MOPS_LAUNCH_ROW_PASSES(1);
+                    MOPS_LAUNCH_BEYOND_32(1, L <= 64);
                 }
             } else if (K <= 32) {
                 if (L <= 16) {
                     MOPS_LAUNCH_ROWS(2, 1);
                 } else if (L <= 32) {
                     MOPS_LAUNCH_ROWS(2, 2);
-                } else if (L <= 64) {
-                    MOPS_LAUNCH_ROWS(2, 4);
                 } else {
-                    MOPS_LAUNCH_ROW_PASSES(2);
+                    MOPS_LAUNCH_BEYOND_32(2, L <= 64);
                 }
             } else if (K <= 48) {
                 if (L <= 16) {
                     MOPS_LAUNCH_ROWS(3, 1);
                 } else if (L <= 32) {
                     MOPS_LAUNCH_ROWS(3, 2);
-                } else if (L <= 64) {
-                    MOPS_LAUNCH_ROWS(3, 4);
                 } else {
-                    MOPS_LAUNCH_ROW_PASSES(3);
+                    MOPS_LAUNCH_BEYOND_32(3, L <= 64);
                 }
             } else {
                 if (L <= 16) {
                     MOPS_LAUNCH_ROWS(4, 1);
                 } else if (L <= 32) {
                     MOPS_LAUNCH_ROWS(4, 2);
-                } else if (L <= 64) {
-                    MOPS_LAUNCH_ROWS(4, 4);
                 } else {
-                    MOPS_LAUNCH_ROW_PASSES(4);
+                    MOPS_LAUNCH_BEYOND_32(4, L <= 64);
                 }
             }
-#undef MOPS_LAUNCH_ROW_PASSES
+#undef MOPS_LAUNCH_BEYOND_32
+#undef MOPS_LAUNCH_ROW_PASSES_OF
 #undef MOPS_LAUNCH_ROWS
 #undef MOPS_LAUNCH_ROWS_AS
 #undef MOPS_LAUNCH_ROWS_WITH
