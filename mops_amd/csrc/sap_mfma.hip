@@ -55,7 +55,7 @@ constexpr int THREADS = 2 * WAVES * WAVE; // two wavefronts per tile of 16 rows
 constexpr int MAX_INNER_GROUPS_FORWARD = 4; // nB <= 16
 constexpr int MAX_INNER_GROUPS_VJP = 16;    // nO <= 64
 constexpr int MAX_OUTER = 16;
-constexpr int MAX_ENTRIES = 2048;
+constexpr int MAX_ENTRIES = 8192;
 constexpr size_t LDS_BUDGET = 156 * 1024; // of the 160 KB of a compute unit (16 values of every index in double need 153 KB for the vjp)
 constexpr size_t LDS_WITHOUT_ASKING = 64 * 1024;
 
@@ -89,12 +89,17 @@ OperandShape operand_shape(int32_t n_outer, int32_t n_inner, int32_t n_columns) 
     return s;
 }
 
-constexpr int ENTRIES_PER_THREAD = MAX_ENTRIES / THREADS;
+// Table entries per thread of the build: 2 for tables of up to 2048 entries (what real
+// Clebsch-Gordan tables of up to 16 x 16 x 16 cells mostly are), 8 beyond (more registers while
+// the table is built). The kernels after the build do not depend on the number of entries.
+constexpr int FEW_ENTRIES_PER_THREAD = 2;
+constexpr int MANY_ENTRIES_PER_THREAD = MAX_ENTRIES / THREADS;
+constexpr int FEW_ENTRIES = FEW_ENTRIES_PER_THREAD * THREADS;
 constexpr int32_t NOBODY = 0x7fffffff;
 
 /// The table entries a thread looks after (entry k = thread + e * THREADS),
 /// loaded once, before anything waits for memory.
-template <typename T> struct MyEntries {
+template <typename T, int ENTRIES_PER_THREAD> struct MyEntries {
     int32_t index_A[ENTRIES_PER_THREAD];
     int32_t index_B[ENTRIES_PER_THREAD];
     int32_t index_O[ENTRIES_PER_THREAD];
@@ -141,10 +146,10 @@ template <typename T> struct BuildAreas {
     T* coefficients;
 };
 
-template <typename T, int TARGETS>
+template <typename T, int TARGETS, int ENTRIES_PER_THREAD>
 __device__ __forceinline__ void build_operands(
     const OperandTarget<T> (&targets)[TARGETS], const BuildAreas<T>& areas, int32_t nA, int32_t nB,
-    int32_t nO, const MyEntries<T>& entries
+    int32_t nO, const MyEntries<T, ENTRIES_PER_THREAD>& entries
 ) {
     const int tid = threadIdx.x;
 #pragma unroll
@@ -543,7 +548,7 @@ size_t build_areas_bytes(const Shape& s, size_t element_size) {
 /// Two wavefronts per tile of 16 rows, as in vjp_kernel below: with an even
 /// number of column tiles each takes half of them (otherwise the second one
 /// only helps with loading and storing).
-template <typename T, int NT, int GROUPS, bool TWO_PAIRS = false>
+template <typename T, int NT, int GROUPS, bool TWO_PAIRS = false, int EPT = FEW_ENTRIES_PER_THREAD>
 __global__ __launch_bounds__(THREADS) void forward_kernel(const Arguments<T> p) {
     using M = Mfma<T>;
     constexpr bool SPLIT = NT % 2 == 0;
@@ -558,7 +563,7 @@ __global__ __launch_bounds__(THREADS) void forward_kernel(const Arguments<T> p) 
     const int tile = wave & (WAVES - 1);
     const bool second_half = wave >= WAVES; // uniform per wavefront
     const int32_t row_width = p.nA + p.nB;
-    MyEntries<T> entries;
+    MyEntries<T, EPT> entries;
     entries.load(p.C, p.PA, p.PB, p.PO, p.K);
     T* mine = reinterpret_cast<T*>(cursor) + tile * ROWS_PER_WAVE * max(row_width, p.nO);
     T* a_tile = mine;                          // [16][nA]
@@ -573,7 +578,7 @@ __global__ __launch_bounds__(THREADS) void forward_kernel(const Arguments<T> p) 
         stage_rows<T>(a_tile, p.A + static_cast<size_t>(safe_first) * p.nA, p.nA, valid_rows, ROWS_PER_WAVE, lane);
     }
     const OperandTarget<T> targets[1] = {{operand, p.first, {0, 1, 2}}};
-    build_operands<T, 1>(targets, areas, p.nA, p.nB, p.nO, entries); // ends with a barrier: the tiles are there
+    build_operands<T, 1, EPT>(targets, areas, p.nA, p.nB, p.nO, entries); // ends with a barrier: the tiles are there
 
     const int i = lane & 15;
     const int q = lane >> 4;
@@ -638,7 +643,7 @@ __global__ __launch_bounds__(THREADS) void forward_kernel(const Arguments<T> p) 
 /// Two wavefronts per tile of 16 rows: wavefront t computes grad_A of tile t,
 /// wavefront t + 8 grad_B, from the same rows in LDS; four wavefronts per SIMD
 /// keep the matrix cores busier than two.
-template <typename T, int GROUPS>
+template <typename T, int GROUPS, int EPT = FEW_ENTRIES_PER_THREAD>
 __global__ __launch_bounds__(THREADS) void vjp_kernel(const Arguments<T> p) {
     using M = Mfma<T>;
     extern __shared__ __align__(16) char lds_raw[];
@@ -655,7 +660,7 @@ __global__ __launch_bounds__(THREADS) void vjp_kernel(const Arguments<T> p) {
     const int tile = wave & (WAVES - 1);
     const bool second_half = wave >= WAVES; // uniform per wavefront
     const int32_t row_width = p.nA + p.nB + p.nO;
-    MyEntries<T> entries;
+    MyEntries<T, EPT> entries;
     entries.load(p.C, p.PA, p.PB, p.PO, p.K);
     T* mine = reinterpret_cast<T*>(cursor) + tile * ROWS_PER_WAVE * row_width;
     T* a_tile = mine;                                  // [16][nA]
@@ -675,7 +680,7 @@ __global__ __launch_bounds__(THREADS) void vjp_kernel(const Arguments<T> p) {
         {want_A ? operand_A : nullptr, p.first, {1, 2, 0}},
         {want_B ? operand_B : nullptr, p.second, {0, 2, 1}},
     };
-    build_operands<T, 2>(targets, areas, p.nA, p.nB, p.nO, entries); // ends with a barrier: the tiles are there
+    build_operands<T, 2, EPT>(targets, areas, p.nA, p.nB, p.nO, entries); // ends with a barrier: the tiles are there
 
     const int i = lane & 15;
     const int q = lane >> 4;
@@ -761,7 +766,7 @@ __device__ __forceinline__ void place_rows(T* __restrict__ lds, const T (&values
 /// Loads per lane for a tile of 16 rows of up to 16 values (A and B of the vjp, A of the forward pass).
 constexpr int SHORT_ROW_LOADS = 4;
 
-template <typename T, int NT, int GROUPS>
+template <typename T, int NT, int GROUPS, int EPT = FEW_ENTRIES_PER_THREAD>
 __global__ __launch_bounds__(WALK_THREADS) void forward_walk_kernel(const Arguments<T> p) {
     using M = Mfma<T>;
     extern __shared__ __align__(16) char lds_raw[];
@@ -771,7 +776,7 @@ __global__ __launch_bounds__(WALK_THREADS) void forward_walk_kernel(const Argume
     const BuildAreas<T> areas = carve_build_areas<T>(cursor, p.nA * p.nB * p.nO, p.K);
     const int lane = threadIdx.x & (WAVE - 1);
     const int wave = threadIdx.x >> 6;
-    MyEntries<T> entries;
+    MyEntries<T, EPT> entries;
     entries.load(p.C, p.PA, p.PB, p.PO, p.K);
     T* mine = reinterpret_cast<T*>(cursor) + wave * ROWS_PER_WAVE * max(p.nA + p.nB, p.nO);
     T* a_tile = mine;                        // [16][nA]
@@ -795,7 +800,7 @@ __global__ __launch_bounds__(WALK_THREADS) void forward_walk_kernel(const Argume
     fetch(even, tile);
     fetch(odd, tile + stride);
     const OperandTarget<T> targets[1] = {{operand, p.first, {0, 1, 2}}};
-    build_operands<T, 1>(targets, areas, p.nA, p.nB, p.nO, entries); // ends with a barrier
+    build_operands<T, 1, EPT>(targets, areas, p.nA, p.nB, p.nO, entries); // ends with a barrier
 
     const int i = lane & 15;
     const int q = lane >> 4;
@@ -838,7 +843,7 @@ __global__ __launch_bounds__(WALK_THREADS) void forward_walk_kernel(const Argume
     }
 }
 
-template <typename T, int GROUPS>
+template <typename T, int GROUPS, int EPT = FEW_ENTRIES_PER_THREAD>
 __global__ __launch_bounds__(WALK_THREADS) void vjp_walk_kernel(const Arguments<T> p) {
     using M = Mfma<T>;
     extern __shared__ __align__(16) char lds_raw[];
@@ -852,7 +857,7 @@ __global__ __launch_bounds__(WALK_THREADS) void vjp_walk_kernel(const Arguments<
     const BuildAreas<T> areas = carve_build_areas<T>(cursor, p.nA * p.nB * p.nO, p.K);
     const int lane = threadIdx.x & (WAVE - 1);
     const int wave = threadIdx.x >> 6;
-    MyEntries<T> entries;
+    MyEntries<T, EPT> entries;
     entries.load(p.C, p.PA, p.PB, p.PO, p.K);
     T* mine = reinterpret_cast<T*>(cursor) + wave * ROWS_PER_WAVE * (p.nA + p.nB + p.nO);
     T* a_tile = mine;                          // [16][nA]
@@ -882,7 +887,7 @@ __global__ __launch_bounds__(WALK_THREADS) void vjp_walk_kernel(const Arguments<
         {want_A ? operand_A : nullptr, p.first, {1, 2, 0}},
         {want_B ? operand_B : nullptr, p.second, {0, 2, 1}},
     };
-    build_operands<T, 2>(targets, areas, p.nA, p.nB, p.nO, entries); // ends with a barrier
+    build_operands<T, 2, EPT>(targets, areas, p.nA, p.nB, p.nO, entries); // ends with a barrier
 
     const int i = lane & 15;
     const int q = lane >> 4;
@@ -1059,8 +1064,10 @@ void forward(T* output, const T* A, const T* B, const Table& table, const Shape&
     const size_t lds = walk ? walk_lds : forward_lds(s, sizeof(T));
     const LaunchEvents events = launch_events(stream);
     with_constants<4, 4>(p.first.n_tiles, p.first.n_groups, [&](auto tiles, auto groups) {
-        auto kernel = walk ? forward_walk_kernel<T, decltype(tiles)::value, decltype(groups)::value>
-                           : forward_kernel<T, decltype(tiles)::value, decltype(groups)::value>;
+        constexpr int NT = decltype(tiles)::value, GROUPS = decltype(groups)::value, MANY = MANY_ENTRIES_PER_THREAD;
+        auto kernel = s.K <= FEW_ENTRIES
+                          ? (walk ? forward_walk_kernel<T, NT, GROUPS> : forward_kernel<T, NT, GROUPS>)
+                          : (walk ? forward_walk_kernel<T, NT, GROUPS, MANY> : forward_kernel<T, NT, GROUPS, false, MANY>);
         allow_lds(kernel, lds);
         hipExtLaunchKernelGGL(kernel, dim3(grid), dim3(THREADS), lds, stream, events.start, events.stop, 0, p);
     });
@@ -1084,7 +1091,9 @@ void forward_of_two_pairs(
     const unsigned grid = static_cast<unsigned>((s.n_rows + ROWS_PER_GROUP - 1) / ROWS_PER_GROUP);
     const size_t lds = forward_lds(s, sizeof(T));
     with_constants<4, 4>(p.first.n_tiles, p.first.n_groups, [&](auto tiles, auto groups) {
-        auto kernel = forward_kernel<T, decltype(tiles)::value, decltype(groups)::value, true>;
+        constexpr int NT = decltype(tiles)::value, GROUPS = decltype(groups)::value;
+        auto kernel = s.K <= FEW_ENTRIES ? forward_kernel<T, NT, GROUPS, true>
+                                         : forward_kernel<T, NT, GROUPS, true, MANY_ENTRIES_PER_THREAD>;
         allow_lds(kernel, lds);
         hipLaunchKernelGGL(kernel, dim3(grid), dim3(THREADS), lds, stream, p);
     });
@@ -1109,7 +1118,9 @@ void vjp(
     const size_t lds = walk ? walk_lds : vjp_lds(s, sizeof(T), grad_A != nullptr, grad_B != nullptr);
     const LaunchEvents events = launch_events(stream);
     with_constants<1, 16>(1, p.first.n_groups, [&](auto, auto groups) {
-        auto kernel = walk ? vjp_walk_kernel<T, decltype(groups)::value> : vjp_kernel<T, decltype(groups)::value>;
+        constexpr int GROUPS = decltype(groups)::value, MANY = MANY_ENTRIES_PER_THREAD;
+        auto kernel = s.K <= FEW_ENTRIES ? (walk ? vjp_walk_kernel<T, GROUPS> : vjp_kernel<T, GROUPS>)
+                                         : (walk ? vjp_walk_kernel<T, GROUPS, MANY> : vjp_kernel<T, GROUPS, MANY>);
         allow_lds(kernel, lds);
         hipExtLaunchKernelGGL(kernel, dim3(grid), dim3(THREADS), lds, stream, events.start, events.stop, 0, p);
     });

@@ -44,6 +44,11 @@ CASES = {
         "unsorted": lambda s, d: support.sap_case(s, d, I=130, nA=6, nB=9, K=150, nO=11, sort_output=False),
         "wide": lambda s, d: support.sap_case(s, d, I=100, nA=70, nB=50, K=400, nO=300),
         "one_product": lambda s, d: support.sap_case(s, d, I=65, nA=3, nB=3, K=1, nO=4),
+        # (more than 2048 entries on the matrix-core path: eight entries per thread while the dense table is built;
+        # many entries per cell, added in ascending entry order)
+        "table_of_2500": lambda s, d: support.sap_case(s, d, I=500, nA=9, nB=9, K=2500, nO=9),
+        "table_of_8192_unsorted": lambda s, d: support.sap_case(s, d, I=300, nA=4, nB=5, K=8192, nO=6, sort_output=False),
+        "table_of_2049": lambda s, d: support.sap_case(s, d, I=300, nA=13, nB=7, K=2049, nO=20),
     },
     "opsa": {
         "tiny": lambda s, d: support.opsa_case(s, d, J=6, K=2, L=3, n_out=4, allow_empty=True),
