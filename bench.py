@@ -75,8 +75,8 @@ TRAFFIC_FILE = os.path.join(ROOT, "profiles", "all_ops_baseline_shapes_hbm_traff
 MAIN_KERNELS = {
     ("hpe", "forward"): "hpe::forward_ordered_kernel<{T}, 4>",
     ("hpe", "vjp"): "hpe::vjp_ordered_kernel<{T}, 4, true>",
-    ("sap", "forward"): "sap_mfma::forward_kernel<{T}, 2, 2>",
-    ("sap", "vjp"): "sap_mfma::vjp_kernel<{T}, 5>",
+    ("sap", "forward"): "sap_mfma::forward_kernel<{T}, 2, 2, false, 2>",
+    ("sap", "vjp"): "sap_mfma::vjp_kernel<{T}, 5, 2>",
     ("opsa", "forward"): "opsa::forward_kernel<{T}, 2, false, true, true>",
     ("opsa", "vjp"): "opsa::edge_rows_vjp_kernel<{T}, 1, 2, false, true, false, false>",
     ("opsaw", "forward"): "opsa::forward_kernel<{T}, 2, true, true, true>",
